@@ -1,0 +1,299 @@
+"""CPU restatement of the lm-head log-prob + entropy path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the shipped package may import this module: it exists so that tests, the smoke check
+and the benchmark's CPU-baseline leg have an independent statement of what the HIP kernels must
+compute.  It materialises logits (chunked over tokens so any size fits in host memory) and uses
+only torch library routines, evaluated in fp32 or fp64 on whatever inputs it is given.
+
+What each function follows in the reference tree (paths relative to the reference root):
+
+* ``lce_forward``            tests/utils/test_linear_cross_entropy.py:49-62 (``run_torch_entropy``),
+                             verl/utils/kernel/kernels.py:306-329,419-433 (scale after the GEMM,
+                             ``entropy = log(accu) + max - b``, ``logprob = label_logit - lse``)
+* ``lce_backward``           verl/utils/kernel/kernels.py:1443-1507 (closed-form ``d_logits``),
+                             :1714-1724 (``d_hidden = dz @ W``, ``d_weight = dz.T @ h``),
+                             verl/utils/experimental/torch_functional.py:61-93 (same math)
+* ``logprobs_from_logits``   verl/utils/torch_functional.py:155-207
+* ``entropy_from_logits``    verl/utils/torch_functional.py:231-245
+* ``logits_backward``        autograd of the two functions above, spelled out
+* ``masked_sum/masked_mean`` verl/utils/torch_functional.py:273-308
+* ``agg_loss``               verl/trainer/ppo/core_algos.py:1140-1206
+* ``policy_loss_vanilla``    verl/trainer/ppo/core_algos.py:1286-1376
+* ``ppo_actor_loss``         verl/workers/utils/losses.py:57-140 (policy loss minus entropy bonus)
+
+How each is pinned (see tests/test_oracle_*.py): the reference's own known-answer vector for the
+padded-vocab regression (tests/utils/test_linear_cross_entropy.py:352-395, closed form
+``3 - log(e^3 + (V-1)e^-15)``), uniform-logit closed forms (entropy ``log V``), shift invariance,
+fp64 brute force in pure Python on tiny inputs, ``torch.autograd`` and central finite differences
+for the gradients, the invariant ``sum_v dz = 0``, the independent C restatement in
+``lce_oracle.c``, and the reference's known answers for ``agg_loss`` / ``masked_mean``
+(tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-65, tests/utils/test_torch_functional.py:61-72).
+No function here is "parity unpinned".
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+_REDUCTIONS = ("none", "sum", "mean")
+
+
+def _check_reduction(reduction: str) -> str:
+    reduction = reduction.lower()
+    if reduction not in _REDUCTIONS:
+        raise ValueError(f"Invalid reduction: {reduction}")
+    return reduction
+
+
+def _flatten(hidden: torch.Tensor, labels: torch.Tensor):
+    return hidden.reshape(-1, hidden.shape[-1]), labels.reshape(-1).long()
+
+
+def lce_forward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    reduction: str = "none",
+    compute_dtype: torch.dtype = torch.float32,
+    chunk: int = 1024,
+    return_stats: bool = False,
+):
+    """logits = (h @ W^T) / tau in ``compute_dtype``; logprob = log_softmax(logits)[label];
+    entropy = logsumexp(logits) - sum(softmax(logits) * logits).  Outputs are flattened [T]."""
+    reduction = _check_reduction(reduction)
+    h2, y = _flatten(hidden, labels)
+    T = h2.shape[0]
+    w = weight.to(compute_dtype)
+    logprobs = torch.empty(T, dtype=compute_dtype, device=h2.device)
+    entropy = torch.empty_like(logprobs)
+    mx = torch.empty_like(logprobs)
+    acc = torch.empty_like(logprobs)
+    eb = torch.empty_like(logprobs)
+    for s in range(0, T, chunk):
+        e = min(T, s + chunk)
+        z = h2[s:e].to(compute_dtype) @ w.t()
+        z /= temperature
+        lse = torch.logsumexp(z, dim=-1)
+        pd = torch.softmax(z, dim=-1)
+        b = torch.sum(pd * z, dim=-1)
+        entropy[s:e] = lse - b
+        logprobs[s:e] = torch.gather(z, -1, y[s:e].unsqueeze(-1)).squeeze(-1) - lse
+        m = z.max(dim=-1).values
+        mx[s:e] = m
+        acc[s:e] = torch.exp(z - m.unsqueeze(-1)).sum(-1)
+        eb[s:e] = b
+    if reduction == "sum":
+        logprobs = logprobs.sum()
+    elif reduction == "mean":
+        logprobs = logprobs.sum() / T
+    if return_stats:
+        return logprobs, entropy, mx, acc, eb
+    return logprobs, entropy
+
+
+def lce_backward(
+    dlogprobs: torch.Tensor,
+    dentropy: Optional[torch.Tensor],
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    reduction: str = "none",
+    compute_dtype: torch.dtype = torch.float32,
+    chunk: int = 1024,
+):
+    """dz = g_lp * (onehot - p) - g_ent * p * (z - b), then dz /= tau;
+    d_hidden = dz @ W, d_weight = dz^T @ h.  Returned in ``compute_dtype``."""
+    reduction = _check_reduction(reduction)
+    h2, y = _flatten(hidden, labels)
+    T = h2.shape[0]
+    w = weight.to(compute_dtype)
+    if reduction == "none":
+        g_lp = dlogprobs.reshape(-1).to(compute_dtype)
+    elif reduction == "sum":
+        g_lp = dlogprobs.to(compute_dtype).reshape(()).expand(T)
+    else:
+        g_lp = (dlogprobs.to(compute_dtype).reshape(()) / T).expand(T)
+    g_ent = None if dentropy is None else dentropy.reshape(-1).to(compute_dtype)
+    d_hidden = torch.empty(h2.shape, dtype=compute_dtype, device=h2.device)
+    d_weight = torch.zeros(w.shape, dtype=compute_dtype, device=w.device)
+    for s in range(0, T, chunk):
+        e = min(T, s + chunk)
+        hc = h2[s:e].to(compute_dtype)
+        z = hc @ w.t()
+        z /= temperature
+        p = torch.softmax(z, dim=-1)
+        b = torch.sum(p * z, dim=-1, keepdim=True)
+        dz = -p * g_lp[s:e].unsqueeze(-1)
+        dz.scatter_add_(-1, y[s:e].unsqueeze(-1), g_lp[s:e].unsqueeze(-1).clone())
+        if g_ent is not None:
+            dz -= g_ent[s:e].unsqueeze(-1) * p * (z - b)
+        dz /= temperature
+        d_hidden[s:e] = dz @ w
+        d_weight += dz.t() @ hc
+    return d_hidden.reshape(hidden.shape), d_weight
+
+
+def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, compute_dtype=torch.float32):
+    """log_softmax(logits)[label], with an explicit upcast (CPU log_softmax does not upcast bf16)."""
+    z = logits.to(compute_dtype)
+    lp = torch.log_softmax(z, dim=-1)
+    return torch.gather(lp, -1, labels.long().unsqueeze(-1)).squeeze(-1)
+
+
+def entropy_from_logits(logits: torch.Tensor, compute_dtype=torch.float32):
+    """logsumexp(z) - sum(softmax(z) * z)."""
+    z = logits.to(compute_dtype)
+    pd = torch.softmax(z, dim=-1)
+    return torch.logsumexp(z, dim=-1) - torch.sum(pd * z, dim=-1)
+
+
+def logits_backward(
+    logits: torch.Tensor,
+    labels: Optional[torch.Tensor],
+    dlogprobs: Optional[torch.Tensor],
+    dentropy: Optional[torch.Tensor],
+    compute_dtype=torch.float32,
+):
+    """d_logits of ``sum(dlogprobs * logprobs) + sum(dentropy * entropy)`` w.r.t. the logits."""
+    z = logits.to(compute_dtype)
+    p = torch.softmax(z, dim=-1)
+    dz = torch.zeros_like(z)
+    if dlogprobs is not None:
+        g = dlogprobs.to(compute_dtype).unsqueeze(-1)
+        dz -= g * p
+        dz.scatter_add_(-1, labels.long().unsqueeze(-1), g.expand(*labels.shape, 1).clone())
+    if dentropy is not None:
+        b = torch.sum(p * z, dim=-1, keepdim=True)
+        dz -= dentropy.to(compute_dtype).unsqueeze(-1) * p * (z - b)
+    return dz
+
+
+# ----------------------------------------------------------------------------------------------
+# consumer of the path's output: the PPO actor loss
+# ----------------------------------------------------------------------------------------------
+
+
+def masked_sum(values, mask, axis=None):
+    valid = torch.where(mask.bool(), values, torch.zeros((), dtype=values.dtype, device=values.device))
+    return (valid * mask).sum(axis=axis)
+
+
+def masked_mean(values, mask, axis=None):
+    return masked_sum(values, mask, axis) / (mask.sum(axis=axis) + 1e-8)
+
+
+def agg_loss(
+    loss_mat,
+    loss_mask,
+    loss_agg_mode: str,
+    dp_size: int = 1,
+    batch_num_tokens=None,
+    global_batch_size=None,
+    loss_scale_factor=None,
+):
+    if loss_agg_mode == "token-mean":
+        if batch_num_tokens is None:
+            if dp_size > 1:
+                raise ValueError("(global) batch_num_tokens is required when dp_size > 1")
+            batch_num_tokens = loss_mask.sum()
+        return masked_sum(loss_mat, loss_mask) / batch_num_tokens * dp_size
+    if loss_agg_mode == "token-sum":
+        return masked_sum(loss_mat, loss_mask) * dp_size
+    if loss_agg_mode in ("seq-mean-token-sum", "seq-mean-token-sum-norm"):
+        seq_losses = torch.sum(loss_mat * loss_mask, dim=-1)
+        seq_mask = (torch.sum(loss_mask, dim=-1) > 0).float()
+        if global_batch_size is None:
+            if dp_size > 1:
+                raise ValueError("global_batch_size is required when dp_size > 1")
+            global_batch_size = seq_mask.sum()
+        loss = masked_sum(seq_losses, seq_mask) / global_batch_size * dp_size
+        if loss_agg_mode == "seq-mean-token-sum-norm":
+            loss = loss / (loss_mask.shape[-1] if loss_scale_factor is None else loss_scale_factor)
+        return loss
+    if loss_agg_mode == "seq-mean-token-mean":
+        cnt = torch.sum(loss_mask, dim=-1)
+        seq_losses = torch.sum(loss_mat * loss_mask, dim=-1) / (cnt + 1e-8)
+        seq_mask = (cnt > 0).float()
+        if global_batch_size is None:
+            if dp_size > 1:
+                raise ValueError("global_batch_size is required when dp_size > 1")
+            global_batch_size = seq_mask.sum()
+        return masked_sum(seq_losses, seq_mask) / global_batch_size * dp_size
+    raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+
+
+def policy_loss_vanilla(
+    old_log_prob,
+    log_prob,
+    advantages,
+    response_mask,
+    loss_agg_mode: str = "token-mean",
+    clip_ratio: float = 0.2,
+    clip_ratio_low: Optional[float] = None,
+    clip_ratio_high: Optional[float] = None,
+    clip_ratio_c: float = 3.0,
+    rollout_is_weights=None,
+    **global_batch_info,
+):
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    assert clip_ratio_c > 1.0
+    nkl = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(nkl)
+    ppo_kl = masked_mean(-nkl, response_mask)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - lo, 1 + hi)
+    lc1 = torch.maximum(l1, l2)
+    clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
+    l3 = -advantages * clip_ratio_c
+    lc2 = torch.min(l3, lc1)
+    clipfrac_lower = masked_mean(torch.gt(lc1, l3) * (advantages < 0).float(), response_mask)
+    losses = torch.where(advantages < 0, lc2, lc1)
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    loss = agg_loss(losses, response_mask, loss_agg_mode, **global_batch_info)
+    metrics = {
+        "actor/pg_clipfrac": clipfrac.detach().item(),
+        "actor/ppo_kl": ppo_kl.detach().item(),
+        "actor/pg_clipfrac_lower": clipfrac_lower.detach().item(),
+    }
+    return loss, metrics
+
+
+def ppo_actor_loss(
+    log_prob,
+    entropy,
+    old_log_prob,
+    advantages,
+    response_mask,
+    clip_ratio: float = 0.2,
+    entropy_coeff: float = 0.0,
+    loss_agg_mode: str = "token-mean",
+    clip_ratio_c: float = 3.0,
+):
+    """policy loss - entropy_coeff * agg(entropy): the scalar the actor back-propagates."""
+    pg, metrics = policy_loss_vanilla(
+        old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, clip_ratio, clip_ratio_c=clip_ratio_c
+    )
+    loss = pg
+    if entropy is not None:
+        ent = agg_loss(entropy, response_mask, loss_agg_mode)
+        loss = loss - entropy_coeff * ent
+        metrics["actor/entropy_loss"] = ent.detach().item()
+    metrics["actor/pg_loss"] = pg.detach().item()
+    return loss, metrics
+
+
+def padded_vocab_known_answer(V: int):
+    """Closed form of the reference's padded-vocab regression: one logit +3 and V-1 logits -15.
+    Returns (logprob of label 0, entropy) in double precision."""
+    z0, z1, n1 = 3.0, -15.0, V - 1
+    lse = z0 + math.log1p(n1 * math.exp(z1 - z0))
+    p0 = math.exp(z0 - lse)
+    p1 = math.exp(z1 - lse)
+    return z0 - lse, lse - (p0 * z0 + n1 * p1 * z1)
