@@ -1,0 +1,92 @@
+/* C ABI of liblce_gfx950.so: fused lm-head linear + log-prob + entropy for MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; every buffer is owned by the caller and lives in device memory
+ * of the current HIP device; every call is asynchronous on `stream` (a hipStream_t passed as
+ * void*) and allocates nothing.  All functions return 0 on success or a negative LCE_E_* code and
+ * never throw; lce_last_error() gives the text of the calling thread's last failure.
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to the
+ * reference tree).  The reference has no native ABI of its own (its kernels are Triton), so what
+ * is replaced are its Python host launchers.
+ */
+#ifndef LCE_ABI_H
+#define LCE_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LCE_ABI_VERSION 1
+
+enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1 };
+enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
+enum {
+  LCE_OK = 0,
+  LCE_E_ARG = -1,       /* bad shape, dtype, alignment or null pointer */
+  LCE_E_WORKSPACE = -2, /* workspace too small */
+  LCE_E_LAUNCH = -3     /* HIP reported an error at launch */
+};
+
+int lce_abi_version(void);
+const char* lce_last_error(void);
+
+/* Forward.  Replaces efficient_entropy_forward (verl/utils/kernel/kernels.py:569-759) and the two
+ * Triton kernels it launches (:186-349 mainloop, :352-441 epilogue).
+ *   hidden [T, H] row stride ldh, weight [V, H] row stride ldw (elements; K-contiguous), dtype LCE_DTYPE_*
+ *   labels [T] int64, values outside [0, V) give logprob = -logsumexp (no label logit)
+ *   logits = (hidden . weight^T) * (1 / temperature), accumulated in fp32, never written to memory
+ * Outputs, all fp32:
+ *   logprobs [T] (reduction none) or [1] (sum / mean over tokens); entropy [T];
+ *   maximum [T], accumulate [T], entropy_b [T]: per-token max logit, sum exp(logit - max) and
+ *   sum softmax * logit, kept for the backward.
+ * H must be a multiple of 64 (bf16) / 32 (fp32); pointers 16-byte aligned; ldh, ldw multiples of
+ * 8 (bf16) / 4 (fp32) elements. */
+size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype);
+int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                void* stream);
+
+/* Backward.  Replaces efficient_entropy_backward (verl/utils/kernel/kernels.py:1518-1729): its
+ * d_logits kernel (:1380-1515) and the two vendor GEMMs per vocab split (:1714-1724).
+ *   dlogprobs [T] fp32 (reduction none) or [1] fp32 (sum / mean); dentropy [T] fp32 or NULL (treated as zero)
+ *   d_hidden [T, H] and d_weight [V, H], contiguous, in the input dtype.
+ * The vocabulary is processed in chunks of `vchunk` columns (0 = library default, else a multiple
+ * of 256); per chunk the gradient of the logits exists only as a [T, vchunk] tile pair in the
+ * workspace.  Sums over the vocabulary (d_hidden) and over tokens (d_weight) are carried in fp32
+ * and rounded once. */
+size_t lce_backward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype, int64_t vchunk);
+int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                 const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                 void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                 void* stream);
+
+/* Unfused twins on logits that already exist in memory.
+ * Replaces logprobs_from_logits (verl/utils/torch_functional.py:73-107, :155-207) and
+ * entropy_from_logits (:231-245) with one pass over the rows.
+ *   logits [R, V] row stride ldl, dtype LCE_DTYPE_*; labels [R] int64 or NULL; logprobs / entropy [R] fp32, either may be NULL. */
+int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
+                       float* logprobs, float* entropy, void* stream);
+/* d_logits [R, V] (row stride ldd, same dtype as logits) of sum(dlogprobs*logprobs) + sum(dentropy*entropy);
+ * dlogprobs / dentropy [R] fp32, either may be NULL.  Autograd twin of the two functions above. */
+int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
+                        const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream);
+
+/* Diagnostic: C[M, N] (fp32, row stride ldc) = A[M, K] . B[N, K]^T with the library's MFMA
+ * mainloop (the same code that the entry points above use).  K a multiple of 64 (bf16) / 32 (fp32).
+ * No counterpart in the reference; exists so the mainloop can be tested and timed on its own. */
+int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
+                int64_t K, int dtype, int variant, void* stream);
+
+/* Tuning hook: selects the tile configuration used by the mainloops (0 = default).  Process-wide. */
+int lce_set_variant(int variant);
+int lce_num_variants(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LCE_ABI_H */

@@ -1,0 +1,291 @@
+// Shared MFMA mainloop for gfx950 (MI355X): C[m][n] = sum_k A[m][k] * B[n][k].
+//
+// Both operands are K-contiguous in memory ("NT" GEMM).  One workgroup owns a BM x BN tile of C;
+// its waves are arranged WAVES_M x WAVES_N and each wave owns (BM/WAVES_M) x (BN/WAVES_N) as
+// 32x32 MFMA blocks.  K is streamed in slabs of BKB bytes per row through an NSTAGE-deep LDS ring
+// that is filled by direct global->LDS loads (16 bytes per lane, no VGPR staging).
+//
+// LDS layout of one operand slab: row-major, BKB bytes per row, the 16-byte chunk index of every
+// row XOR-ed with a function of the row number so that the 16-byte MFMA operand reads of 32
+// consecutive rows spread over all banks.
+//
+// Accumulator layout of one 32x32 block (v_mfma_f32_32x32x*): lane l holds column n = l % 32 and
+// the 16 rows m = 8*(r/4) + 4*(l/32) + (r%4), r = 0..15.  Epilogues rely on this: everything a lane
+// holds belongs to ONE column n per block, so per-column reductions over m are lane-local.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lce {
+
+typedef __bf16 bf16_t;
+typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+#define LCE_DEV __device__ __forceinline__
+
+typedef const void __attribute__((address_space(1))) * gptr_t;
+typedef void __attribute__((address_space(3))) * lptr_t;
+
+template <typename T>
+struct Mma;
+
+// one 16-byte chunk (8 bf16 along K) per lane of A and of B -> one 32x32x16 MFMA
+template <>
+struct Mma<bf16_t> {
+  static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                  acc, 0, 0, 0);
+  }
+};
+
+// one 16-byte chunk (4 fp32 along K) per lane -> four 32x32x2 MFMAs (true fp32 multiply-add)
+template <>
+struct Mma<float> {
+  static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    const f32x4_t af = __builtin_bit_cast(f32x4_t, a);
+    const f32x4_t bf = __builtin_bit_cast(f32x4_t, b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[i], acc, 0, 0, 0);
+  }
+};
+
+template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_>
+struct GemmCfg {
+  typedef TIN_ TIN;
+  static constexpr int BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
+  static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr int NW = WAVES_M * WAVES_N;
+  static constexpr int NTHREADS = NW * 64;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int FM = WM / 32, FN = WN / 32;
+  static constexpr int BK = BKB / (int)sizeof(TIN);  // K elements per slab
+  static constexpr int CH = BKB / 16;                 // 16-byte chunks per row
+  static constexpr int KSUB = CH / 2;                 // MFMA k-substeps per slab (2 chunks each)
+  static constexpr int ROWS_PER_LOAD = 64 / CH;       // rows one wave-wide 16B/lane load covers
+  static constexpr int A_LOADS = BM / ROWS_PER_LOAD / NW;
+  static constexpr int B_LOADS = BN / ROWS_PER_LOAD / NW;
+  static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+  static_assert(BKB == 128 || BKB == 64, "slab rows are 64 or 128 bytes");
+  static_assert(BM % (ROWS_PER_LOAD * NW) == 0 && BN % (ROWS_PER_LOAD * NW) == 0, "tile/loader mismatch");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 blocks");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(KSUB % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 4, "pipeline shape");
+
+  // XOR pattern applied to the chunk index of a row (uses row bits 0..3 only, so it is the same
+  // for rows that differ by a multiple of 32).
+  static LCE_DEV int swz(int row) {
+    if constexpr (CH == 8) return (row ^ ((row >> 3) & 1)) & 7;
+    else return ((row >> 1) ^ (row >> 3)) & 3;
+  }
+};
+
+// Per-lane addressing state for streaming one operand slab (A or B) from global memory.
+template <int NLOADS>
+struct SlabLoader {
+  uint32_t voff[NLOADS];  // byte offset of this lane's 16-byte chunk relative to the tile's first row, k = 0
+};
+
+template <typename Cfg>
+struct GemmCore {
+  typedef typename Cfg::TIN TIN;
+
+  const char* a_base;  // &A[m0][0]
+  const char* b_base;  // &B[n0][0]
+  SlabLoader<Cfg::A_LOADS> la;
+  SlabLoader<Cfg::B_LOADS> lb;
+  int wave, lane, wave_m, wave_n;
+  uint32_t a_rd, b_rd;  // LDS byte offsets (within a stage) of this lane's operand rows, swizzle folded in
+
+  // rows beyond the matrix are clamped to its last row (their results are discarded by the epilogue)
+  LCE_DEV void init(const TIN* A, int64_t lda, int64_t m0, int64_t M, const TIN* B, int64_t ldb, int64_t n0,
+                    int64_t N) {
+    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    lane = threadIdx.x & 63;
+    wave_m = wave / Cfg::WAVES_N;
+    wave_n = wave % Cfg::WAVES_N;
+    a_base = reinterpret_cast<const char*>(A + m0 * lda);
+    b_base = reinterpret_cast<const char*>(B + n0 * ldb);
+    const int rows_a = (int)((M - m0) < (int64_t)Cfg::BM ? (M - m0) : (int64_t)Cfg::BM);
+    const int rows_b = (int)((N - n0) < (int64_t)Cfg::BN ? (N - n0) : (int64_t)Cfg::BN);
+    const int lr = lane / Cfg::CH, pc = lane % Cfg::CH;
+#pragma unroll
+    for (int j = 0; j < Cfg::A_LOADS; ++j) {
+      const int row = (j * Cfg::NW + wave) * Cfg::ROWS_PER_LOAD + lr;
+      const int c = pc ^ Cfg::swz(row);
+      const int crow = row < rows_a ? row : rows_a - 1;
+      la.voff[j] = (uint32_t)((int64_t)crow * lda * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < Cfg::B_LOADS; ++j) {
+      const int row = (j * Cfg::NW + wave) * Cfg::ROWS_PER_LOAD + lr;
+      const int c = pc ^ Cfg::swz(row);
+      const int crow = row < rows_b ? row : rows_b - 1;
+      lb.voff[j] = (uint32_t)((int64_t)crow * ldb * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
+    }
+    const int r32 = lane & 31, hh = lane >> 5;
+    const int x = (hh ^ Cfg::swz(r32)) * 16;
+    a_rd = (uint32_t)((wave_m * Cfg::WM + r32) * Cfg::BKB + x);
+    b_rd = (uint32_t)(Cfg::A_BYTES + (wave_n * Cfg::WN + r32) * Cfg::BKB + x);
+  }
+
+  static constexpr int PER = Cfg::A_LOADS + Cfg::B_LOADS;  // wave-wide DMA loads per slab
+  static constexpr int N_READS = Cfg::FM + Cfg::FN;       // LDS operand reads per k-substep
+  static constexpr int N_BLK = Cfg::FM * Cfg::FN;         // 32x32 blocks per wave
+
+  // one of the PER wave-wide 16-byte-per-lane global->LDS loads of a slab (A loads first)
+  LCE_DEV void dma_one(char* lds, int stage, int64_t kbyte, int idx) const {
+    char* sa = lds + stage * Cfg::STAGE_BYTES;
+    if (idx < Cfg::A_LOADS) {
+      __builtin_amdgcn_global_load_lds((gptr_t)(a_base + kbyte + la.voff[idx]),
+                                       (lptr_t)(sa + (idx * Cfg::NW + wave) * 1024), 16, 0, 0);
+    } else {
+      const int j = idx - Cfg::A_LOADS;
+      __builtin_amdgcn_global_load_lds((gptr_t)(b_base + kbyte + lb.voff[j]),
+                                       (lptr_t)(sa + Cfg::A_BYTES + (j * Cfg::NW + wave) * 1024), 16, 0, 0);
+    }
+  }
+  LCE_DEV void issue_slab(char* lds, int stage, int64_t kbyte) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) dma_one(lds, stage, kbyte, i);
+  }
+
+  // one of the N_READS operand reads of k-substep kk, in the order a0, b0..b(FN-1), a1..a(FM-1)
+  LCE_DEV void read_one(const char* s, int kk, int idx, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
+    const uint32_t ao = a_rd ^ (uint32_t)(kk * 32);
+    const uint32_t bo = b_rd ^ (uint32_t)(kk * 32);
+    if (idx == 0) af[0] = *reinterpret_cast<const u32x4_t*>(s + ao);
+    else if (idx <= Cfg::FN) bf[idx - 1] = *reinterpret_cast<const u32x4_t*>(s + bo + (idx - 1) * 32 * Cfg::BKB);
+    else af[idx - Cfg::FN] = *reinterpret_cast<const u32x4_t*>(s + ao + (idx - Cfg::FN) * 32 * Cfg::BKB);
+  }
+  LCE_DEV void load_frags(const char* s, int kk, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
+#pragma unroll
+    for (int i = 0; i < N_READS; ++i) read_one(s, kk, i, af, bf);
+  }
+
+  // One k-substep with a hand-placed instruction order (pinned by scheduling barriers): the MFMAs
+  // of this substep, with the operand reads of the NEXT substep (from `s_next`, substep `kk_next`)
+  // and, when DMA is set, the global->LDS loads of a future slab dealt out between them.
+  template <bool DMA>
+  LCE_DEV void substep(f32x16_t (&acc)[Cfg::FM][Cfg::FN], const u32x4_t (&af)[Cfg::FM], const u32x4_t (&bf)[Cfg::FN],
+                       const char* s_next, int kk_next, u32x4_t (&af_n)[Cfg::FM], u32x4_t (&bf_n)[Cfg::FN],
+                       char* lds, int dma_stage, int64_t dma_kbyte) const {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int b = 0; b < N_BLK; ++b) {
+      Mma<TIN>::run(acc[b / Cfg::FN][b % Cfg::FN], af[b / Cfg::FN], bf[b % Cfg::FN]);
+      // reads: spread over the first blocks, one read after every `rstep`-th MFMA
+      constexpr int rstep = 1;
+      if ((b % rstep) == rstep - 1 && b / rstep < N_READS) read_one(s_next, kk_next, b / rstep, af_n, bf_n);
+      if (N_BLK < N_READS && b == N_BLK - 1) {
+#pragma unroll
+        for (int r = N_BLK; r < N_READS; ++r) read_one(s_next, kk_next, r, af_n, bf_n);
+      }
+      if (DMA) {
+#pragma unroll
+        for (int d = b * PER / N_BLK; d < (b + 1) * PER / N_BLK; ++d) dma_one(lds, dma_stage, dma_kbyte, d);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // Full K loop.  K must be a multiple of Cfg::BK (and > 0).  The k-substeps are software
+  // pipelined: operand fragments of substep s+1 are read from LDS while the MFMAs of substep s run,
+  // and the workgroup barrier that hands a ring stage back to the loader sits before the LAST
+  // substep of a slab, so the matrix pipe keeps working across the barrier.  The loop body is
+  // branch-free: past the end of K the loader re-fetches the last slab into a stage nobody reads.
+  LCE_DEV void run(char* lds, int64_t K, f32x16_t (&acc)[Cfg::FM][Cfg::FN]) const {
+    constexpr int NS = Cfg::NSTAGE, KSUB = Cfg::KSUB;
+    const int nk = (int)(K / Cfg::BK);
+    const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int64_t kb = (int64_t)s * Cfg::BKB;
+      issue_slab(lds, s, kb < last_kbyte ? kb : last_kbyte);
+    }
+    wait_vm<(NS - 1) * PER>();
+    __builtin_amdgcn_s_barrier();
+    u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];
+    load_frags(lds, 0, af[0], bf[0]);
+    int stage = 0;
+    int64_t kb_next = (int64_t)NS * Cfg::BKB;
+    for (int it = 0; it < nk; ++it) {
+      const char* s = lds + stage * Cfg::STAGE_BYTES;
+#pragma unroll
+      for (int kk = 0; kk < KSUB - 1; ++kk)
+        substep<false>(acc, af[kk & 1], bf[kk & 1], s, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1], lds, 0, 0);
+      // last substep of this slab: its fragments are in registers, so this wave is done with the stage
+      const int nstage = stage + 1 == NS ? 0 : stage + 1;
+      wait_vm<(NS - 2) * PER>();           // slab it+1 has landed (only the younger slabs may be in flight)
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of the stage have returned
+      __builtin_amdgcn_s_barrier();
+      substep<true>(acc, af[(KSUB - 1) & 1], bf[(KSUB - 1) & 1], lds + nstage * Cfg::STAGE_BYTES, 0, af[0], bf[0], lds,
+                    stage, kb_next < last_kbyte ? kb_next : last_kbyte);
+      kb_next += Cfg::BKB;
+      stage = nstage;
+    }
+    wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
+  }
+
+  template <int N>
+  static LCE_DEV void wait_vm() {
+    // gfx9 s_waitcnt simm16: vmcnt[3:0] bits 3:0, expcnt bits 6:4, lgkmcnt bits 11:8, vmcnt[5:4] bits 15:14
+    static_assert(N < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt(((N & 0xF) | ((N >> 4) << 14)) | 0x0F70);
+  }
+};
+
+// XCD-aware decode of a flat workgroup id into a (row-tile, col-tile) pair.
+// Hardware deals workgroup ids round-robin over the 8 XCDs (each with its own L2), so ids with the
+// same (id % 8) share an L2.  We hand each XCD a contiguous range of "virtual" ids and cut the
+// virtual id space into blocks of 32 tiles shaped BR x (32/BR): the 32 workgroups resident on one
+// XCD then touch only BR row-tiles and 32/BR col-tiles of the operands.
+struct TileMap {
+  int nrow_tiles, ncol_tiles;  // tiles along the "row" operand (blocks of BR) and "col" operand
+  int br, bc;                  // block shape, br * bc == 32
+  int nrb, ncb;                // blocks along rows / cols
+  int rows_fastest;            // 1: consecutive blocks walk the row dimension first
+  int total;                   // launched workgroups (multiple of 8)
+
+  __host__ __device__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
+    TileMap t;
+    t.nrow_tiles = nrow_tiles;
+    t.ncol_tiles = ncol_tiles;
+    t.br = br;
+    t.bc = 32 / br;
+    t.nrb = (nrow_tiles + t.br - 1) / t.br;
+    t.ncb = (ncol_tiles + t.bc - 1) / t.bc;
+    t.rows_fastest = rows_fastest;
+    t.total = t.nrb * t.ncb * 32;
+    return t;
+  }
+  // returns false when the slot is padding (no tile)
+  __device__ bool decode(int bid, int& rt, int& ct) const {
+    const int per_xcd = total >> 3;
+    const int vid = (bid & 7) * per_xcd + (bid >> 3);
+    const int blk = vid >> 5, within = vid & 31;
+    int rb, cb;
+    if (rows_fastest) {
+      rb = blk % nrb;
+      cb = blk / nrb;
+    } else {
+      cb = blk % ncb;
+      rb = blk / ncb;
+    }
+    rt = rb * br + within / bc;
+    ct = cb * bc + within % bc;
+    return rt < nrow_tiles && ct < ncol_tiles;
+  }
+};
+
+}  // namespace lce

@@ -1,0 +1,379 @@
+// C ABI of liblce_gfx950.so (see include/lce_abi.h).  Host-side launch logic only; the kernels
+// live in lce_kernels.hpp.  Nothing here allocates device memory: callers bring the workspace.
+#include "../../include/lce_abi.h"
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "lce_kernels.hpp"
+
+using namespace lce;
+
+namespace {
+
+thread_local char g_err[512] = "";
+int g_variant = 0;
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(LCE_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return LCE_OK;
+}
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// tile configurations of the mainloop, selectable for tuning
+//            TIN     BM   BN   BKB NSTAGE WAVES_M WAVES_N
+template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 2, 2, 2> Cfg; };
+template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 64, 4, 2, 2> Cfg; };
+template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 64, 4, 4, 2> Cfg; };
+template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };
+template <typename TIN> struct Variant4 { typedef GemmCfg<TIN, 256, 128, 128, 3, 2, 2> Cfg; };
+constexpr int kNumVariants = 5;
+
+template <typename K>
+void allow_lds(K kernel, int bytes) {
+  // dynamic LDS above 64 KiB has to be enabled per kernel; cheap and idempotent
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+// choose the shape of the 32-tile blocks that one XCD works on (rows = `nrow_tiles` side)
+int block_rows(int nrow_tiles) {
+  int br = 1;
+  while (br < 8 && br < nrow_tiles) br <<= 1;
+  return br;
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename Cfg>
+int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN* B, int64_t ldb, int64_t M, int64_t N,
+                int64_t K, float* Cf, int64_t ldcf, typename Cfg::TIN* Ct, int64_t ldct, int out_mode,
+                hipStream_t st) {
+  typedef typename Cfg::TIN TIN;
+  if (M <= 0 || N <= 0) return LCE_OK;
+  if (K <= 0 || K % Cfg::BK != 0) return fail(LCE_E_ARG, "gemm: K=%lld must be a positive multiple of %d", (long long)K, Cfg::BK);
+  GemmArgs<TIN> p;
+  p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
+  p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
+  const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
+  p.map = TileMap::make(tm, tn, block_rows(tm), 1);
+  allow_lds(gemm_nt_kernel<Cfg>, Cfg::LDS_BYTES);
+  hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  return check_launch("gemm_nt_kernel");
+}
+
+template <typename Cfg>
+int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
+                 int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* logprobs, float* entropy,
+                 float* maximum, float* accumulate, float* entropy_b, char* ws, hipStream_t st) {
+  typedef typename Cfg::TIN TIN;
+  const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
+  const int nvt = (int)((V + Cfg::BM - 1) / Cfg::BM);
+  // splits: enough workgroups to fill 256 CUs, in multiples of the XCD block width
+  const int br = block_rows(ntt), bc = 32 / br;
+  const int nrb = (ntt + br - 1) / br;
+  int S = bc * ((8 + nrb - 1) / nrb);
+  if (S > nvt) S = nvt;
+  FwdArgs<TIN> p;
+  p.W = W; p.ldw = ldw; p.h = h; p.ldh = ldh; p.labels = labels; p.T = T; p.V = V; p.H = H;
+  p.c = kLog2e / temperature;
+  p.parts = reinterpret_cast<f32x4_t*>(ws);
+  p.S = S; p.nvt = nvt;
+  p.map = TileMap::make(ntt, S, br, 1);
+  float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16));
+  allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
+  hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  int rc = check_launch("lce_fwd_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, S, T, p.c,
+                     1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
+  rc = check_launch("lce_fwd_merge_kernel");
+  if (rc) return rc;
+  if (reduction != LCE_REDUCTION_NONE) {
+    const float scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
+    hipLaunchKernelGGL(lce_reduce_sum_kernel, dim3(1), dim3(1024), 0, st, lp_tok, T, scale, logprobs);
+    rc = check_launch("lce_reduce_sum_kernel");
+  }
+  return rc;
+}
+
+// upper bound of the number of vocabulary splits forward_impl picks, over the token-tile widths in use
+int forward_splits_upper_bound(int64_t T) {
+  int best = 1;
+  for (int bn = 128; bn <= 256; bn <<= 1) {
+    const int ntt = (int)((T + bn - 1) / bn);
+    const int br = block_rows(ntt), bc = 32 / br, nrb = (ntt + br - 1) / br;
+    const int S = bc * ((8 + nrb - 1) / nrb);
+    if (S > best) best = S;
+  }
+  return best;
+}
+
+struct BwdLayout {
+  int64_t vchunk, ldS, ldST, ldWt, ldHt;
+  size_t off_dS, off_dST, off_Wt, off_Ht, off_dHacc, total;
+  int nchunks;
+};
+
+BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk) {
+  BwdLayout L;
+  if (vchunk <= 0) vchunk = 8192;
+  vchunk = round_up(vchunk, 256);
+  if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
+  L.vchunk = vchunk;
+  L.nchunks = (int)((V + vchunk - 1) / vchunk);
+  L.ldS = vchunk;
+  L.ldST = round_up(T, 64);
+  L.ldWt = round_up(V, 64);
+  L.ldHt = round_up(T, 64);
+  size_t o = 0;
+  L.off_dS = o;    o += align256((size_t)T * L.ldS * esz);
+  L.off_dST = o;   o += align256((size_t)vchunk * L.ldST * esz);
+  L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
+  L.off_Ht = o;    o += align256((size_t)H * L.ldHt * esz);
+  L.off_dHacc = o; o += L.nchunks > 1 ? align256((size_t)T * H * 4) : 0;
+  L.total = o;
+  return L;
+}
+
+template <typename Cfg>
+int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
+                  int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
+                  const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                  typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st) {
+  typedef typename Cfg::TIN TIN;
+  const BwdLayout L = bwd_layout(T, H, V, sizeof(TIN), vchunk);
+  TIN* dS = reinterpret_cast<TIN*>(ws + L.off_dS);
+  TIN* dST = reinterpret_cast<TIN*>(ws + L.off_dST);
+  TIN* Wt = reinterpret_cast<TIN*>(ws + L.off_Wt);
+  TIN* Ht = reinterpret_cast<TIN*>(ws + L.off_Ht);
+  float* dHacc = reinterpret_cast<float*>(ws + L.off_dHacc);
+  int rc;
+  // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
+  hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldWt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
+                     W, ldw, V, H, Wt, L.ldWt);
+  if ((rc = check_launch("transpose W"))) return rc;
+  hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldHt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
+                     h, ldh, T, H, Ht, L.ldHt);
+  if ((rc = check_launch("transpose h"))) return rc;
+
+  const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
+  allow_lds(lce_bwd_ds_kernel<Cfg>, Cfg::LDS_BYTES);
+  for (int c = 0; c < L.nchunks; ++c) {
+    const int64_t v0 = (int64_t)c * L.vchunk;
+    const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
+    DsArgs<TIN> p;
+    p.W = W + v0 * ldw; p.ldw = ldw; p.h = h; p.ldh = ldh; p.labels = labels; p.T = T; p.H = H;
+    p.v0 = v0; p.vrows = vrows; p.rcp_tau = 1.0f / temperature; p.c = kLog2e / temperature;
+    p.maximum = maximum; p.accumulate = accumulate; p.entropy_b = entropy_b;
+    p.g_lp = dlogprobs; p.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
+    p.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
+    p.g_ent = dentropy;
+    p.dS = dS; p.ldS = L.ldS; p.dST = dST; p.ldST = L.ldST;
+    const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
+    p.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
+    hipLaunchKernelGGL(lce_bwd_ds_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    if ((rc = check_launch("lce_bwd_ds_kernel"))) return rc;
+    // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
+    const int64_t kc = round_up(vrows, 64);
+    const bool first = c == 0, last = c == L.nchunks - 1;
+    const int mode_h = (first ? 0 : 1) | (last ? 2 : 0);
+    rc = launch_gemm<Cfg>(dS, L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h, st);
+    if (rc) return rc;
+    // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
+    rc = launch_gemm<Cfg>(dST, L.ldST, Ht, L.ldHt, vrows, H, L.ldST, nullptr, 0, d_weight + v0 * H, H, 2, st);
+    if (rc) return rc;
+  }
+  return LCE_OK;
+}
+
+template <template <typename> class Vt>
+int dispatch_dtype_forward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
+                           int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* lp, float* ent,
+                           float* mx, float* ac, float* eb, char* ws, hipStream_t st) {
+  if (dtype == LCE_DTYPE_BF16)
+    return forward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
+                                                  reduction, lp, ent, mx, ac, eb, ws, st);
+  return forward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
+                                               reduction, lp, ent, mx, ac, eb, ws, st);
+}
+
+template <template <typename> class Vt>
+int dispatch_dtype_backward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
+                            int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* mx,
+                            const float* ac, const float* eb, const float* glp, const float* gent, void* dh, void* dw,
+                            char* ws, int64_t vchunk, hipStream_t st) {
+  if (dtype == LCE_DTYPE_BF16)
+    return backward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
+                                                   reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st);
+  return backward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
+                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st);
+}
+
+template <template <typename> class Vt>
+int dispatch_dtype_gemm(int dtype, const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M,
+                        int64_t N, int64_t K, hipStream_t st) {
+  if (dtype == LCE_DTYPE_BF16)
+    return launch_gemm<typename Vt<bf16_t>::Cfg>((const bf16_t*)A, lda, (const bf16_t*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0, st);
+  return launch_gemm<typename Vt<float>::Cfg>((const float*)A, lda, (const float*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0, st);
+}
+
+int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, int dtype, float temperature, int reduction) {
+  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  const int64_t kmul = dtype == LCE_DTYPE_BF16 ? 64 : 32, ldmul = dtype == LCE_DTYPE_BF16 ? 8 : 4;
+  if (T < 0 || H <= 0 || V <= 0) return fail(LCE_E_ARG, "bad shape T=%lld H=%lld V=%lld", (long long)T, (long long)H, (long long)V);
+  if (V >= (1LL << 31) || T >= (1LL << 31)) return fail(LCE_E_ARG, "T and V must be below 2^31");
+  if (H % kmul != 0) return fail(LCE_E_ARG, "hidden size %lld must be a multiple of %lld", (long long)H, (long long)kmul);
+  if (ldh < H || ldw < H || ldh % ldmul != 0 || ldw % ldmul != 0) return fail(LCE_E_ARG, "bad row strides ldh=%lld ldw=%lld", (long long)ldh, (long long)ldw);
+  if (T > 0 && (!hidden || !weight || !labels)) return fail(LCE_E_ARG, "null input pointer");
+  if (!aligned16(hidden) || !aligned16(weight)) return fail(LCE_E_ARG, "hidden and weight must be 16-byte aligned");
+  if (!(temperature > 0.f)) return fail(LCE_E_ARG, "temperature must be positive");
+  if (reduction < 0 || reduction > 2) return fail(LCE_E_ARG, "Invalid reduction: %d", reduction);
+  return LCE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lce_abi_version(void) { return LCE_ABI_VERSION; }
+const char* lce_last_error(void) { return g_err; }
+int lce_num_variants(void) { return kNumVariants; }
+int lce_set_variant(int variant) {
+  if (variant < 0 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
+  g_variant = variant;
+  return LCE_OK;
+}
+
+size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
+  (void)H; (void)V; (void)dtype;
+  if (T <= 0) return 256;
+  return align256((size_t)forward_splits_upper_bound(T) * (size_t)T * 16) + align256((size_t)T * 4);
+}
+
+int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                void* stream) {
+  int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
+  if (rc) return rc;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (T == 0) {
+    if (reduction != LCE_REDUCTION_NONE && logprobs) {
+      hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t*>(logprobs), (int64_t)1);
+      return check_launch("fill_zero_kernel");
+    }
+    return LCE_OK;
+  }
+  if (!logprobs || !entropy || !maximum || !accumulate || !entropy_b) return fail(LCE_E_ARG, "null output pointer");
+  if (!workspace || workspace_bytes < lce_forward_workspace_bytes(T, H, V, dtype))
+    return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
+  char* ws = static_cast<char*>(workspace);
+#define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st)
+  switch (g_variant) {
+    case 1: return LCE_FWD(Variant1);
+    case 2: return LCE_FWD(Variant2);
+    case 3: return LCE_FWD(Variant3);
+    case 4: return LCE_FWD(Variant4);
+    default: return LCE_FWD(Variant0);
+  }
+#undef LCE_FWD
+}
+
+size_t lce_backward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype, int64_t vchunk) {
+  if (T <= 0 || H <= 0 || V <= 0) return 256;
+  return bwd_layout(T, H, V, dtype == LCE_DTYPE_BF16 ? 2 : 4, vchunk).total + 256;
+}
+
+int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                 const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                 void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                 void* stream) {
+  int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
+  if (rc) return rc;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const size_t esz = dtype == LCE_DTYPE_BF16 ? 2 : 4;
+  if (!d_weight) return fail(LCE_E_ARG, "null d_weight");
+  if (T == 0) {
+    const int64_t words = (int64_t)((size_t)V * H * esz / 4);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<uint32_t*>(d_weight), words);
+    return check_launch("fill_zero_kernel");
+  }
+  if (!d_hidden || !maximum || !accumulate || !entropy_b || !dlogprobs) return fail(LCE_E_ARG, "null pointer");
+  if (!aligned16(d_hidden) || !aligned16(d_weight)) return fail(LCE_E_ARG, "gradients must be 16-byte aligned");
+  if (vchunk < 0) return fail(LCE_E_ARG, "vchunk must be >= 0");
+  if (!workspace || workspace_bytes < lce_backward_workspace_bytes(T, H, V, dtype, vchunk))
+    return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, lce_backward_workspace_bytes(T, H, V, dtype, vchunk));
+  char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
+#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st)
+  switch (g_variant) {
+    case 1: return LCE_BWD(Variant1);
+    case 2: return LCE_BWD(Variant2);
+    case 3: return LCE_BWD(Variant3);
+    case 4: return LCE_BWD(Variant4);
+    default: return LCE_BWD(Variant0);
+  }
+#undef LCE_BWD
+}
+
+int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
+                int64_t K, int dtype, int variant, void* stream) {
+  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (!A || !B || !C || !aligned16(A) || !aligned16(B)) return fail(LCE_E_ARG, "bad pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define LCE_GEMM(Vt) dispatch_dtype_gemm<Vt>(dtype, A, lda, B, ldb, C, ldc, M, N, K, st)
+  switch (variant) {
+    case 0: return LCE_GEMM(Variant0);
+    case 1: return LCE_GEMM(Variant1);
+    case 2: return LCE_GEMM(Variant2);
+    case 3: return LCE_GEMM(Variant3);
+    case 4: return LCE_GEMM(Variant4);
+    default: return fail(LCE_E_ARG, "variant %d out of range", variant);
+  }
+#undef LCE_GEMM
+}
+
+int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
+                       float* logprobs, float* entropy, void* stream) {
+  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
+  if (R == 0) return LCE_OK;
+  if (!logits || (logprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  constexpr int NT = 512;
+  if (dtype == LCE_DTYPE_BF16)
+    hipLaunchKernelGGL((logits_fwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, logprobs, entropy);
+  else
+    hipLaunchKernelGGL((logits_fwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, logprobs, entropy);
+  return check_launch("logits_fwd_kernel");
+}
+
+int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
+                        const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream) {
+  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (R < 0 || V <= 0 || ldl < V || ldd < V) return fail(LCE_E_ARG, "bad shape");
+  if (R == 0) return LCE_OK;
+  if (!logits || !d_logits || (dlogprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  constexpr int NT = 512;
+  if (dtype == LCE_DTYPE_BF16)
+    hipLaunchKernelGGL((logits_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, dlogprobs, dentropy, (bf16_t*)d_logits, ldd);
+  else
+    hipLaunchKernelGGL((logits_bwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, dlogprobs, dentropy, (float*)d_logits, ldd);
+  return check_launch("logits_bwd_kernel");
+}
+
+}  // extern "C"

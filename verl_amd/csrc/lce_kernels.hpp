@@ -1,0 +1,492 @@
+// Device kernels of the fused lm-head log-prob + entropy path (gfx950).
+//
+// Orientation used by the fused kernels: the MFMA "A" operand is the weight tile (rows = vocabulary)
+// and the "B" operand is the hidden tile (rows = tokens), so the accumulator holds S^T[vocab][token].
+// With the 32x32 accumulator layout each lane then owns ONE token per block and 16 vocabulary
+// entries of it: max / sum-exp / sum x*exp over the vocabulary are lane-local, and per-token
+// constants (statistics, upstream gradients, label) are per-lane scalars.
+#pragma once
+#include "gemm_core.hpp"
+
+namespace lce {
+
+static constexpr float kLog2e = 1.4426950408889634f;
+static constexpr float kLn2 = 0.6931471805599453f;
+static constexpr float kNegBig = -1.0e30f;  // running-max seed: finite so that (seed - seed) is 0, not NaN
+
+LCE_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// (m, a, b) partial statistics in raw-accumulator units x (logit = x / tau), c = log2(e) / tau:
+// a = sum 2^((x - m) c), b = sum x 2^((x - m) c)
+LCE_DEV void merge_stats(float& m, float& a, float& b, float m2, float a2, float b2, float c) {
+  const float mn = fmaxf(m, m2);
+  const float s1 = fast_exp2((m - mn) * c), s2 = fast_exp2((m2 - mn) * c);
+  a = a * s1 + a2 * s2;
+  b = b * s1 + b2 * s2;
+  m = mn;
+}
+
+// vocabulary index (relative to the wave tile's first row) of accumulator register r in block row i
+LCE_DEV int acc_row(int i, int r, int hh) { return i * 32 + 8 * (r >> 2) + 4 * hh + (r & 3); }
+
+// ------------------------------------------------------------------------------------------------
+// forward: partial statistics per (vocabulary split, token)
+// ------------------------------------------------------------------------------------------------
+template <typename TIN>
+struct FwdArgs {
+  const TIN* W;
+  int64_t ldw;
+  const TIN* h;
+  int64_t ldh;
+  const int64_t* labels;
+  int64_t T, V, H;
+  float c;           // log2(e) / temperature
+  f32x4_t* parts;    // [S][T] of (m, a, b, x_label)
+  int S;             // vocabulary splits; split s owns vocab tiles s, s+S, s+2S, ...
+  int nvt;           // vocabulary tiles
+  TileMap map;       // rows = token tiles, cols = splits
+};
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  int tt, s;
+  if (!p.map.decode(blockIdx.x, tt, s)) return;
+  const int64_t n0 = (int64_t)tt * Cfg::BN;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
+  GemmCore<Cfg> g;
+
+  float m[Cfg::FN], a[Cfg::FN], b[Cfg::FN], zy[Cfg::FN];
+  int lab[Cfg::FN];
+  {
+    const int wave = threadIdx.x >> 6;
+    const int wave_n = wave % Cfg::WAVES_N;
+#pragma unroll
+    for (int j = 0; j < Cfg::FN; ++j) {
+      m[j] = kNegBig;
+      a[j] = 0.f;
+      b[j] = 0.f;
+      zy[j] = 0.f;
+      const int64_t t = n0 + wave_n * Cfg::WN + j * 32 + ln;
+      const int64_t y = t < p.T ? p.labels[t] : -1;
+      lab[j] = (y >= 0 && y < p.V) ? (int)y : -1;
+    }
+  }
+
+  f32x16_t acc[Cfg::FM][Cfg::FN];
+  for (int vt = s; vt < p.nvt; vt += p.S) {
+    const int64_t m0 = (int64_t)vt * Cfg::BM;
+    g.init(p.W, p.ldw, m0, p.V, p.h, p.ldh, n0, p.T);
+    g.run(lds, p.H, acc);
+    const int vbase = (int)m0 + g.wave_m * Cfg::WM;  // vocabulary index of this wave's first row
+    const bool full = m0 + Cfg::BM <= p.V;
+    if (!full) {
+#pragma unroll
+      for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (vbase + acc_row(i, r, hh) >= p.V) acc[i][j][r] = -INFINITY;
+    }
+#pragma unroll
+    for (int j = 0; j < Cfg::FN; ++j) {
+      __builtin_amdgcn_sched_barrier(0);  // keep one block column in flight at a time (register pressure)
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, acc[i][j][r]);
+      __builtin_amdgcn_sched_barrier(0);
+      const float mn = fmaxf(m[j], tmax);
+      const float sc = fast_exp2((m[j] - mn) * p.c);
+      const float mc = mn * p.c;
+      float aj = a[j] * sc, bj = b[j] * sc;
+      m[j] = mn;
+      if (full) {
+#pragma unroll
+        for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float x = acc[i][j][r];
+            const float e = fast_exp2(__builtin_fmaf(x, p.c, -mc));
+            aj += e;
+            bj = __builtin_fmaf(x, e, bj);
+          }
+      } else {
+        // padded vocabulary rows: -inf in the log-sum-exp, 0 in the sum of x * exp
+#pragma unroll
+        for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float x = acc[i][j][r];
+            const float e = fast_exp2(__builtin_fmaf(x, p.c, -mc));
+            aj += e;
+            bj = __builtin_fmaf(x == -INFINITY ? 0.f : x, e, bj);
+          }
+      }
+      a[j] = aj;
+      b[j] = bj;
+      // label logit: rare (a token's label falls in this wave tile with probability WM / V)
+      const int rel = lab[j] - vbase;
+      const bool mine = lab[j] >= 0 && rel >= 0 && rel < Cfg::WM && (((rel >> 2) & 1) == hh);
+      if (__builtin_amdgcn_ballot_w64(mine) != 0) {
+        float pick = 0.f;
+#pragma unroll
+        for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (mine && acc_row(i, r, hh) == rel) pick = acc[i][j][r];
+        zy[j] += pick;
+      }
+    }
+    __syncthreads();  // every wave is done with LDS before the next tile's loads overwrite it
+  }
+
+  // merge the two lane halves (same token, different vocabulary rows), then the WAVES_M waves
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [WAVES_M][BN]
+#pragma unroll
+  for (int j = 0; j < Cfg::FN; ++j) {
+    const float m2 = __shfl_xor(m[j], 32), a2 = __shfl_xor(a[j], 32), b2 = __shfl_xor(b[j], 32);
+    const float z2 = __shfl_xor(zy[j], 32);
+    merge_stats(m[j], a[j], b[j], m2, a2, b2, p.c);
+    zy[j] += z2;
+    if (hh == 0) {
+      f32x4_t v = {m[j], a[j], b[j], zy[j]};
+      red[g.wave_m * Cfg::BN + g.wave_n * Cfg::WN + j * 32 + ln] = v;
+    }
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < Cfg::BN; t += Cfg::NTHREADS) {
+    const f32x4_t v0 = red[t];
+    float vm = v0[0], va = v0[1], vb = v0[2], vz = v0[3];
+#pragma unroll
+    for (int w = 1; w < Cfg::WAVES_M; ++w) {
+      const f32x4_t u = red[w * Cfg::BN + t];
+      merge_stats(vm, va, vb, u[0], u[1], u[2], p.c);
+      vz += u[3];
+    }
+    const int64_t tok = n0 + t;
+    const f32x4_t v = {vm, va, vb, vz};
+    if (tok < p.T) p.parts[(int64_t)s * p.T + tok] = v;
+  }
+}
+
+// merge the S partials of every token and emit the five per-token outputs
+__global__ void lce_fwd_merge_kernel(const f32x4_t* parts, int S, int64_t T, float c, float rcp_tau, float* logprobs,
+                                     float* entropy, float* maximum, float* accumulate, float* entropy_b) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const f32x4_t v0 = parts[t];
+  float vm = v0[0], va = v0[1], vb = v0[2], vz = v0[3];
+  for (int s = 1; s < S; ++s) {
+    const f32x4_t u = parts[(int64_t)s * T + t];
+    merge_stats(vm, va, vb, u[0], u[1], u[2], c);
+    vz += u[3];
+  }
+  const float mz = vm * rcp_tau;
+  const float lse = mz + logf(va);
+  const float eb = (vb / va) * rcp_tau;
+  maximum[t] = mz;
+  accumulate[t] = va;
+  entropy_b[t] = eb;
+  entropy[t] = lse - eb;
+  logprobs[t] = vz * rcp_tau - lse;
+}
+
+// deterministic single-workgroup sum of x[0..n) * scale -> out[0]
+__global__ void lce_reduce_sum_kernel(const float* x, int64_t n, float scale, float* out) {
+  __shared__ double sh[1024];
+  double acc = 0.0;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) acc += (double)x[i];
+  sh[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = (float)(sh[0] * (double)scale);
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward, stage 1: recompute a [vocab chunk] x [tokens] logit tile and write d_logits in both
+// layouts (token-major for d_hidden's GEMM, vocab-major for d_weight's GEMM)
+// ------------------------------------------------------------------------------------------------
+template <typename TIN>
+struct DsArgs {
+  const TIN* W;  // first row of the chunk
+  int64_t ldw;
+  const TIN* h;
+  int64_t ldh;
+  const int64_t* labels;
+  int64_t T, H;
+  int64_t v0;     // vocabulary index of the chunk's first row
+  int64_t vrows;  // valid rows in the chunk
+  float c, rcp_tau;
+  const float* maximum;
+  const float* accumulate;
+  const float* entropy_b;
+  const float* g_lp;  // [T] or [1]
+  int64_t g_lp_stride;  // 1 or 0
+  float g_lp_scale;     // 1, or 1/T for mean
+  const float* g_ent;   // [T] or null
+  TIN* dS;              // [T][ldS]      (token-major)
+  int64_t ldS;
+  TIN* dST;             // [vchunk][ldST] (vocab-major)
+  int64_t ldST;
+  TileMap map;          // rows = token tiles, cols = vocab tiles of the chunk
+};
+
+template <typename T>
+LCE_DEV void store4(T* dst, float a, float b, float c, float d);
+template <>
+LCE_DEV void store4<float>(float* dst, float a, float b, float c, float d) {
+  f32x4_t v = {a, b, c, d};
+  *reinterpret_cast<f32x4_t*>(dst) = v;
+}
+template <>
+LCE_DEV void store4<bf16_t>(bf16_t* dst, float a, float b, float c, float d) {
+  typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+  bf16x4_t v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
+  *reinterpret_cast<bf16x4_t*>(dst) = v;
+}
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_ds_kernel(DsArgs<typename Cfg::TIN> p) {
+  typedef typename Cfg::TIN TIN;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  int tt, vt;
+  if (!p.map.decode(blockIdx.x, tt, vt)) return;
+  const int64_t n0 = (int64_t)tt * Cfg::BN, m0 = (int64_t)vt * Cfg::BM;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
+  GemmCore<Cfg> g;
+  g.init(p.W, p.ldw, m0, p.vrows, p.h, p.ldh, n0, p.T);
+  f32x16_t acc[Cfg::FM][Cfg::FN];
+  g.run(lds, p.H, acc);
+
+  const int vloc0 = (int)m0 + g.wave_m * Cfg::WM;  // chunk-local vocabulary index of this wave's first row
+#pragma unroll
+  for (int j = 0; j < Cfg::FN; ++j) {
+    const int64_t tok = n0 + g.wave_n * Cfg::WN + j * 32 + ln;
+    const bool tok_ok = tok < p.T;
+    float lse2 = 0.f, C0 = 0.f, C1 = 0.f, G = 0.f;
+    int rel = -1;
+    if (tok_ok) {
+      const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
+      const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
+      lse2 = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
+      G = glp * p.rcp_tau;
+      C1 = -gent * p.rcp_tau * p.rcp_tau;
+      C0 = -G + gent * p.entropy_b[tok] * p.rcp_tau;
+      const int64_t y = p.labels[tok] - p.v0;
+      rel = (y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        __builtin_amdgcn_sched_barrier(0);
+        float d[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int r = q * 4 + u;
+          const float x = acc[i][j][r];
+          const float pr = fast_exp2(__builtin_fmaf(x, p.c, -lse2));
+          float dv = pr * __builtin_fmaf(x, C1, C0);
+          const int row = acc_row(i, r, hh);
+          if (row == rel) dv += G;
+          if (!tok_ok || vloc0 + row >= p.vrows) dv = 0.f;
+          d[u] = dv;
+        }
+        const int vrow = vloc0 + i * 32 + 8 * q + 4 * hh;  // chunk-local vocab index of d[0]
+        if (tok_ok && vrow < p.ldS) store4<TIN>(p.dS + tok * p.ldS + vrow, d[0], d[1], d[2], d[3]);
+        if (tok < p.ldST) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) p.dST[(int64_t)(vrow + u) * p.ldST + tok] = (TIN)d[u];
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// plain NT GEMM with the shared mainloop: C[m][n] = sum_k A[m][k] B[n][k]
+//   out_mode 0: Cf = acc           1: Cf += acc
+//            2: Ct = (TIN)acc      3: Ct = (TIN)(Cf + acc)
+// ------------------------------------------------------------------------------------------------
+template <typename TIN>
+struct GemmArgs {
+  const TIN* A;
+  int64_t lda;
+  const TIN* B;
+  int64_t ldb;
+  int64_t M, N, K;
+  float* Cf;
+  int64_t ldcf;
+  TIN* Ct;
+  int64_t ldct;
+  int out_mode;
+  TileMap map;  // rows = M tiles, cols = N tiles
+};
+
+template <typename Cfg, int MODE, bool EDGE>
+LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t m0,
+                           int64_t n0, int wave_m, int wave_n, int hh, int ln) {
+  typedef typename Cfg::TIN TIN;
+  const int64_t mw = m0 + wave_m * Cfg::WM + 4 * hh;  // row of register 0 of block row 0
+#pragma unroll
+  for (int j = 0; j < Cfg::FN; ++j) {
+    const int64_t n = n0 + wave_n * Cfg::WN + j * 32 + ln;
+    if (EDGE && n >= p.N) continue;
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i) {
+      __builtin_amdgcn_sched_barrier(0);  // one 32x32 block at a time (register pressure)
+      float* cf = (MODE != 2) ? p.Cf + (mw + i * 32) * p.ldcf + n : nullptr;
+      TIN* ct = (MODE & 2) ? p.Ct + (mw + i * 32) * p.ldct + n : nullptr;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (EDGE && mw + i * 32 + 8 * q + u >= p.M) continue;
+          float v = acc[i][j][q * 4 + u];
+          if (MODE & 1) v += cf[(8 * q + u) * p.ldcf];
+          if (MODE & 2) ct[(8 * q + u) * p.ldct] = (TIN)v;
+          else cf[(8 * q + u) * p.ldcf] = v;
+        }
+      }
+    }
+  }
+}
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void gemm_nt_kernel(GemmArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  int tm, tn;
+  if (!p.map.decode(blockIdx.x, tm, tn)) return;
+  const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
+  GemmCore<Cfg> g;
+  g.init(p.A, p.lda, m0, p.M, p.B, p.ldb, n0, p.N);
+  f32x16_t acc[Cfg::FM][Cfg::FN];
+  g.run(lds, p.K, acc);
+  const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
+#define LCE_EPI(MODE)                                                                           \
+  if (edge) gemm_epilogue<Cfg, MODE, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);         \
+  else gemm_epilogue<Cfg, MODE, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln)
+  switch (p.out_mode) {
+    case 0: LCE_EPI(0); break;
+    case 1: LCE_EPI(1); break;
+    case 2: LCE_EPI(2); break;
+    default: LCE_EPI(3); break;
+  }
+#undef LCE_EPI
+}
+
+__global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+// out[c][r] = in[r][c] for r < R, c < C; out has `ldo` columns and columns [R, ldo) are zero-filled.
+// Grid: (ceil(ldo/64), ceil(C/64)), 256 threads.
+template <typename TIN>
+__global__ void transpose_pad_kernel(const TIN* in, int64_t ldi, int64_t R, int64_t C, TIN* out, int64_t ldo) {
+  __shared__ TIN tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? in[r * ldi + c] : (TIN)0.f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t c = c0 + i, r = r0 + tx;
+    if (c < C && r < ldo) out[c * ldo + r] = tile[tx][i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// unfused twins on materialised logits: one workgroup per row, one pass
+// ------------------------------------------------------------------------------------------------
+template <typename TIN>
+LCE_DEV float load_as_float(const TIN* p, int64_t i) { return (float)p[i]; }
+
+template <typename TIN, int NT>
+LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, float* sh) {
+  // per-thread online (max, sum exp, sum z exp) in natural-log units scaled to base 2
+  float tm = kNegBig, ta = 0.f, tb = 0.f;
+  for (int64_t v = threadIdx.x; v < V; v += NT) {
+    const float z = load_as_float(row, v);
+    if (z > tm) {
+      const float sc = fast_exp2((tm - z) * kLog2e);
+      ta *= sc;
+      tb *= sc;
+      tm = z;
+    }
+    const float e = fast_exp2((z - tm) * kLog2e);
+    ta += e;
+    tb = __builtin_fmaf(z, e, tb);
+  }
+  // wave reduce
+  for (int off = 32; off > 0; off >>= 1) {
+    const float m2 = __shfl_xor(tm, off), a2 = __shfl_xor(ta, off), b2 = __shfl_xor(tb, off);
+    merge_stats(tm, ta, tb, m2, a2, b2, kLog2e);
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) {
+    sh[wave * 3 + 0] = tm;
+    sh[wave * 3 + 1] = ta;
+    sh[wave * 3 + 2] = tb;
+  }
+  __syncthreads();
+  tm = sh[0];
+  ta = sh[1];
+  tb = sh[2];
+  for (int w = 1; w < NT / 64; ++w) merge_stats(tm, ta, tb, sh[w * 3], sh[w * 3 + 1], sh[w * 3 + 2], kLog2e);
+  m = tm;
+  a = ta;
+  b = tb;
+  __syncthreads();
+}
+
+template <typename TIN, int NT>
+__global__ __launch_bounds__(NT) void logits_fwd_kernel(const TIN* logits, int64_t ldl, const int64_t* labels, int64_t V,
+                                                        float* logprobs, float* entropy) {
+  __shared__ float sh[3 * NT / 64];
+  const int64_t r = blockIdx.x;
+  const TIN* row = logits + r * ldl;
+  float m, a, b;
+  row_stats<TIN, NT>(row, V, m, a, b, sh);
+  if (threadIdx.x == 0) {
+    const float lse = m + logf(a);
+    if (entropy) entropy[r] = lse - b / a;
+    if (logprobs) {
+      const int64_t y = labels[r];
+      const float zy = (y >= 0 && y < V) ? load_as_float(row, y) : 0.f;
+      logprobs[r] = zy - lse;
+    }
+  }
+}
+
+template <typename TIN, int NT>
+__global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64_t ldl, const int64_t* labels, int64_t V,
+                                                        const float* g_lp, const float* g_ent, TIN* dl, int64_t ldd) {
+  __shared__ float sh[3 * NT / 64];
+  const int64_t r = blockIdx.x;
+  const TIN* row = logits + r * ldl;
+  float m, a, b;
+  row_stats<TIN, NT>(row, V, m, a, b, sh);
+  const float lse2 = (m + logf(a)) * kLog2e;
+  const float eb = b / a;
+  const float glp = g_lp ? g_lp[r] : 0.f;
+  const float gent = g_ent ? g_ent[r] : 0.f;
+  const int64_t y = (g_lp && labels) ? labels[r] : -1;
+  TIN* out = dl + r * ldd;
+  for (int64_t v = threadIdx.x; v < V; v += NT) {
+    const float z = load_as_float(row, v);
+    const float pr = fast_exp2(__builtin_fmaf(z, kLog2e, -lse2));
+    float d = pr * (-glp - gent * (z - eb));
+    if (v == y) d += glp;
+    out[v] = (TIN)d;
+  }
+}
+
+}  // namespace lce

@@ -1,0 +1,189 @@
+"""Host launchers of the fused lm-head log-prob + entropy kernels.
+
+Same names, argument meaning, return tuples and error behaviour as the reference's
+``verl/utils/kernel/kernels.py`` (enums :102-156, ``Config`` :160-172, ``set_backward_method`` :175-180,
+``efficient_entropy_forward`` :569-759, ``efficient_entropy_backward`` :1518-1729); the device work is
+done by hand-written gfx950 kernels behind the C ABI of ``liblce_gfx950.so``.
+
+Differences that are deliberate (all inside the reference's own tolerances):
+* the per-token max is the true max of the logits (the reference seeds its merge with 0);
+* ``d_hidden`` / ``d_weight`` are accumulated in fp32 over vocabulary chunks and rounded once;
+* ``BackwardEnum`` values are accepted by ``set_backward_method`` but select nothing: there is one
+  backward schedule (recompute a vocab-chunk of d_logits, then two MFMA GEMMs);
+* labels outside ``[0, V)`` give ``logprob = -logsumexp`` instead of reading uninitialised memory;
+* ``dist_process_group`` (vocab-parallel) raises ``NotImplementedError``.
+"""
+
+from __future__ import annotations
+
+import typing
+from dataclasses import dataclass
+
+import torch
+
+from ... import _abi
+
+
+@dataclass
+class EntropyReductionEnum:
+    _None = 0
+    _Sum = 1
+    _Mean = 2
+
+
+def get_entropy_reduction_enum_number(reduction: str) -> int:
+    if reduction == "none":
+        return EntropyReductionEnum._None
+    if reduction == "sum":
+        return EntropyReductionEnum._Sum
+    if reduction == "mean":
+        return EntropyReductionEnum._Mean
+    raise ValueError(f"Invalid reduction: {reduction}")
+
+
+def get_entropy_reduction_enum(ce_reduction: int) -> int:
+    if ce_reduction in (0, 1, 2):
+        return ce_reduction
+    raise ValueError(f"Invalid ce_reduction: {ce_reduction}")
+
+
+@dataclass
+class BackwardEnum:
+    _Total_Fuse_MN = 0
+    _Total_Separate = 1
+    _Split_Dlogits_N = 2
+    _Split_Dlogits_M = 3
+
+
+@dataclass
+class Config:
+    _backward: int = BackwardEnum._Split_Dlogits_N
+    _use_triton: bool = False  # kept for attribute compatibility; there is no Triton here
+    _vocab_chunk: int = 0  # columns of d_logits alive at once in the backward (0 = library default)
+
+
+_config = Config()
+
+
+def set_backward_method(backward_method: int):
+    """Accepted for compatibility; every method maps to the one HIP backward schedule."""
+    global _config
+    _config._backward = backward_method
+
+
+def set_vocab_chunk(columns: int):
+    """Vocabulary columns of d_logits materialised per backward step (multiple of 256; 0 = default)."""
+    global _config
+    _config._vocab_chunk = int(columns)
+
+
+def _check_inputs(hidden, weight, labels):
+    assert hidden.is_cuda and weight.is_cuda and labels.is_cuda
+    assert weight.device == hidden.device and labels.device == hidden.device
+    assert hidden.dim() == 2 and weight.dim() == 2 and labels.dim() == 1
+    assert hidden.is_contiguous() and weight.is_contiguous() and labels.is_contiguous()
+    assert hidden.shape[0] == labels.shape[0] and hidden.shape[1] == weight.shape[1]
+    assert hidden.shape[1] % 128 == 0
+    if hidden.dtype != weight.dtype:
+        raise NotImplementedError(f"hidden ({hidden.dtype}) and weight ({weight.dtype}) must share a dtype")
+    if labels.dtype != torch.int64:
+        raise NotImplementedError(f"labels must be int64, got {labels.dtype}")
+    return _abi.dtype_code(hidden.dtype)
+
+
+def efficient_entropy_forward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    reduction: typing.Optional[int] = 2,
+    temperature: typing.Optional[float] = 1.0,
+    dist_process_group=None,
+) -> list[torch.Tensor]:
+    """Returns (logprobs, entropy, maximum, accumulate, entropy_b), all fp32."""
+    if dist_process_group is not None:
+        raise NotImplementedError("vocab-parallel (dist_process_group) is not built: one GPU, no collectives")
+    code = _check_inputs(hidden, weight, labels)
+    reduction = get_entropy_reduction_enum(reduction)
+    assert temperature > 0, "temperature must be positive"
+    T, H = hidden.shape
+    V = weight.shape[0]
+    dev = hidden.device
+    f32 = dict(device=dev, dtype=torch.float32)
+    logprobs = torch.empty((T,) if reduction == 0 else (), **f32)
+    entropy = torch.empty((T,), **f32)
+    maximum = torch.empty((T,), **f32)
+    acc_eb = torch.empty((2, T), **f32)
+    accumulate, entropy_b = acc_eb[0], acc_eb[1]
+    if T == 0:
+        if reduction != 0:
+            logprobs.zero_()
+        return logprobs, entropy, maximum, accumulate, entropy_b
+    lib = _abi.load()
+    with torch.cuda.device(dev):
+        ws_bytes = lib.lce_forward_workspace_bytes(T, H, V, code)
+        ws = torch.empty((ws_bytes,), device=dev, dtype=torch.uint8)
+        rc = lib.lce_forward(
+            hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V, code,
+            float(temperature), reduction, logprobs.data_ptr(), entropy.data_ptr(), maximum.data_ptr(),
+            accumulate.data_ptr(), entropy_b.data_ptr(), ws.data_ptr(), ws_bytes, _abi.current_stream(dev),
+        )  # fmt: skip
+        _abi.check(rc, "lce_forward")
+    return logprobs, entropy, maximum, accumulate, entropy_b
+
+
+def efficient_entropy_backward(
+    dlogprobs: torch.Tensor,
+    dentropy: typing.Optional[torch.Tensor],
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    maximum: torch.Tensor,
+    acc: torch.Tensor,
+    entropy_b: torch.Tensor,
+    reduction: typing.Optional[int] = 2,
+    should_return_fp32_grad: bool = False,
+    temperature: typing.Optional[float] = 1.0,
+    dist_process_group=None,
+) -> list[torch.Tensor]:
+    """Returns (d_hidden, d_weight) in ``hidden.dtype`` (fp32 when ``should_return_fp32_grad``)."""
+    if dist_process_group is not None:
+        raise NotImplementedError("vocab-parallel (dist_process_group) is not built: one GPU, no collectives")
+    if _config._backward == BackwardEnum._Split_Dlogits_M:
+        raise NotImplementedError("BackwardEnum._Split_Dlogits_M is not implemented yet")
+    code = _check_inputs(hidden, weight, labels)
+    reduction = get_entropy_reduction_enum(reduction)
+    T, H = hidden.shape
+    V = weight.shape[0]
+    dev = hidden.device
+    if reduction == 0:
+        assert dlogprobs.shape == (T,)
+    else:
+        assert dlogprobs.dim() == 0
+    assert dlogprobs.is_cuda and dlogprobs.device == dev
+    assert maximum.shape == labels.shape == acc.shape and entropy_b.shape == (T,)
+    assert maximum.is_contiguous() and acc.is_contiguous() and entropy_b.is_contiguous()
+    g_lp = dlogprobs.detach().to(torch.float32).contiguous()
+    g_ent = None
+    if dentropy is not None:
+        assert dentropy.is_cuda and dentropy.device == dev and dentropy.shape == (T,)
+        g_ent = dentropy.detach().to(torch.float32).contiguous()
+    d_hidden = torch.empty_like(hidden)
+    d_weight = torch.empty((V, H), device=dev, dtype=hidden.dtype)
+    if T == 0:
+        d_weight.zero_()
+    else:
+        lib = _abi.load()
+        with torch.cuda.device(dev):
+            vchunk = _config._vocab_chunk
+            ws_bytes = lib.lce_backward_workspace_bytes(T, H, V, code, vchunk)
+            ws = torch.empty((ws_bytes,), device=dev, dtype=torch.uint8)
+            rc = lib.lce_backward(
+                hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
+                code, float(temperature), reduction, maximum.data_ptr(), acc.data_ptr(), entropy_b.data_ptr(),
+                g_lp.data_ptr(), _abi.ptr(g_ent), d_hidden.data_ptr(), d_weight.data_ptr(), ws.data_ptr(), ws_bytes,
+                vchunk, _abi.current_stream(dev),
+            )  # fmt: skip
+            _abi.check(rc, "lce_backward")
+    if should_return_fp32_grad:
+        d_hidden, d_weight = d_hidden.float(), d_weight.float()
+    return d_hidden, d_weight

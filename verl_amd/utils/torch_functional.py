@@ -1,0 +1,127 @@
+"""Unfused twins on logits that already exist: ``logprobs_from_logits`` and ``entropy_from_logits``.
+
+Same signatures and result dtypes/shapes as the reference's ``verl/utils/torch_functional.py``
+(``gather_from_labels`` :50-70, ``logprobs_from_logits`` :73-107, ``logprobs_from_logits_naive`` :155-170,
+``logprobs_from_logits_v2`` :173-207, ``entropy_from_logits`` :231-245, ``entropy_from_logits_with_chunking``
+:248-270, ``masked_sum`` :273-291, ``masked_mean`` :294-308).  The row reductions run as single-pass
+HIP kernels (one read of the logits; fp32 arithmetic whatever the storage dtype) with an autograd
+backward that is one more fused pass; there is no eager fallback on this path.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _abi
+
+
+def gather_from_labels(data: torch.Tensor, label: torch.Tensor) -> torch.Tensor:
+    return torch.gather(data, -1, label.unsqueeze(-1)).squeeze(-1)
+
+
+def _as_rows(logits: torch.Tensor):
+    V = logits.shape[-1]
+    rows = logits.reshape(-1, V)
+    if rows.stride(-1) != 1:
+        rows = rows.contiguous()
+    return rows, V
+
+
+def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool):
+    assert logits.is_cuda, "verl_amd.utils.torch_functional runs on the GPU only"
+    code = _abi.dtype_code(logits.dtype)
+    rows, V = _as_rows(logits)
+    R = rows.shape[0]
+    dev = logits.device
+    lp = torch.empty((R,), device=dev, dtype=torch.float32) if want_logprobs else None
+    ent = torch.empty((R,), device=dev, dtype=torch.float32) if want_entropy else None
+    y = None
+    if want_logprobs:
+        y = labels.reshape(-1).to(torch.int64).contiguous()
+        assert y.shape[0] == R and y.device == dev
+    if R > 0:
+        with torch.cuda.device(dev):
+            rc = _abi.load().lce_logits_forward(
+                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, code, _abi.ptr(lp), _abi.ptr(ent),
+                _abi.current_stream(dev),
+            )  # fmt: skip
+            _abi.check(rc, "lce_logits_forward")
+    return rows, y, lp, ent
+
+
+def _logits_backward(rows, y, g_lp, g_ent, out_shape, out_dtype):
+    R, V = rows.shape
+    dev = rows.device
+    d = torch.empty((R, V), device=dev, dtype=rows.dtype)
+    g_lp = None if g_lp is None else g_lp.reshape(-1).to(torch.float32).contiguous()
+    g_ent = None if g_ent is None else g_ent.reshape(-1).to(torch.float32).contiguous()
+    if R > 0:
+        with torch.cuda.device(dev):
+            rc = _abi.load().lce_logits_backward(
+                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, _abi.dtype_code(rows.dtype), _abi.ptr(g_lp),
+                _abi.ptr(g_ent), d.data_ptr(), d.stride(0), _abi.current_stream(dev),
+            )  # fmt: skip
+            _abi.check(rc, "lce_logits_backward")
+    return d.reshape(out_shape).to(out_dtype)
+
+
+class _LogprobsFromLogits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, labels):
+        rows, y, lp, _ = _logits_forward(logits, labels, True, False)
+        ctx.save_for_backward(rows, y)
+        ctx.shape, ctx.dtype = logits.shape, logits.dtype
+        return lp.reshape(logits.shape[:-1]).to(logits.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        rows, y = ctx.saved_tensors
+        return _logits_backward(rows, y, g, None, ctx.shape, ctx.dtype), None
+
+
+class _EntropyFromLogits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, out_dtype):
+        rows, _, _, ent = _logits_forward(logits, None, False, True)
+        ctx.save_for_backward(rows)
+        ctx.shape, ctx.dtype = logits.shape, logits.dtype
+        return ent.reshape(logits.shape[:-1]).to(out_dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        (rows,) = ctx.saved_tensors
+        return _logits_backward(rows, None, None, g, ctx.shape, ctx.dtype), None
+
+
+def logprobs_from_logits(logits, labels, inplace_backward=True):
+    """log_softmax(logits)[label]; shape ``logits.shape[:-1]``, dtype of ``logits``.
+    ``inplace_backward`` is accepted for signature compatibility; the logits are never overwritten."""
+    return _LogprobsFromLogits.apply(logits, labels)
+
+
+def logprobs_from_logits_naive(logits, labels):
+    return _LogprobsFromLogits.apply(logits, labels)
+
+
+def logprobs_from_logits_v2(logits, labels):
+    return _LogprobsFromLogits.apply(logits, labels)
+
+
+def entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """logsumexp(logits) - sum(softmax(logits) * logits); dtype of ``logits``."""
+    return _EntropyFromLogits.apply(logits, logits.dtype)
+
+
+def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048) -> torch.Tensor:
+    """Same value, always fp32 like the reference's chunked variant; the kernel needs no chunking."""
+    return _EntropyFromLogits.apply(logits, torch.float32)
+
+
+def masked_sum(values, mask, axis=None):
+    valid_values = torch.where(mask.bool(), values, 0.0)
+    return (valid_values * mask).sum(axis=axis)
+
+
+def masked_mean(values, mask, axis=None):
+    s = masked_sum(values, mask, axis)
+    return s / (mask.sum(axis=axis) + 1e-8)
