@@ -1,0 +1,176 @@
+"""Headline benchmark: fwd+bwd tokens/s of the fused lm-head log-prob + entropy at a Qwen2.5-7B-shaped head.
+
+One "step" = linear_cross_entropy forward + backward over one synthetic micro-batch that is
+already resident in HBM (T=16384, H=3584, V=152064, bf16, temperature 1.0, upstream grads ~N(0,1)).
+Prints ONE JSON line with the throughput, the roofline of the dominant kernel (HIP-event timed in
+this run) and the CPU baseline (the oracle's torch restatement on the host cores, bounded sample).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
+WORKLOADS = {
+    # name: (T, H, V, temperature, weight std)
+    "qwen2.5-7b-head-T16384": (16384, 3584, 152064, 1.0, 0.02),
+    "llama3-8b-head-T32768": (32768, 4096, 128256, 0.6, 0.02),
+    "qwen2.5-32b-head-T65536": (65536, 5120, 152064, 1.0, 0.015),
+    "small": (2048, 1024, 32768, 1.0, 0.02),
+}
+
+
+def cpu_baseline(seconds_budget: float = 20.0):
+    """The oracle's torch restatement (materialised fp32 logits) on the host cores: forward on the
+    CPU-runnable reference case (T=1024, H=896, V=151936), bounded to a sample of rows sized so the
+    whole leg takes about `seconds_budget`; reported in tokens/s."""
+    import torch
+
+    from oracle import lce_oracle as O
+
+    cores = os.cpu_count() or 1
+    # respect the box's CPU share if it is advertised
+    for var in ("OMP_NUM_THREADS", "MAX_JOBS"):
+        if os.environ.get(var, "").isdigit():
+            cores = min(cores, int(os.environ[var]))
+            break
+    torch.set_num_threads(cores)
+    T, H, V = 1024, 896, 151936
+    g = torch.Generator().manual_seed(1235)
+    h = torch.randn(T, H, generator=g)
+    w = torch.randn(V, H, generator=g) * 0.02
+    y = torch.randint(0, V, (T,), generator=g)
+    rows = 128
+    t0 = time.perf_counter()
+    O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)  # warm-up, also sizes the sample
+    dt = time.perf_counter() - t0
+    rows = int(max(128, min(T, rows * (seconds_budget / 3.0) / max(dt, 1e-3))))
+    rows = (rows // 128) * 128
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[1]
+    return {
+        "value": rows / med,
+        "unit": "tokens/s (forward only, fp32)",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"oracle torch restatement, forward, first {rows} of T=1024 rows, H=896, V=151936, fp32, median of 3",
+        "gflops": 2.0 * rows * H * V / med / 1e9,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--variant", type=int, default=-1)
+    ap.add_argument("--vchunk", type=int, default=-1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from verl_amd import _abi, linear_cross_entropy
+    from verl_amd.utils.kernel import kernels as K
+
+    lib = _abi.load()
+    if args.variant >= 0:
+        _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
+    if args.vchunk >= 0:
+        K.set_vocab_chunk(args.vchunk)
+    dev = torch.device("cuda:0")
+    T, H, V, tau, wstd = WORKLOADS[args.workload]
+    g = torch.Generator(device=dev).manual_seed(1234 + 2)
+    h = torch.randn(T, H, device=dev, generator=g).bfloat16().requires_grad_(True)
+    w = (torch.randn(V, H, device=dev, generator=g) * wstd).bfloat16().requires_grad_(True)
+    y = torch.randint(0, V, (T,), device=dev, generator=g)
+    g_lp = torch.randn(T, device=dev, generator=g)
+    g_ent = torch.randn(T, device=dev, generator=g)
+
+    def step():
+        h.grad = None
+        w.grad = None
+        lp, ent = linear_cross_entropy(h, w, y, tau, "none")
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = T / (elapsed / args.steps)
+
+    # per-kernel durations with HIP events on the launch stream (second pass, same process)
+    lib.lce_profile_enable(1)
+    _abi.profile_read(reset=True)
+    nprof = max(2, min(args.steps, 5))
+    for _ in range(nprof):
+        step()
+    torch.cuda.synchronize()
+    prof = _abi.profile_read(reset=True)
+    lib.lce_profile_enable(0)
+    kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
+    # the dominant kernel (largest share of the step) and its algorithmic FLOPs per launch:
+    # every MFMA kernel of the path does 2*T*V*H per step split over its launches
+    mfma = {k: v for k, v in kernels.items() if k.startswith(("lce_fwd_kernel", "lce_bwd_ds", "gemm_nt"))}
+    dom = max(mfma, key=lambda k: mfma[k]["ms_per_step"])
+    flops_per_launch = 2.0 * T * V * H / mfma[dom]["launches_per_step"]
+    achieved = flops_per_launch / (mfma[dom]["avg_ms"] * 1e-3)
+    roofline = {
+        "bound": "mfma",
+        "kernel": dom,
+        "achieved": achieved / 1e12,
+        "peak": PEAK_BF16 / 1e12,
+        "unit": "TFLOP/s",
+        "frac": achieved / PEAK_BF16,
+        "traffic": None,
+        "avg_launch_ms": mfma[dom]["avg_ms"],
+        "flops_per_launch": flops_per_launch,
+    }
+    algorithmic = 6.0 * T * V * H / (elapsed / args.steps)
+    out = {
+        "metric": "fwd+bwd tokens/s, 7B lm-head logprob+entropy; % of bf16 MFMA peak",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd+bwd"},
+        "algorithmic_tflops": algorithmic / 1e12,  # 6*T*V*H per step
+        "frac_of_bf16_peak": algorithmic / PEAK_BF16,
+        "executed_tflops": 8.0 * T * V * H / (elapsed / args.steps) / 1e12,  # one recompute of the logits
+        "roofline": roofline,
+        "kernels": kernels,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

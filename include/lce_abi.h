@@ -86,6 +86,16 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 int lce_set_variant(int variant);
 int lce_num_variants(void);
 
+/* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every kernel
+ * launch of the library is bracketed by HIP events on the caller's stream; lce_profile_read waits
+ * for them and returns, per kernel class c < lce_profile_num_classes(), the summed duration in
+ * milliseconds and the number of launches (arrays sized by the caller).  Creating events allocates
+ * host-side driver objects, so keep it disabled under graph capture. */
+int lce_profile_enable(int on);
+int lce_profile_num_classes(void);
+const char* lce_profile_class_name(int cls);
+int lce_profile_read(double* total_ms, int64_t* launches, int reset);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,112 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports every symbol the
+header declares, and the Python surface rejects bad arguments the way the reference does
+(verl/utils/kernel/linear_cross_entropy.py:64-65, verl/utils/kernel/kernels.py:113-126)."""
+
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from verl_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_functions():
+    text = open(os.path.join(ROOT, "include", "lce_abi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lce_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _header_functions()
+    assert len(names) >= 12
+    lib = ctypes.CDLL(_abi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/lce_abi.h but not exported"
+    assert sorted(_abi.SYMBOLS) == names, "python binding and header disagree"
+
+
+def test_abi_version_and_error_string():
+    lib = _abi.load()
+    assert lib.lce_abi_version() == _abi.ABI_VERSION
+    assert lib.lce_num_variants() >= 1
+    assert lib.lce_set_variant(10_000) != 0
+    assert b"variant" in lib.lce_last_error()
+    # argument validation happens before any device work
+    rc = lib.lce_forward(None, 128, None, 128, None, 4, 100, 10, 0, 1.0, 0, None, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"multiple of 64" in lib.lce_last_error()
+    rc = lib.lce_forward(None, 128, None, 128, None, 4, 128, 10, 7, 1.0, 0, None, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"dtype" in lib.lce_last_error()
+    assert lib.lce_forward_workspace_bytes(16384, 3584, 152064, 0) < (64 << 20)
+    # backward workspace stays far below a [T, V] tile pair: bounded d_logits chunk + transposed operands + fp32 d_hidden
+    T, H, V = 16384, 3584, 152064
+    assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) < 0.25 * T * V * 2 + 4 * V * H
+
+
+def test_signature_matches_reference():
+    from verl_amd.utils.kernel.linear_cross_entropy import LinearCrossEntropy
+    from verl_amd.utils.kernel import kernels
+
+    sig = inspect.signature(LinearCrossEntropy.forward)
+    assert list(sig.parameters) == ["ctx", "hidden", "weight", "labels", "temperature", "reduction", "dist_process_group"]
+    assert sig.parameters["temperature"].default == 1.0 and sig.parameters["reduction"].default == "none"
+    fsig = inspect.signature(kernels.efficient_entropy_forward)
+    assert list(fsig.parameters) == ["hidden", "weight", "labels", "reduction", "temperature", "dist_process_group"]
+    bsig = inspect.signature(kernels.efficient_entropy_backward)
+    assert list(bsig.parameters) == [
+        "dlogprobs", "dentropy", "hidden", "weight", "labels", "maximum", "acc", "entropy_b", "reduction",
+        "should_return_fp32_grad", "temperature", "dist_process_group",
+    ]  # fmt: skip
+    assert kernels.get_entropy_reduction_enum_number("none") == 0
+    assert kernels.get_entropy_reduction_enum_number("sum") == 1
+    assert kernels.get_entropy_reduction_enum_number("mean") == 2
+    with pytest.raises(ValueError, match="Invalid reduction"):
+        kernels.get_entropy_reduction_enum_number("max")
+    kernels.set_backward_method(kernels.BackwardEnum._Total_Separate)
+    kernels.set_backward_method(kernels.BackwardEnum._Split_Dlogits_N)
+
+
+def test_argument_errors_before_device_work():
+    from verl_amd import linear_cross_entropy
+
+    h = torch.zeros(4, 128)
+    w = torch.zeros(16, 128)
+    y = torch.zeros(4, dtype=torch.long)
+    with pytest.raises(AssertionError, match="temperature must be a float"):
+        linear_cross_entropy(h, w, y, 1, "none")
+    with pytest.raises(AssertionError, match="reduction must be a str"):
+        linear_cross_entropy(h, w, y, 1.0, None)
+    with pytest.raises(ValueError, match="Invalid reduction"):
+        linear_cross_entropy(h, w, y, 1.0, "max")
+    with pytest.raises(AssertionError):  # CPU tensors: the reference asserts is_cuda
+        linear_cross_entropy(h, w, y, 1.0, "none")
+
+
+def test_no_fallback_when_library_is_missing(monkeypatch, tmp_path):
+    monkeypatch.setattr(_abi, "_lib", None)
+    monkeypatch.setattr(_abi, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_abi.LceError, match="no CPU or eager fallback"):
+        _abi.load()
+
+
+def test_product_code_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "verl_amd")
+    for d, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(d, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_fused_linear_for_ppo_constructor():
+    from verl_amd.utils.experimental.torch_functional import FusedLinearForPPO
+
+    with pytest.raises(ValueError):  # tests/utils/test_experimental_torch_functional_on_cpu.py:127-129
+        FusedLinearForPPO(impl_backend="nope")
+    m = FusedLinearForPPO(chunk_size=3)
+    with pytest.raises(ValueError):
+        m(torch.zeros(2, 3, 4, 8), torch.zeros(5, 8), torch.zeros(2, 3, 4, dtype=torch.long))

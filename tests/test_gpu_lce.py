@@ -1,0 +1,319 @@
+"""Parity of the HIP path against the oracle, through the Python surface that sits on the C ABI.
+
+Shapes, input distributions and tolerances of the first block are the reference's own
+(tests/utils/test_linear_cross_entropy.py:101-163, :219-224, :271-276).  North-star bars are stated
+where they are applied: 2e-2 absolute for bf16 inputs, 1e-5 relative for fp32 inputs, on values and
+gradients alike.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import lce_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _uniform_case(T, H, V, dtype, seed, tau=1.5):
+    g = torch.Generator().manual_seed(seed)
+    h = (torch.rand(T, H, generator=g) - 0.5).to(dtype).to(DEV)
+    w = (torch.rand(V, H, generator=g) - 0.5).to(dtype).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_ent = (torch.rand(T, generator=g) - 0.5).to(dtype).to(DEV)
+    g_lp = (torch.rand(T, generator=g) * 2 - 1).to(dtype).to(DEV)
+    return h, w, y, g_lp, g_ent
+
+
+def _run(h, w, y, tau, g_lp, g_ent, reduction="none"):
+    from verl_amd import linear_cross_entropy
+
+    h = h.clone().requires_grad_(True)
+    w = w.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(h, w, y, tau, reduction)
+    torch.autograd.backward([lp, ent], [g_lp, g_ent])
+    torch.cuda.synchronize()
+    return lp, ent, h.grad, w.grad
+
+
+REFERENCE_SHAPES = [(1937, 3584, 152064), (2169, 896, 151936), (1530, 2048, 32256), (1388, 4096, 102400),
+                    (8192, 4096, 102400)]
+
+
+@pytest.mark.parametrize("shape", REFERENCE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_reference_shapes_bf16(shape):
+    T, H, V = shape
+    tau = 1.5
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=T)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau)
+    assert lp.dtype == torch.float32 and ent.dtype == torch.float32 and lp.shape == (T,) and ent.shape == (T,)
+    torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+    torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    assert dh.dtype == torch.bfloat16 and dw.dtype == torch.bfloat16 and dh.shape == h.shape and dw.shape == w.shape
+    torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    # north-star bar: 2e-2 absolute on values and gradients
+    assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2
+    assert (dh.float() - rdh).abs().max() < 2e-2 and (dw.float() - rdw).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("V", [152064, 149 * 1024])
+def test_padded_vocab_known_answer(V):
+    """The reference's regression vector (tests/utils/test_linear_cross_entropy.py:352-395): padded
+    vocabulary columns must count as -inf, not as logit 0.  Every row: one logit +3, V-1 logits -15."""
+    from verl_amd import linear_cross_entropy
+
+    tau, H, T = 1.5, 3584, 512
+    w = torch.zeros(V, H, dtype=torch.bfloat16, device=DEV)
+    w[:, 0] = -15.0 * tau
+    w[0, 0] = 3.0 * tau
+    h = torch.zeros(1, T, H, dtype=torch.bfloat16, device=DEV)
+    h[:, :, 0] = 1.0
+    y = torch.zeros(1, T, dtype=torch.long, device=DEV)
+    lp, ent = linear_cross_entropy(h, w, y, tau, "none")
+    want_lp, want_ent = O.padded_vocab_known_answer(V)
+    assert want_lp == pytest.approx({152064: -0.00231323880878, 152576: -0.00232101851094}[V], rel=1e-9)
+    torch.testing.assert_close(lp, torch.full((T,), want_lp, device=DEV), atol=1e-5, rtol=1e-3)
+    torch.testing.assert_close(ent, torch.full((T,), want_ent, device=DEV), atol=1e-5, rtol=1e-3)
+
+
+@pytest.mark.parametrize("shape", [(300, 256, 1000), (1025, 128, 4099), (64, 384, 50257), (2048, 1024, 8192)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("tau", [1.0, 0.6])
+def test_fp32_inputs_relative_1e5(shape, tau):
+    """fp32 inputs take true-fp32 MFMA; the bar is 1e-5 relative (to the largest magnitude of each
+    output) against the oracle evaluated in fp64."""
+    T, H, V = shape
+    g = torch.Generator().manual_seed(V)
+    h = torch.randn(T, H, generator=g).to(DEV)
+    w = (torch.randn(V, H, generator=g) * 0.05).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = torch.randn(T, generator=g).to(DEV)
+    g_ent = torch.randn(T, generator=g).to(DEV)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau, compute_dtype=torch.float64)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+    for got, want in ((lp, rlp), (ent, rent), (dh, rdh), (dw, rdw)):
+        assert got.dtype == torch.float32
+        err = (got.double() - want).abs().max().item()
+        assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
+
+
+@pytest.mark.parametrize("reduction", ["sum", "mean"])
+def test_reductions(reduction):
+    T, H, V, tau = 700, 256, 3001, 1.3
+    h, w, y, _, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=5, tau=tau)
+    g_lp = torch.tensor(0.7, device=DEV)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent.float(), reduction)
+    rlp, rent = O.lce_forward(h, w, y, tau, reduction)
+    assert lp.dim() == 0 and ent.shape == (T,)
+    torch.testing.assert_close(lp, rlp, atol=1e-2 if reduction == "sum" else 1e-4, rtol=1e-4)
+    torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+    rdh, rdw = O.lce_backward(g_lp, g_ent.float(), h, w, y, tau, reduction)
+    torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
+def test_api_contract_on_device():
+    from verl_amd import linear_cross_entropy
+    from verl_amd.utils.kernel import kernels
+
+    T, H, V = 96, 128, 777
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=9)
+    # 3-D hidden / 2-D labels: outputs stay flattened, d_hidden is viewed back
+    h3 = h.view(2, 48, H).clone().requires_grad_(True)
+    w_ = w.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(h3, w_, y.view(2, 48), 1.5, "none")
+    assert lp.shape == (T,) and ent.shape == (T,)
+    # only log-probs used: entropy's gradient arrives as None and must behave as zero
+    lp.sum().backward()
+    torch.cuda.synchronize()
+    assert h3.grad.shape == (2, 48, H) and w_.grad.dtype == torch.bfloat16
+    rdh, rdw = O.lce_backward(torch.ones(T, device=DEV), None, h, w, y, 1.5)
+    torch.testing.assert_close(h3.grad.float().view(T, H), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(w_.grad.float(), rdw, atol=2e-2, rtol=4e-2)
+    # no_grad mode (log-prob passes): same values, no graph
+    with torch.no_grad():
+        lp2, ent2 = linear_cross_entropy(h, w, y, 1.5, "none")
+    assert not lp2.requires_grad
+    torch.testing.assert_close(lp2, lp.detach())
+    torch.testing.assert_close(ent2, ent.detach())
+    # non-contiguous upstream gradients are accepted
+    hh = h.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(hh, w, y, 1.5, "none")
+    g2 = torch.randn(T, 2, device=DEV)
+    torch.autograd.backward([lp, ent], [g2[:, 0], g2[:, 1]])
+    rdh, _ = O.lce_backward(g2[:, 0], g2[:, 1], h, w, y, 1.5)
+    torch.testing.assert_close(hh.grad.float(), rdh, atol=2e-2, rtol=4e-2)
+    # empty micro-batch
+    e_lp, e_ent = linear_cross_entropy(h[:0].clone().requires_grad_(True), w_, y[:0], 1.5, "none")
+    assert e_lp.shape == (0,) and e_ent.shape == (0,)
+    # unsupported pieces fail loudly
+    with pytest.raises(NotImplementedError):
+        linear_cross_entropy(h, w, y, 1.5, "none", object())
+    with pytest.raises(NotImplementedError):
+        linear_cross_entropy(h.half(), w.half(), y, 1.5, "none")
+    with pytest.raises(AssertionError):
+        linear_cross_entropy(h[:, :100].contiguous(), w[:, :100].contiguous(), y, 1.5, "none")  # H % 128
+    with pytest.raises(AssertionError):
+        linear_cross_entropy(h.t().contiguous().t(), w, y, 1.5, "none")  # non-contiguous hidden
+    # out-of-range labels are defined: no label logit, logprob = -logsumexp
+    y_bad = y.clone()
+    y_bad[0] = -100
+    lp_bad, _ = linear_cross_entropy(h, w, y_bad, 1.5, "none")
+    z0 = (h[0].float() @ w.float().t()) / 1.5
+    assert lp_bad[0].item() == pytest.approx(-torch.logsumexp(z0, -1).item(), abs=1e-3)
+    # saved statistics have the reference's meaning
+    lp_, ent_, mx, acc, eb = kernels.efficient_entropy_forward(h, w, y, 0, 1.5)
+    _, _, rmx, racc, reb = O.lce_forward(h, w, y, 1.5, return_stats=True)
+    torch.testing.assert_close(mx, rmx, atol=1e-4, rtol=1e-5)
+    torch.testing.assert_close(acc, racc, atol=1e-3, rtol=1e-4)
+    torch.testing.assert_close(eb, reb, atol=1e-4, rtol=1e-4)
+
+
+def _config_case(T, H, V, wstd, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    h = torch.randn(T, H, device=DEV, generator=g).bfloat16()
+    w = (torch.randn(V, H, device=DEV, generator=g) * wstd).bfloat16()
+    y = torch.randint(0, V, (T,), device=DEV, generator=g)
+    g_lp = torch.randn(T, device=DEV, generator=g)
+    g_ent = torch.randn(T, device=DEV, generator=g)
+    return h, w, y, g_lp, g_ent
+
+
+def test_config2_full_size_properties_and_sampled_parity():
+    """Qwen2.5-7B-shaped head at full size (T=16384, H=3584, V=152064).  The oracle is run on a
+    sample of rows for values and d_hidden, and on a slice of vocabulary rows for d_weight;
+    size-independent properties cover the rest: sum_v d_weight[v] = 0, log-probs <= 0,
+    0 <= entropy <= log V, linearity of the backward in the upstream gradients, determinism."""
+    from verl_amd import linear_cross_entropy
+
+    T, H, V, tau = 16384, 3584, 152064, 1.0
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.02, seed=1236)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    assert torch.isfinite(lp).all() and torch.isfinite(ent).all() and torch.isfinite(dh).all() and torch.isfinite(dw).all()
+    assert (lp <= 1e-6).all() and (ent >= -1e-4).all() and (ent <= math.log(V) + 1e-4).all()
+    rows = torch.arange(0, T, 61, device=DEV)
+    rlp, rent = O.lce_forward(h[rows], w, y[rows], tau)
+    assert (lp[rows] - rlp).abs().max() < 2e-2 and (ent[rows] - rent).abs().max() < 2e-2
+    torch.testing.assert_close(lp[rows], rlp, atol=1e-3, rtol=2e-4)
+    torch.testing.assert_close(ent[rows], rent, atol=5e-3, rtol=5e-4)
+    rdh, _ = O.lce_backward(g_lp[rows], g_ent[rows], h[rows], w, y[rows], tau)
+    assert (dh[rows].float() - rdh).abs().max() < 2e-2
+    # d_weight needs every token: check it through sum_v dz = 0  =>  sum_v d_weight[v, :] = 0
+    col = dw.float().sum(0)
+    scale = dw.float().abs().sum(0)
+    assert (col.abs() <= 2e-2 * scale + 1e-2).all()
+    # and exactly, on a vocabulary slice, against the closed form dz^T h restricted to that slice
+    vs = slice(70000, 70256)
+    _, _, mx, acc, eb = O.lce_forward(h, w, y, tau, return_stats=True, chunk=2048)
+    zs = (h.float() @ w[vs].float().t()) / tau
+    p = torch.exp(zs - (mx + acc.log()).unsqueeze(-1))
+    dz = -p * g_lp.unsqueeze(-1) - g_ent.unsqueeze(-1) * p * (zs - eb.unsqueeze(-1))
+    hit = (y >= vs.start) & (y < vs.stop)
+    dz[hit, y[hit] - vs.start] += g_lp[hit]
+    want = (dz / tau).t() @ h.float()
+    assert (dw[vs].float() - want).abs().max() < 2e-2
+    torch.testing.assert_close(dw[vs].float(), want, atol=2e-2, rtol=4e-2)
+    # determinism (no float atomics): bit-identical on a second run
+    lp2, ent2, dh2, dw2 = _run(h, w, y, tau, g_lp, g_ent)
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2) and torch.equal(dh, dh2) and torch.equal(dw, dw2)
+
+
+def test_config3_masked_rows_temperature_06():
+    """Llama-3-8B-shaped head, tau = 0.6, a response mask zeroing a random suffix of each row
+    (reduced token count; upstream gradients are zero on masked positions)."""
+    H, V, tau = 4096, 128256, 0.6
+    rows, L = 4, 512
+    T = rows * L
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.02, seed=1237)
+    g = torch.Generator().manual_seed(3)
+    valid = torch.randint(64, L + 1, (rows,), generator=g)
+    mask = (torch.arange(L)[None, :] < valid[:, None]).reshape(-1).to(DEV)
+    g_lp, g_ent = g_lp * mask, g_ent * mask
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2
+    assert (dh.float() - rdh).abs().max() < 2e-2 and (dw.float() - rdw).abs().max() < 2e-2
+    assert (dh[~mask] == 0).all()  # masked tokens receive exactly zero gradient
+
+
+def test_config4_weight_grad_accumulates_over_many_tokens():
+    """Qwen2.5-32B-shaped head (H=5120, V=152064, W ~ N(0, 0.015)); T reduced to 8192 so the oracle
+    finishes in seconds.  Exercises d_weight's sum over tokens and several vocabulary chunks."""
+    T, H, V, tau = 8192, 5120, 152064, 1.0
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.015, seed=1238)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2
+    assert (dh.float() - rdh).abs().max() < 2e-2 and (dw.float() - rdw).abs().max() < 2e-2
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
+@pytest.mark.parametrize("vchunk", [256, 1024, 8192])
+def test_vocab_chunking_is_transparent(vchunk):
+    from verl_amd.utils.kernel import kernels
+
+    T, H, V, tau = 513, 256, 5000, 1.5
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=11)
+    try:
+        kernels.set_vocab_chunk(vchunk)
+        _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    finally:
+        kernels.set_vocab_chunk(0)
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
+def test_every_tile_variant_agrees():
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V, tau = 700, 384, 3001, 1.5
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=13)
+    rlp, rent = O.lce_forward(h, w, y, tau)
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    try:
+        for v in range(lib.lce_num_variants()):
+            assert lib.lce_set_variant(v) == 0
+            lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+            torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+            torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+            torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+            torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    finally:
+        lib.lce_set_variant(3)
+
+
+def test_memory_gate_no_T_by_V_tensor():
+    """Zero [T, V] logits materialised: peak extra memory of forward and of backward stays below a
+    quarter of one bf16 [T, V] tile plus one fp32 [V, H] (the reference's test prints the same peaks,
+    tests/utils/test_linear_cross_entropy.py:323-349)."""
+    from verl_amd import linear_cross_entropy
+
+    T, H, V, tau = 8192, 2048, 152064, 1.0
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.02, seed=17)
+    h.requires_grad_(True)
+    w.requires_grad_(True)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    lp, ent = linear_cross_entropy(h, w, y, tau, "none")
+    torch.cuda.synchronize()
+    fwd_peak = torch.cuda.max_memory_allocated() - base
+    assert fwd_peak < 64 << 20, fwd_peak  # partial statistics only
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    torch.autograd.backward([lp, ent], [g_lp, g_ent])
+    torch.cuda.synchronize()
+    bwd_peak = torch.cuda.max_memory_allocated() - base
+    grads = (T * H + V * H) * 2
+    assert bwd_peak - grads < 0.25 * T * V * 2 + 4 * V * H, (bwd_peak, grads)

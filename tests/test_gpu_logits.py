@@ -1,0 +1,63 @@
+"""logprobs_from_logits / entropy_from_logits on materialised logits: HIP single-pass kernels
+against the oracle (verl/utils/torch_functional.py:73-107, :155-207, :231-270)."""
+
+import pytest
+import torch
+
+from oracle import lce_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 6, 50), (33, 152064), (2, 7, 4099), (1, 1)])
+def test_forward_and_backward(dtype, shape):
+    from verl_amd.utils import torch_functional as F
+
+    g = torch.Generator().manual_seed(shape[-1])
+    z = (torch.randn(*shape, generator=g) * 3).to(dtype).to(DEV)
+    y = torch.randint(0, shape[-1], shape[:-1], generator=g).to(DEV)
+    zz = z.clone().requires_grad_(True)
+    lp = F.logprobs_from_logits(zz, y)
+    ent = F.entropy_from_logits(zz)
+    assert lp.shape == shape[:-1] and ent.shape == shape[:-1] and lp.dtype == dtype and ent.dtype == dtype
+    rlp = O.logprobs_from_logits(z, y)
+    rent = O.entropy_from_logits(z)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(lp.float(), rlp, **tol)
+    torch.testing.assert_close(ent.float(), rent, **tol)
+    g_lp = torch.randn(shape[:-1], generator=g).to(DEV)
+    g_ent = torch.randn(shape[:-1], generator=g).to(DEV)
+    torch.autograd.backward([lp, ent], [g_lp.to(dtype), g_ent.to(dtype)])
+    want = O.logits_backward(z, y, g_lp.to(dtype).float(), g_ent.to(dtype).float())
+    assert zz.grad.dtype == dtype and zz.grad.shape == z.shape
+    torch.testing.assert_close(zz.grad.float(), want, **(dict(atol=1e-5, rtol=1e-4) if dtype == torch.float32 else tol))
+
+
+def test_extreme_logits_and_variants():
+    from verl_amd.utils import torch_functional as F
+
+    big = torch.tensor([[1000.0, -1000.0, 0.0], [-1e4, -1e4, -1e4]], device=DEV)
+    ent = F.entropy_from_logits(big)
+    lp = F.logprobs_from_logits(big, torch.tensor([0, 2], device=DEV))
+    assert torch.isfinite(ent).all() and torch.isfinite(lp).all()
+    assert lp[0].item() == pytest.approx(0.0, abs=1e-6) and ent[1].item() == pytest.approx(1.0986123, rel=1e-5)
+    z = torch.randn(5, 1000, device=DEV).bfloat16()
+    y = torch.randint(0, 1000, (5,), device=DEV)
+    a = F.logprobs_from_logits_v2(z, y)
+    b = F.logprobs_from_logits_naive(z, y)
+    assert torch.equal(a, b)
+    c = F.entropy_from_logits_with_chunking(z, chunk_size=2)
+    assert c.dtype == torch.float32
+    torch.testing.assert_close(c, O.entropy_from_logits(z), atol=1e-4, rtol=1e-4)
+    assert F.gather_from_labels(z, y).shape == (5,)
+
+
+def test_masked_reductions_known_answers():
+    from verl_amd.utils import torch_functional as F
+
+    v = torch.tensor([1.0, 2.0, 3.0, 4.0], device=DEV)
+    m = torch.tensor([0.0, 1.0, 1.0, 0.0], device=DEV)
+    assert F.masked_mean(v, m).item() == pytest.approx(2.5)
+    assert F.masked_mean(torch.tensor([float("nan"), 2.0, 3.0, float("nan")], device=DEV), m).item() == pytest.approx(2.5)

@@ -30,6 +30,10 @@ SYMBOLS = {
     "lce_gemm_nt": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _i, _p]),
     "lce_set_variant": (_i, [_i]),
     "lce_num_variants": (_i, []),
+    "lce_profile_enable": (_i, [_i]),
+    "lce_profile_num_classes": (_i, []),
+    "lce_profile_class_name": (_c.c_char_p, [_i]),
+    "lce_profile_read": (_i, [_p, _p, _i]),
 }
 
 _lib = None
@@ -90,3 +94,13 @@ def current_stream(device) -> int:
     import torch
 
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def profile_read(reset: bool = True) -> dict[str, tuple[float, int]]:
+    """{kernel class: (total ms, launches)} since profiling was enabled / last reset."""
+    lib = load()
+    n = lib.lce_profile_num_classes()
+    ms = (ctypes.c_double * n)()
+    cnt = (ctypes.c_int64 * n)()
+    check(lib.lce_profile_read(ctypes.addressof(ms), ctypes.addressof(cnt), 1 if reset else 0), "lce_profile_read")
+    return {lib.lce_profile_class_name(i).decode(): (ms[i], cnt[i]) for i in range(n) if cnt[i] > 0}

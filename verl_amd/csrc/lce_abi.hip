@@ -6,6 +6,9 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <vector>
+
 #include "lce_kernels.hpp"
 
 using namespace lce;
@@ -13,7 +16,7 @@ using namespace lce;
 namespace {
 
 thread_local char g_err[512] = "";
-int g_variant = 0;
+int g_variant = 3;
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -22,6 +25,30 @@ int fail(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
+
+// ---- optional per-kernel-class timing with HIP events (off by default; used by the benchmark) ----
+enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_COUNT };
+struct ProfRec { int cls; hipEvent_t a, b; };
+std::mutex g_prof_mu;
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof_recs;
+std::vector<hipEvent_t> g_prof_pool;
+
+hipEvent_t prof_event() {
+  if (!g_prof_pool.empty()) { hipEvent_t e = g_prof_pool.back(); g_prof_pool.pop_back(); return e; }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+struct ProfScope {
+  bool on; int cls; hipStream_t st; hipEvent_t a;
+  ProfScope(int c, hipStream_t s) : on(g_prof_on), cls(c), st(s), a(nullptr) {
+    if (on) { std::lock_guard<std::mutex> l(g_prof_mu); a = prof_event(); (void)hipEventRecord(a, st); }
+  }
+  ~ProfScope() {
+    if (on) { std::lock_guard<std::mutex> l(g_prof_mu); hipEvent_t b = prof_event(); (void)hipEventRecord(b, st); g_prof_recs.push_back({cls, a, b}); }
+  }
+};
 
 int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
@@ -59,7 +86,7 @@ int block_rows(int nrow_tiles) {
 template <typename Cfg>
 int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN* B, int64_t ldb, int64_t M, int64_t N,
                 int64_t K, float* Cf, int64_t ldcf, typename Cfg::TIN* Ct, int64_t ldct, int out_mode,
-                hipStream_t st) {
+                hipStream_t st, int prof_cls = PC_GEMM_DH) {
   typedef typename Cfg::TIN TIN;
   if (M <= 0 || N <= 0) return LCE_OK;
   if (K <= 0 || K % Cfg::BK != 0) return fail(LCE_E_ARG, "gemm: K=%lld must be a positive multiple of %d", (long long)K, Cfg::BK);
@@ -69,6 +96,7 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   allow_lds(gemm_nt_kernel<Cfg>, Cfg::LDS_BYTES);
+  ProfScope prof(prof_cls, st);
   hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
   return check_launch("gemm_nt_kernel");
 }
@@ -93,12 +121,19 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16));
   allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
-  hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
-  int rc = check_launch("lce_fwd_kernel");
+  int rc;
+  {
+    ProfScope prof(PC_FWD, st);
+    hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    rc = check_launch("lce_fwd_kernel");
+  }
   if (rc) return rc;
-  hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, S, T, p.c,
-                     1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
-  rc = check_launch("lce_fwd_merge_kernel");
+  {
+    ProfScope prof(PC_FWD_MERGE, st);
+    hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, S, T, p.c,
+                       1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
+    rc = check_launch("lce_fwd_merge_kernel");
+  }
   if (rc) return rc;
   if (reduction != LCE_REDUCTION_NONE) {
     const float scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
@@ -161,12 +196,15 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   float* dHacc = reinterpret_cast<float*>(ws + L.off_dHacc);
   int rc;
   // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
-  hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldWt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
-                     W, ldw, V, H, Wt, L.ldWt);
-  if ((rc = check_launch("transpose W"))) return rc;
-  hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldHt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
-                     h, ldh, T, H, Ht, L.ldHt);
-  if ((rc = check_launch("transpose h"))) return rc;
+  {
+    ProfScope prof(PC_TRANSPOSE, st);
+    hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldWt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
+                       W, ldw, V, H, Wt, L.ldWt);
+    if ((rc = check_launch("transpose W"))) return rc;
+    hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldHt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
+                       h, ldh, T, H, Ht, L.ldHt);
+    if ((rc = check_launch("transpose h"))) return rc;
+  }
 
   const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
   allow_lds(lce_bwd_ds_kernel<Cfg>, Cfg::LDS_BYTES);
@@ -183,16 +221,19 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     p.dS = dS; p.ldS = L.ldS; p.dST = dST; p.ldST = L.ldST;
     const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
     p.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
-    hipLaunchKernelGGL(lce_bwd_ds_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
-    if ((rc = check_launch("lce_bwd_ds_kernel"))) return rc;
+    {
+      ProfScope prof(PC_BWD_DS, st);
+      hipLaunchKernelGGL(lce_bwd_ds_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+      if ((rc = check_launch("lce_bwd_ds_kernel"))) return rc;
+    }
     // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
     const int64_t kc = round_up(vrows, 64);
     const bool first = c == 0, last = c == L.nchunks - 1;
     const int mode_h = (first ? 0 : 1) | (last ? 2 : 0);
-    rc = launch_gemm<Cfg>(dS, L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h, st);
+    rc = launch_gemm<Cfg>(dS, L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h, st, PC_GEMM_DH);
     if (rc) return rc;
     // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
-    rc = launch_gemm<Cfg>(dST, L.ldST, Ht, L.ldHt, vrows, H, L.ldST, nullptr, 0, d_weight + v0 * H, H, 2, st);
+    rc = launch_gemm<Cfg>(dST, L.ldST, Ht, L.ldHt, vrows, H, L.ldST, nullptr, 0, d_weight + v0 * H, H, 2, st, PC_GEMM_DW);
     if (rc) return rc;
   }
   return LCE_OK;
@@ -254,6 +295,34 @@ int lce_num_variants(void) { return kNumVariants; }
 int lce_set_variant(int variant) {
   if (variant < 0 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
   g_variant = variant;
+  return LCE_OK;
+}
+
+int lce_profile_enable(int on) {
+  std::lock_guard<std::mutex> l(g_prof_mu);
+  g_prof_on = on != 0;
+  return LCE_OK;
+}
+int lce_profile_num_classes(void) { return PC_COUNT; }
+const char* lce_profile_class_name(int cls) {
+  static const char* names[PC_COUNT] = {"lce_fwd_kernel", "lce_fwd_merge_kernel", "lce_bwd_ds_kernel", "gemm_nt_kernel(d_hidden)",
+                                        "gemm_nt_kernel(d_weight)", "transpose_pad_kernel", "logits_fwd_kernel", "logits_bwd_kernel"};
+  return (cls >= 0 && cls < PC_COUNT) ? names[cls] : "";
+}
+int lce_profile_read(double* total_ms, int64_t* launches, int reset) {
+  std::lock_guard<std::mutex> l(g_prof_mu);
+  for (int c = 0; c < PC_COUNT; ++c) { total_ms[c] = 0.0; launches[c] = 0; }
+  for (const ProfRec& r : g_prof_recs) {
+    if (hipEventSynchronize(r.b) != hipSuccess) return fail(LCE_E_LAUNCH, "profile: event synchronize failed");
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, r.a, r.b) != hipSuccess) return fail(LCE_E_LAUNCH, "profile: elapsed time failed");
+    total_ms[r.cls] += ms;
+    launches[r.cls] += 1;
+  }
+  if (reset) {
+    for (const ProfRec& r : g_prof_recs) { g_prof_pool.push_back(r.a); g_prof_pool.push_back(r.b); }
+    g_prof_recs.clear();
+  }
   return LCE_OK;
 }
 
@@ -354,6 +423,7 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   if (!logits || (logprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   constexpr int NT = 512;
+  ProfScope prof(PC_LOGITS_FWD, st);
   if (dtype == LCE_DTYPE_BF16)
     hipLaunchKernelGGL((logits_fwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, logprobs, entropy);
   else
@@ -369,6 +439,7 @@ int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, 
   if (!logits || !d_logits || (dlogprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   constexpr int NT = 512;
+  ProfScope prof(PC_LOGITS_BWD, st);
   if (dtype == LCE_DTYPE_BF16)
     hipLaunchKernelGGL((logits_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, dlogprobs, dentropy, (bf16_t*)d_logits, ldd);
   else
