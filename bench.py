@@ -79,6 +79,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -102,6 +104,14 @@ def main():
     y = torch.randint(0, V, (T,), device=dev, generator=g)
     g_lp = torch.randn(T, device=dev, generator=g)
     g_ent = torch.randn(T, device=dev, generator=g)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB per launch
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         h.grad = None

@@ -42,7 +42,10 @@ def test_extreme_logits_and_variants():
     ent = F.entropy_from_logits(big)
     lp = F.logprobs_from_logits(big, torch.tensor([0, 2], device=DEV))
     assert torch.isfinite(ent).all() and torch.isfinite(lp).all()
-    assert lp[0].item() == pytest.approx(0.0, abs=1e-6) and ent[1].item() == pytest.approx(1.0986123, rel=1e-5)
+    assert lp[0].item() == pytest.approx(0.0, abs=1e-6)
+    # logsumexp - sum p z cancels at |z| = 1e4: one fp32 ulp of 1e4 is 1e-3 (the torch formula has the same limit)
+    assert ent[1].item() == pytest.approx(1.0986123, abs=2e-3)
+    assert ent[1].item() == pytest.approx(O.entropy_from_logits(big)[1].item(), abs=2e-3)
     z = torch.randn(5, 1000, device=DEV).bfloat16()
     y = torch.randint(0, 1000, (5,), device=DEV)
     a = F.logprobs_from_logits_v2(z, y)
