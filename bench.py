@@ -79,6 +79,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
+    ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
+    ap.add_argument("--ds-dbg", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -94,6 +96,10 @@ def main():
     lib = _abi.load()
     if args.variant >= 0:
         _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
+    if args.split_backward:
+        _abi.check(lib.lce_set_option(1, 1), "lce_set_option")
+    if args.ds_dbg:
+        lib.lce_set_option(99, args.ds_dbg)
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
@@ -142,10 +148,20 @@ def main():
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
     # the dominant kernel (largest share of the step) and its algorithmic FLOPs per launch:
     # every MFMA kernel of the path does 2*T*V*H per step split over its launches
-    mfma = {k: v for k, v in kernels.items() if k.startswith(("lce_fwd_kernel", "lce_bwd_ds", "gemm_nt"))}
+    # algorithmic FLOPs per step of each MFMA kernel class (the recompute of the logits in the
+    # backward is executed but not counted): forward 2TVH; backward d_hidden + d_weight 4TVH
+    algo = {"lce_fwd_kernel": 2.0, "lce_bwd_chunk_kernel": 4.0}
+    if args.split_backward:
+        algo.update({"gemm_nt_kernel(d_hidden)": 2.0, "gemm_nt_kernel(d_weight)": 2.0})
+    executed = {"lce_fwd_kernel": 2.0, "lce_bwd_chunk_kernel": 6.0, "gemm_nt_kernel(d_hidden)": 2.0,
+                "gemm_nt_kernel(d_weight)": 2.0, "lce_bwd_ds_kernel": 2.0}
+    mfma = {k: v for k, v in kernels.items() if k in algo}
     dom = max(mfma, key=lambda k: mfma[k]["ms_per_step"])
-    flops_per_launch = 2.0 * T * V * H / mfma[dom]["launches_per_step"]
+    flops_per_launch = algo[dom] * T * V * H / mfma[dom]["launches_per_step"]
     achieved = flops_per_launch / (mfma[dom]["avg_ms"] * 1e-3)
+    for k, v in kernels.items():
+        if k in executed:
+            v["executed_tflops"] = executed[k] * T * V * H / (v["ms_per_step"] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
         "kernel": dom,

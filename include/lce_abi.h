@@ -85,6 +85,10 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 /* Tuning hook: selects the tile configuration used by the mainloops (0 = default).  Process-wide. */
 int lce_set_variant(int variant);
 int lce_num_variants(void);
+/* Diagnostic options (process-wide).  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and
+ * the two gradient GEMMs of a backward chunk as three kernels instead of one (for per-phase timing). */
+enum { LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1 };
+int lce_set_option(int key, int64_t value);
 
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every kernel
  * launch of the library is bracketed by HIP events on the caller's stream; lce_profile_read waits

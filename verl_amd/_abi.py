@@ -30,6 +30,7 @@ SYMBOLS = {
     "lce_gemm_nt": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _i, _p]),
     "lce_set_variant": (_i, [_i]),
     "lce_num_variants": (_i, []),
+    "lce_set_option": (_i, [_i, _i64]),
     "lce_profile_enable": (_i, [_i]),
     "lce_profile_num_classes": (_i, []),
     "lce_profile_class_name": (_c.c_char_p, [_i]),

@@ -17,6 +17,8 @@ namespace {
 
 thread_local char g_err[512] = "";
 int g_variant = 3;
+int g_split_bwd = 0;
+int g_ds_dbg = 0;  // diagnostic: launch the three sub-problems of a backward chunk separately
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -27,7 +29,7 @@ int fail(int code, const char* fmt, ...) {
 }
 
 // ---- optional per-kernel-class timing with HIP events (off by default; used by the benchmark) ----
-enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_COUNT };
+enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_BWD_CHUNK, PC_COUNT };
 struct ProfRec { int cls; hipEvent_t a, b; };
 std::mutex g_prof_mu;
 bool g_prof_on = false;
@@ -84,17 +86,25 @@ int block_rows(int nrow_tiles) {
 
 // ---------------------------------------------------------------------------------------------
 template <typename Cfg>
+GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN* B, int64_t ldb,
+                                           int64_t M, int64_t N, int64_t K, float* Cf, int64_t ldcf, typename Cfg::TIN* Ct,
+                                           int64_t ldct, int out_mode) {
+  GemmArgs<typename Cfg::TIN> p;
+  p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
+  p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
+  const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
+  p.map = TileMap::make(tm, tn, block_rows(tm), 1);
+  return p;
+}
+
+template <typename Cfg>
 int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN* B, int64_t ldb, int64_t M, int64_t N,
                 int64_t K, float* Cf, int64_t ldcf, typename Cfg::TIN* Ct, int64_t ldct, int out_mode,
                 hipStream_t st, int prof_cls = PC_GEMM_DH) {
   typedef typename Cfg::TIN TIN;
   if (M <= 0 || N <= 0) return LCE_OK;
   if (K <= 0 || K % Cfg::BK != 0) return fail(LCE_E_ARG, "gemm: K=%lld must be a positive multiple of %d", (long long)K, Cfg::BK);
-  GemmArgs<TIN> p;
-  p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
-  p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
-  const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
-  p.map = TileMap::make(tm, tn, block_rows(tm), 1);
+  const GemmArgs<TIN> p = make_gemm_args<Cfg>(A, lda, B, ldb, M, N, K, Cf, ldcf, Ct, ldct, out_mode);
   allow_lds(gemm_nt_kernel<Cfg>, Cfg::LDS_BYTES);
   ProfScope prof(prof_cls, st);
   hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
@@ -156,25 +166,37 @@ int forward_splits_upper_bound(int64_t T) {
 }
 
 struct BwdLayout {
-  int64_t vchunk, ldS, ldST, ldWt, ldHt;
-  size_t off_dS, off_dST, off_Wt, off_Ht, off_dHacc, total;
+  int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, total;
   int nchunks;
 };
 
-BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk) {
+BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   BwdLayout L;
   if (vchunk <= 0) vchunk = 8192;
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
   L.nchunks = (int)((V + vchunk - 1) / vchunk);
-  L.ldS = vchunk;
-  L.ldST = round_up(T, 64);
-  L.ldWt = round_up(V, 64);
-  L.ldHt = round_up(T, 64);
+  // Row strides are kept away from large powers of two (+128 bytes): with a 16 or 32 KiB stride the
+  // 256 rows of an operand tile would all fall into the same L2 channel.
+  // tokens / vocabulary rounded up to the K-permutation groups (gt, gv: at most one workgroup tile,
+  // which is what the size query assumes; the launch passes the tile variant's wave-tile sizes)
+  L.tpad = round_up(T, gt);
+  L.vpad = round_up(V, gv);
+  L.ldS = vchunk + 64;
+  L.ldST = L.tpad + 64;
+  L.ldWt = L.vpad + 64;
+  L.ldHt = L.tpad + 64;
   size_t o = 0;
-  L.off_dS = o;    o += align256((size_t)T * L.ldS * esz);
-  L.off_dST = o;   o += align256((size_t)vchunk * L.ldST * esz);
+  // the d_logits pair is double buffered when there is more than one chunk: chunk c is produced
+  // while the GEMMs of chunk c-1 consume the other pair
+  for (int b = 0; b < 2; ++b) {
+    L.off_dS[b] = o;
+    if (b == 0 || L.nchunks > 1) o += align256((size_t)T * L.ldS * esz);
+    L.off_dST[b] = o;
+    if (b == 0 || L.nchunks > 1) o += align256((size_t)vchunk * L.ldST * esz);
+  }
   L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
   L.off_Ht = o;    o += align256((size_t)H * L.ldHt * esz);
   L.off_dHacc = o; o += L.nchunks > 1 ? align256((size_t)T * H * 4) : 0;
@@ -188,9 +210,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                   const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                   typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st) {
   typedef typename Cfg::TIN TIN;
-  const BwdLayout L = bwd_layout(T, H, V, sizeof(TIN), vchunk);
-  TIN* dS = reinterpret_cast<TIN*>(ws + L.off_dS);
-  TIN* dST = reinterpret_cast<TIN*>(ws + L.off_dST);
+  const BwdLayout L = bwd_layout(T, H, V, sizeof(TIN), vchunk, KPerm<Cfg>::GT, KPerm<Cfg>::GV);
+  TIN* dS[2] = {reinterpret_cast<TIN*>(ws + L.off_dS[0]), reinterpret_cast<TIN*>(ws + L.off_dS[1])};
+  TIN* dST[2] = {reinterpret_cast<TIN*>(ws + L.off_dST[0]), reinterpret_cast<TIN*>(ws + L.off_dST[1])};
   TIN* Wt = reinterpret_cast<TIN*>(ws + L.off_Wt);
   TIN* Ht = reinterpret_cast<TIN*>(ws + L.off_Ht);
   float* dHacc = reinterpret_cast<float*>(ws + L.off_dHacc);
@@ -198,43 +220,67 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
   {
     ProfScope prof(PC_TRANSPOSE, st);
-    hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldWt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
-                       W, ldw, V, H, Wt, L.ldWt);
+    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)(L.vpad / 64), (unsigned)((H + 63) / 64)), dim3(256), 0,
+                       st, W, ldw, V, H, Wt, L.ldWt, L.vpad);
     if ((rc = check_launch("transpose W"))) return rc;
-    hipLaunchKernelGGL(transpose_pad_kernel<TIN>, dim3((unsigned)(L.ldHt / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st,
-                       h, ldh, T, H, Ht, L.ldHt);
+    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)(L.tpad / 64), (unsigned)((H + 63) / 64)), dim3(256), 0,
+                       st, h, ldh, T, H, Ht, L.ldHt, L.tpad);
     if ((rc = check_launch("transpose h"))) return rc;
   }
 
   const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
-  allow_lds(lce_bwd_ds_kernel<Cfg>, Cfg::LDS_BYTES);
-  for (int c = 0; c < L.nchunks; ++c) {
-    const int64_t v0 = (int64_t)c * L.vchunk;
-    const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
-    DsArgs<TIN> p;
-    p.W = W + v0 * ldw; p.ldw = ldw; p.h = h; p.ldh = ldh; p.labels = labels; p.T = T; p.H = H;
-    p.v0 = v0; p.vrows = vrows; p.rcp_tau = 1.0f / temperature; p.c = kLog2e / temperature;
-    p.maximum = maximum; p.accumulate = accumulate; p.entropy_b = entropy_b;
-    p.g_lp = dlogprobs; p.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
-    p.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
-    p.g_ent = dentropy;
-    p.dS = dS; p.ldS = L.ldS; p.dST = dST; p.ldST = L.ldST;
-    const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
-    p.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
-    {
-      ProfScope prof(PC_BWD_DS, st);
-      hipLaunchKernelGGL(lce_bwd_ds_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
-      if ((rc = check_launch("lce_bwd_ds_kernel"))) return rc;
+  allow_lds(lce_bwd_chunk_kernel<Cfg>, Cfg::LDS_BYTES);
+  // launch c (0 <= c <= nchunks): d_logits of chunk c (if any) + the two gradient GEMMs of chunk c-1 (if any)
+  for (int c = 0; c <= L.nchunks; ++c) {
+    BwdChunkArgs<TIN> p;
+    p.n_gw = p.n_gh = p.n_ds = 0;
+    if (c < L.nchunks) {
+      const int64_t v0 = (int64_t)c * L.vchunk;
+      const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
+      DsArgs<TIN>& d = p.ds;
+      d.W = W + v0 * ldw; d.ldw = ldw; d.h = h; d.ldh = ldh; d.labels = labels; d.T = T; d.H = H;
+      d.v0 = v0; d.vrows = vrows; d.rcp_tau = 1.0f / temperature; d.c = kLog2e / temperature;
+      d.maximum = maximum; d.accumulate = accumulate; d.entropy_b = entropy_b;
+      d.g_lp = dlogprobs; d.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
+      d.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
+      d.g_ent = dentropy;
+      d.dbg = g_ds_dbg;
+      d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
+      const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
+      d.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
+      p.n_ds = d.map.total;
     }
-    // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
-    const int64_t kc = round_up(vrows, 64);
-    const bool first = c == 0, last = c == L.nchunks - 1;
-    const int mode_h = (first ? 0 : 1) | (last ? 2 : 0);
-    rc = launch_gemm<Cfg>(dS, L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h, st, PC_GEMM_DH);
-    if (rc) return rc;
-    // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
-    rc = launch_gemm<Cfg>(dST, L.ldST, Ht, L.ldHt, vrows, H, L.ldST, nullptr, 0, d_weight + v0 * H, H, 2, st, PC_GEMM_DW);
-    if (rc) return rc;
+    if (c > 0) {
+      const int cc = c - 1;
+      const int64_t v0 = (int64_t)cc * L.vchunk;
+      const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
+      // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
+      const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
+      const bool first = cc == 0, last = cc == L.nchunks - 1;
+      const int mode_h = (first ? 0 : 1) | (last ? 2 : 0);
+      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h);
+      // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
+      p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
+      p.n_gh = p.gh.map.total;
+      p.n_gw = p.gw.map.total;
+    }
+    if (g_split_bwd) {
+      const int n[3] = {p.n_gw, p.n_gh, p.n_ds};
+      const int cls[3] = {PC_GEMM_DW, PC_GEMM_DH, PC_BWD_DS};
+      for (int k = 0; k < 3; ++k) {
+        if (n[k] == 0) continue;
+        BwdChunkArgs<TIN> q = p;
+        if (k == 1) q.gw = p.gh;  // sub-problem k is moved to the front slot of a single-problem launch
+        if (k == 2) { q.n_gw = 0; q.n_gh = 0; } else { q.n_gw = n[k]; q.n_gh = 0; q.n_ds = 0; }
+        ProfScope prof(cls[k], st);
+        hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, q);
+        if ((rc = check_launch("lce_bwd_chunk_kernel(split)"))) return rc;
+      }
+      continue;
+    }
+    ProfScope prof(PC_BWD_CHUNK, st);
+    hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
   return LCE_OK;
 }
@@ -297,6 +343,13 @@ int lce_set_variant(int variant) {
   g_variant = variant;
   return LCE_OK;
 }
+int lce_set_option(int key, int64_t value) {
+  switch (key) {
+    case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
+    case 99: g_ds_dbg = (int)value; return LCE_OK;
+    default: return fail(LCE_E_ARG, "unknown option %d", key);
+  }
+}
 
 int lce_profile_enable(int on) {
   std::lock_guard<std::mutex> l(g_prof_mu);
@@ -306,7 +359,8 @@ int lce_profile_enable(int on) {
 int lce_profile_num_classes(void) { return PC_COUNT; }
 const char* lce_profile_class_name(int cls) {
   static const char* names[PC_COUNT] = {"lce_fwd_kernel", "lce_fwd_merge_kernel", "lce_bwd_ds_kernel", "gemm_nt_kernel(d_hidden)",
-                                        "gemm_nt_kernel(d_weight)", "transpose_pad_kernel", "logits_fwd_kernel", "logits_bwd_kernel"};
+                                        "gemm_nt_kernel(d_weight)", "transpose_pad_kernel", "logits_fwd_kernel", "logits_bwd_kernel",
+                                        "lce_bwd_chunk_kernel"};
   return (cls >= 0 && cls < PC_COUNT) ? names[cls] : "";
 }
 int lce_profile_read(double* total_ms, int64_t* launches, int reset) {

@@ -234,29 +234,162 @@ struct DsArgs {
   int64_t ldS;
   TIN* dST;             // [vchunk][ldST] (vocab-major)
   int64_t ldST;
+  int dbg;              // diagnostic bit mask: 1 skip dS stores, 2 skip dS^T stores, 4 skip the epilogue
+  int64_t tpad;         // tokens rounded up to the GEMM K granule: columns [T, tpad) of dST are written as zeros
   TileMap map;          // rows = token tiles, cols = vocab tiles of the chunk
 };
 
-template <typename T>
-LCE_DEV void store4(T* dst, float a, float b, float c, float d);
-template <>
-LCE_DEV void store4<float>(float* dst, float a, float b, float c, float d) {
-  f32x4_t v = {a, b, c, d};
-  *reinterpret_cast<f32x4_t*>(dst) = v;
+// The two gradient GEMMs sum over the vocabulary (d_hidden) and over the tokens (d_weight); any
+// permutation of the summation index is allowed as long as both operands of a GEMM use the same one.
+// The intermediates (dS, dS^T, W^T, h^T) are private to the backward, so their K order is chosen to
+// suit the producer: inside each group of WN tokens / WM vocabulary rows (one wave tile) the index is
+// re-ordered so that everything ONE lane of the d_logits epilogue holds is contiguous, and the
+// epilogue stores 16-byte / 8-byte vectors instead of single elements.
+template <typename Cfg>
+struct KPerm {
+  static constexpr int GT = Cfg::WN, GV = Cfg::WM;
+  // token t (lane ln = t % 32 of block column j = (t % GT) / 32)  ->  ln * FN + j
+  static __host__ __device__ int64_t token(int64_t t) {
+    const int64_t l = t % GT;
+    return t - l + (l % 32) * Cfg::FN + l / 32;
+  }
+  // vocabulary row v = i*32 + 8*(r/4) + 4*hh + r%4 of its group  ->  hh * 16*FM + i*16 + r
+  static __host__ __device__ int64_t vocab(int64_t v) {
+    const int64_t l = v % GV;
+    const int64_t i = l / 32, w = l % 32, hh = (w >> 2) & 1, r = (w >> 3) * 4 + (w & 3);
+    return v - l + hh * 16 * Cfg::FM + i * 16 + r;
+  }
+};
+
+template <typename T, int N>
+struct VecOf;
+template <int N>
+struct VecOf<float, N> { typedef float type __attribute__((ext_vector_type(N))); };
+template <int N>
+struct VecOf<bf16_t, N> { typedef bf16_t type __attribute__((ext_vector_type(N))); };
+
+// store N consecutive elements (N * sizeof(T) <= 16 bytes per store; wider runs are split)
+template <typename T, int N>
+LCE_DEV void store_run(T* dst, const float (&v)[N]) {
+  constexpr int PER = (16 / (int)sizeof(T)) < N ? (16 / (int)sizeof(T)) : N;
+  typedef typename VecOf<T, PER>::type vec_t;
+#pragma unroll
+  for (int k = 0; k < N; k += PER) {
+    vec_t out;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) out[e] = (T)v[k + e];
+    *reinterpret_cast<vec_t*>(dst + k) = out;
+  }
 }
-template <>
-LCE_DEV void store4<bf16_t>(bf16_t* dst, float a, float b, float c, float d) {
-  typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
-  bf16x4_t v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
-  *reinterpret_cast<bf16x4_t*>(dst) = v;
+
+// d_logits of one accumulator element; SLOW adds the label one-hot and masks padded rows / tokens
+template <bool SLOW>
+LCE_DEV float dlogit(float x, float c, float lse2, float C0, float C1, float G, bool hit, bool dead) {
+  const float pr = fast_exp2(__builtin_fmaf(x, c, -lse2));
+  float dv = pr * __builtin_fmaf(x, C1, C0);
+  if (SLOW) {
+    if (hit) dv += G;
+    if (dead) dv = 0.f;
+  }
+  return dv;
+}
+
+// dS (token-major) leaves the wave through a wave-private LDS staging tile so that every store
+// instruction writes whole 128-byte lines (8 lanes x 16 bytes per token row); written straight from
+// the accumulator layout each lane would hit a different row, which costs ~25% of the kernel.
+// 16-byte chunks of a staged row are XOR-swizzled with the row number (conflict-free both ways).
+template <typename Cfg>
+struct DsStage {
+  typedef typename Cfg::TIN TIN;
+  static constexpr bool kEnabled = sizeof(TIN) == 2;                 // fp32 tiles do not fit; they store directly
+  static constexpr int ROW_BYTES = Cfg::WM * (int)sizeof(TIN);       // one token's slice of the wave tile
+  static constexpr int CPR = ROW_BYTES / 16;                          // 16-byte chunks per row
+  static constexpr int WAVE_BYTES = Cfg::WN * ROW_BYTES;
+  static_assert(!kEnabled || WAVE_BYTES * Cfg::NW <= Cfg::LDS_BYTES, "staging tile must fit the mainloop's LDS");
+  static LCE_DEV int swz(int row) { return (row ^ ((row >> 3) & 1)) & 7; }
+};
+
+template <typename Cfg, bool SLOW>
+LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t tok0,
+                         int vloc0, int hh, int ln, char* stage_lds) {
+  typedef typename Cfg::TIN TIN;
+  typedef DsStage<Cfg> Stg;
+  constexpr int FM = Cfg::FM, FN = Cfg::FN;
+  float lse2[FN], C0[FN], C1[FN], G[FN];
+  int rel[FN];
+  bool tok_ok[FN];
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+    const int64_t tok = tok0 + j * 32 + ln;
+    tok_ok[j] = tok < p.T;
+    lse2[j] = C0[j] = C1[j] = G[j] = 0.f;
+    rel[j] = -1;
+    if (tok_ok[j]) {
+      const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
+      const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
+      lse2[j] = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
+      G[j] = glp * p.rcp_tau;
+      C1[j] = -gent * p.rcp_tau * p.rcp_tau;
+      C0[j] = -G[j] + gent * p.entropy_b[tok] * p.rcp_tau;
+      const int64_t y = p.labels[tok] - p.v0;
+      rel[j] = (y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
+    }
+  }
+  const bool tok_group_live = tok0 < p.tpad;                 // the whole token group is inside dS^T's columns
+  TIN* dst_t = p.dST + (tok0 + (int64_t)ln * FN);            // + vocab row * ldST   (token order: ln*FN + j)
+  TIN* dst_s = p.dS + (vloc0 + hh * 16 * FM);                // + token * ldS + i*16 + r (vocab order: hh, i, r)
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      __builtin_amdgcn_sched_barrier(0);  // bound the live range of the staged values
+      float stage[FN][8];
+#pragma unroll
+      for (int rr = 0; rr < 8; ++rr) {
+        const int r = half * 8 + rr;
+        const int row = acc_row(i, r, hh);  // wave-tile-local vocabulary row
+        float d[FN];
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          d[j] = dlogit<SLOW>(acc[i][j][r], p.c, lse2[j], C0[j], C1[j], G[j], row == rel[j],
+                              !tok_ok[j] || vloc0 + row >= p.vrows);
+          stage[j][rr] = d[j];
+        }
+        if (tok_group_live && !(p.dbg & 2)) store_run<TIN, FN>(dst_t + (int64_t)(vloc0 + row) * p.ldST, d);
+      }
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        if constexpr (Stg::kEnabled) {
+          // logical 16-byte chunk of this run inside the token's row: (hh*16*FM + i*16 + half*8) elements
+          const int c = hh * 2 * FM + i * 2 + half, row = j * 32 + ln;
+          store_run<TIN, 8>(reinterpret_cast<TIN*>(stage_lds + row * Stg::ROW_BYTES + ((c ^ Stg::swz(row)) * 16)), stage[j]);
+        } else {
+          if (tok_ok[j] && !(p.dbg & 1))
+            store_run<TIN, 8>(dst_s + (tok0 + j * 32 + ln) * p.ldS + i * 16 + half * 8, stage[j]);
+        }
+      }
+    }
+  }
+  if constexpr (Stg::kEnabled) {
+    // the staging tile is private to this wave: LDS operations of one wave complete in order
+    const int lane = hh * 32 + ln;
+    if (!(p.dbg & 1)) {
+#pragma unroll
+      for (int it = 0; it < Stg::WAVE_BYTES / 1024; ++it) {
+        const int q = it * 64 + lane, row = q / Stg::CPR, pc = q % Stg::CPR;
+        const int c = pc ^ Stg::swz(row);
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage_lds + row * Stg::ROW_BYTES + pc * 16);
+        const int64_t tok = tok0 + row;
+        if (tok < p.T) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
+      }
+    }
+  }
 }
 
 template <typename Cfg>
-__global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_ds_kernel(DsArgs<typename Cfg::TIN> p) {
-  typedef typename Cfg::TIN TIN;
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
+LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   int tt, vt;
-  if (!p.map.decode(blockIdx.x, tt, vt)) return;
+  if (!p.map.decode(bid, tt, vt)) return;
   const int64_t n0 = (int64_t)tt * Cfg::BN, m0 = (int64_t)vt * Cfg::BM;
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
@@ -264,48 +397,27 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_ds_kernel(DsArgs<typena
   f32x16_t acc[Cfg::FM][Cfg::FN];
   g.run(lds, p.H, acc);
 
-  const int vloc0 = (int)m0 + g.wave_m * Cfg::WM;  // chunk-local vocabulary index of this wave's first row
+  const int vloc0 = (int)m0 + g.wave_m * Cfg::WM;      // chunk-local vocabulary index of this wave's first row
+  const int64_t tok0 = n0 + g.wave_n * Cfg::WN;         // first token of this wave's group
+  // fast path: the wave tile is interior (no padded rows or tokens) and holds no label
+  bool has_label = false;
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
-    const int64_t tok = n0 + g.wave_n * Cfg::WN + j * 32 + ln;
-    const bool tok_ok = tok < p.T;
-    float lse2 = 0.f, C0 = 0.f, C1 = 0.f, G = 0.f;
-    int rel = -1;
-    if (tok_ok) {
-      const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
-      const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
-      lse2 = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
-      G = glp * p.rcp_tau;
-      C1 = -gent * p.rcp_tau * p.rcp_tau;
-      C0 = -G + gent * p.entropy_b[tok] * p.rcp_tau;
+    const int64_t tok = tok0 + j * 32 + ln;
+    if (tok < p.T) {
       const int64_t y = p.labels[tok] - p.v0;
-      rel = (y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
+      has_label |= (y >= vloc0 && y < vloc0 + Cfg::WM);
     }
-#pragma unroll
-    for (int i = 0; i < Cfg::FM; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        __builtin_amdgcn_sched_barrier(0);
-        float d[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int r = q * 4 + u;
-          const float x = acc[i][j][r];
-          const float pr = fast_exp2(__builtin_fmaf(x, p.c, -lse2));
-          float dv = pr * __builtin_fmaf(x, C1, C0);
-          const int row = acc_row(i, r, hh);
-          if (row == rel) dv += G;
-          if (!tok_ok || vloc0 + row >= p.vrows) dv = 0.f;
-          d[u] = dv;
-        }
-        const int vrow = vloc0 + i * 32 + 8 * q + 4 * hh;  // chunk-local vocab index of d[0]
-        if (tok_ok && vrow < p.ldS) store4<TIN>(p.dS + tok * p.ldS + vrow, d[0], d[1], d[2], d[3]);
-        if (tok < p.ldST) {
-#pragma unroll
-          for (int u = 0; u < 4; ++u) p.dST[(int64_t)(vrow + u) * p.ldST + tok] = (TIN)d[u];
-        }
-      }
   }
+  const bool interior = vloc0 + Cfg::WM <= p.vrows && tok0 + Cfg::WN <= p.T;
+  if (p.dbg & 4) {
+    if (acc[0][0][0] == 123.456f) p.dS[0] = (typename Cfg::TIN)1.f;
+    return;
+  }
+  __syncthreads();  // every wave's slab loads have landed and its operand reads are done: LDS is free
+  char* stage_lds = lds + g.wave * DsStage<Cfg>::WAVE_BYTES;
+  if (interior && __builtin_amdgcn_ballot_w64(has_label) == 0) ds_epilogue<Cfg, false>(p, acc, tok0, vloc0, hh, ln, stage_lds);
+  else ds_epilogue<Cfg, true>(p, acc, tok0, vloc0, hh, ln, stage_lds);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -358,10 +470,9 @@ LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t 
 }
 
 template <typename Cfg>
-__global__ __launch_bounds__(Cfg::NTHREADS) void gemm_nt_kernel(GemmArgs<typename Cfg::TIN> p) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
+LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   int tm, tn;
-  if (!p.map.decode(blockIdx.x, tm, tn)) return;
+  if (!p.map.decode(bid, tm, tn)) return;
   const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
@@ -381,14 +492,50 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_nt_kernel(GemmArgs<typenam
 #undef LCE_EPI
 }
 
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_ds_kernel(DsArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  ds_tile<Cfg>(p, blockIdx.x, lds);
+}
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void gemm_nt_kernel(GemmArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  gemm_tile<Cfg>(p, blockIdx.x, lds);
+}
+
+// One launch of the backward's steady state: the two gradient GEMMs of vocabulary chunk c-1 and the
+// d_logits tiles of chunk c (which go to the other buffer pair) share a grid, longest tiles first,
+// so the tail of one sub-problem is filled by the next instead of idling the CUs.
+// Sub-grid sizes are multiples of 32, which keeps (block id % 8) -> XCD intact for every sub-problem.
+template <typename TIN>
+struct BwdChunkArgs {
+  GemmArgs<TIN> gw;  // d_weight[chunk c-1] = dS^T . h^T      (K = T: longest tiles)
+  GemmArgs<TIN> gh;  // d_hidden (+)= dS . W^T[chunk c-1]      (K = chunk width)
+  DsArgs<TIN> ds;    // d_logits of chunk c                     (K = H, heavy epilogue)
+  int n_gw, n_gh, n_ds;
+};
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_chunk_kernel(BwdChunkArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int bid = blockIdx.x;
+  if (bid < p.n_gw) gemm_tile<Cfg>(p.gw, bid, lds);
+  else if (bid < p.n_gw + p.n_gh) gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds);
+  else ds_tile<Cfg>(p.ds, bid - p.n_gw - p.n_gh, lds);
+}
+
 __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
-// out[c][r] = in[r][c] for r < R, c < C; out has `ldo` columns and columns [R, ldo) are zero-filled.
-// Grid: (ceil(ldo/64), ceil(C/64)), 256 threads.
-template <typename TIN>
-__global__ void transpose_pad_kernel(const TIN* in, int64_t ldi, int64_t R, int64_t C, TIN* out, int64_t ldo) {
+// out[c][perm(r)] = in[r][c] for r < R, c < C; out has `ldo` columns, columns perm(r) with r in
+// [R, rpad) are zero-filled (rpad a multiple of the permutation's group).  PERM: 0 none,
+// 1 KPerm::token, 2 KPerm::vocab.  Grid: (rpad/64, ceil(C/64)), 256 threads.
+template <typename Cfg, int PERM>
+__global__ void transpose_pad_kernel(const typename Cfg::TIN* in, int64_t ldi, int64_t R, int64_t C, typename Cfg::TIN* out,
+                                     int64_t ldo, int64_t rpad) {
+  typedef typename Cfg::TIN TIN;
   __shared__ TIN tile[64][65];
   const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -399,7 +546,10 @@ __global__ void transpose_pad_kernel(const TIN* in, int64_t ldi, int64_t R, int6
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     const int64_t c = c0 + i, r = r0 + tx;
-    if (c < C && r < ldo) out[c * ldo + r] = tile[tx][i];
+    if (c < C && r < rpad) {
+      const int64_t pr = PERM == 1 ? KPerm<Cfg>::token(r) : (PERM == 2 ? KPerm<Cfg>::vocab(r) : r);
+      out[c * ldo + pr] = tile[tx][i];
+    }
   }
 }
 
