@@ -19,6 +19,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
+# HBM-side bytes per launch (fetch + write) of the MFMA kernels on the default workload, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run
+# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt); counters cannot be read from inside this process.
+MEASURED_TRAFFIC = {
+    "qwen2.5-7b-head-T16384": {
+        "lce_bwd_chunk_kernel": 3962132 * 1024 * 2.0 + 1115442 * 1024 * 1.0,
+        "lce_fwd_kernel": 13898456 * 1024 * 2.0 + 460800 * 1024 * 1.0,
+    }
+}
 WORKLOADS = {
     # name: (T, H, V, temperature, weight std)
     "qwen2.5-7b-head-T16384": (16384, 3584, 152064, 1.0, 0.02),
@@ -80,7 +89,6 @@ def main():
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
     ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
-    ap.add_argument("--ds-dbg", type=int, default=0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -98,8 +106,6 @@ def main():
         _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
     if args.split_backward:
         _abi.check(lib.lce_set_option(1, 1), "lce_set_option")
-    if args.ds_dbg:
-        lib.lce_set_option(99, args.ds_dbg)
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
@@ -169,7 +175,7 @@ def main():
         "peak": PEAK_BF16 / 1e12,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(dom),
         "avg_launch_ms": mfma[dom]["avg_ms"],
         "flops_per_launch": flops_per_launch,
     }

@@ -139,6 +139,9 @@ struct GemmCore {
 
   // one of the PER wave-wide 16-byte-per-lane global->LDS loads of a slab (A loads first)
   LCE_DEV void dma_one(char* lds, int stage, int64_t kbyte, int idx) const {
+#ifdef LCE_DBG_NO_DMA
+    if (kbyte > 0) return;
+#endif
     char* sa = lds + stage * Cfg::STAGE_BYTES;
     if (idx < Cfg::A_LOADS) {
       __builtin_amdgcn_global_load_lds((gptr_t)(a_base + kbyte + la.voff[idx]),
@@ -156,6 +159,9 @@ struct GemmCore {
 
   // one of the N_READS operand reads of k-substep kk, in the order a0, b0..b(FN-1), a1..a(FM-1)
   LCE_DEV void read_one(const char* s, int kk, int idx, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
+#ifdef LCE_DBG_NO_READS
+    if (kk > 0) return;
+#endif
     const uint32_t ao = a_rd ^ (uint32_t)(kk * 32);
     const uint32_t bo = b_rd ^ (uint32_t)(kk * 32);
     if (idx == 0) af[0] = *reinterpret_cast<const u32x4_t*>(s + ao);
@@ -198,7 +204,26 @@ struct GemmCore {
   // and the workgroup barrier that hands a ring stage back to the loader sits before the LAST
   // substep of a slab, so the matrix pipe keeps working across the barrier.  The loop body is
   // branch-free: past the end of K the loader re-fetches the last slab into a stage nobody reads.
+  // Issues the loads of the first NSTAGE slabs.  LDS must be free (every wave past its last read and
+  // its loads drained: a workgroup barrier after the previous main()).
+  LCE_DEV void prologue(char* lds, int64_t K) const {
+    const int nk = (int)(K / Cfg::BK);
+    const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
+#pragma unroll
+    for (int s = 0; s < Cfg::NSTAGE; ++s) {
+      const int64_t kb = (int64_t)s * Cfg::BKB;
+      issue_slab(lds, s, kb < last_kbyte ? kb : last_kbyte);
+    }
+  }
+
   LCE_DEV void run(char* lds, int64_t K, f32x16_t (&acc)[Cfg::FM][Cfg::FN]) const {
+    prologue(lds, K);
+    main(lds, K, acc);
+  }
+
+  // The K loop proper; prologue() must have been called for this tile (no other vector memory
+  // loads may have been issued by this wave in between: the waits count outstanding loads).
+  LCE_DEV void main(char* lds, int64_t K, f32x16_t (&acc)[Cfg::FM][Cfg::FN]) const {
     constexpr int NS = Cfg::NSTAGE, KSUB = Cfg::KSUB;
     const int nk = (int)(K / Cfg::BK);
     const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
@@ -208,11 +233,6 @@ struct GemmCore {
       for (int j = 0; j < Cfg::FN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const int64_t kb = (int64_t)s * Cfg::BKB;
-      issue_slab(lds, s, kb < last_kbyte ? kb : last_kbyte);
-    }
     wait_vm<(NS - 1) * PER>();
     __builtin_amdgcn_s_barrier();
     u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];

@@ -18,7 +18,7 @@ namespace {
 thread_local char g_err[512] = "";
 int g_variant = 3;
 int g_split_bwd = 0;
-int g_ds_dbg = 0;  // diagnostic: launch the three sub-problems of a backward chunk separately
+  // diagnostic: launch the three sub-problems of a backward chunk separately
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -127,11 +127,14 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.W = W; p.ldw = ldw; p.h = h; p.ldh = ldh; p.labels = labels; p.T = T; p.V = V; p.H = H;
   p.c = kLog2e / temperature;
   p.parts = reinterpret_cast<f32x4_t*>(ws);
+  p.xlabel = reinterpret_cast<float*>(ws + align256((size_t)S * T * 16));
   p.S = S; p.nvt = nvt;
   p.map = TileMap::make(ntt, S, br, 1);
-  float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16));
+  float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
   allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
   int rc;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((T + 1023) / 1024)), dim3(256), 0, st, reinterpret_cast<uint32_t*>(p.xlabel), T);
+  if ((rc = check_launch("fill_zero_kernel"))) return rc;
   {
     ProfScope prof(PC_FWD, st);
     hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
@@ -140,7 +143,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   if (rc) return rc;
   {
     ProfScope prof(PC_FWD_MERGE, st);
-    hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, S, T, p.c,
+    hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T, p.c,
                        1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
     rc = check_launch("lce_fwd_merge_kernel");
   }
@@ -173,7 +176,14 @@ struct BwdLayout {
 
 BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   BwdLayout L;
-  if (vchunk <= 0) vchunk = 8192;
+  if (vchunk <= 0) {
+    // default: as wide as possible (fewer, longer launches) while the whole workspace stays below a
+    // quarter of one [T, V] tile plus one fp32 [V, H]:  8*T*vc*esz/2 + esz*V*H + (esz+4)*T*H  <=  0.25*T*V*esz + 4*V*H
+    const double tv = 0.25 * (double)T * V * esz, vh = (4.0 - esz) * (double)V * H, th = (esz + 4.0) * (double)T * H;
+    const double bound = (tv + vh - th) / (4.0 * esz * (double)T);
+    vchunk = bound > 16384.0 ? 16384 : (int64_t)(bound / 1024.0) * 1024;
+    if (vchunk < 2048) vchunk = 2048;
+  }
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
@@ -244,7 +254,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_lp = dlogprobs; d.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
       d.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
       d.g_ent = dentropy;
-      d.dbg = g_ds_dbg;
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       d.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
@@ -346,7 +355,6 @@ int lce_set_variant(int variant) {
 int lce_set_option(int key, int64_t value) {
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
-    case 99: g_ds_dbg = (int)value; return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
 }
@@ -383,7 +391,7 @@ int lce_profile_read(double* total_ms, int64_t* launches, int reset) {
 size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
   (void)H; (void)V; (void)dtype;
   if (T <= 0) return 256;
-  return align256((size_t)forward_splits_upper_bound(T) * (size_t)T * 16) + align256((size_t)T * 4);
+  return align256((size_t)forward_splits_upper_bound(T) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
 }
 
 int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,

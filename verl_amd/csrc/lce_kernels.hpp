@@ -41,7 +41,8 @@ struct FwdArgs {
   const int64_t* labels;
   int64_t T, V, H;
   float c;           // log2(e) / temperature
-  f32x4_t* parts;    // [S][T] of (m, a, b, x_label)
+  f32x4_t* parts;    // [S][T] of (m, a, b, unused)
+  float* xlabel;     // [T] raw accumulator value at the label (pre-zeroed; written by the one lane that owns it)
   int S;             // vocabulary splits; split s owns vocab tiles s, s+S, s+2S, ...
   int nvt;           // vocabulary tiles
   TileMap map;       // rows = token tiles, cols = splits
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
 
-  float m[Cfg::FN], a[Cfg::FN], b[Cfg::FN], zy[Cfg::FN];
+  float m[Cfg::FN], a[Cfg::FN], b[Cfg::FN];
   int lab[Cfg::FN];
   {
     const int wave = threadIdx.x >> 6;
@@ -66,7 +67,6 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       m[j] = kNegBig;
       a[j] = 0.f;
       b[j] = 0.f;
-      zy[j] = 0.f;
       const int64_t t = n0 + wave_n * Cfg::WN + j * 32 + ln;
       const int64_t y = t < p.T ? p.labels[t] : -1;
       lab[j] = (y >= 0 && y < p.V) ? (int)y : -1;
@@ -74,12 +74,20 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
   }
 
   f32x16_t acc[Cfg::FM][Cfg::FN];
+  g.init(p.W, p.ldw, (int64_t)s * Cfg::BM, p.V, p.h, p.ldh, n0, p.T);
+  g.prologue(lds, p.H);
   for (int vt = s; vt < p.nvt; vt += p.S) {
     const int64_t m0 = (int64_t)vt * Cfg::BM;
-    g.init(p.W, p.ldw, m0, p.V, p.h, p.ldh, n0, p.T);
-    g.run(lds, p.H, acc);
+    g.main(lds, p.H, acc);
     const int vbase = (int)m0 + g.wave_m * Cfg::WM;  // vocabulary index of this wave's first row
     const bool full = m0 + Cfg::BM <= p.V;
+    // start fetching the next tile's first slabs now: the loads fly while this tile's statistics are
+    // folded in (the epilogue touches neither LDS nor vector memory on its common path)
+    __syncthreads();  // every wave is past its last LDS read and has drained its own loads
+    if (vt + p.S < p.nvt) {
+      g.init(p.W, p.ldw, (int64_t)(vt + p.S) * Cfg::BM, p.V, p.h, p.ldh, n0, p.T);
+      g.prologue(lds, p.H);
+    }
     if (!full) {
 #pragma unroll
       for (int i = 0; i < Cfg::FM; ++i)
@@ -137,52 +145,51 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (mine && acc_row(i, r, hh) == rel) pick = acc[i][j][r];
-        zy[j] += pick;
+        // exactly one lane in the whole grid owns a token's label: plain store, no merge needed
+        if (mine) p.xlabel[n0 + g.wave_n * Cfg::WN + j * 32 + ln] = pick;
       }
     }
-    __syncthreads();  // every wave is done with LDS before the next tile's loads overwrite it
   }
+  __syncthreads();
 
   // merge the two lane halves (same token, different vocabulary rows), then the WAVES_M waves
   f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);  // [WAVES_M][BN]
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
     const float m2 = __shfl_xor(m[j], 32), a2 = __shfl_xor(a[j], 32), b2 = __shfl_xor(b[j], 32);
-    const float z2 = __shfl_xor(zy[j], 32);
     merge_stats(m[j], a[j], b[j], m2, a2, b2, p.c);
-    zy[j] += z2;
     if (hh == 0) {
-      f32x4_t v = {m[j], a[j], b[j], zy[j]};
+      f32x4_t v = {m[j], a[j], b[j], 0.f};
       red[g.wave_m * Cfg::BN + g.wave_n * Cfg::WN + j * 32 + ln] = v;
     }
   }
   __syncthreads();
   for (int t = threadIdx.x; t < Cfg::BN; t += Cfg::NTHREADS) {
     const f32x4_t v0 = red[t];
-    float vm = v0[0], va = v0[1], vb = v0[2], vz = v0[3];
+    float vm = v0[0], va = v0[1], vb = v0[2];
 #pragma unroll
     for (int w = 1; w < Cfg::WAVES_M; ++w) {
       const f32x4_t u = red[w * Cfg::BN + t];
       merge_stats(vm, va, vb, u[0], u[1], u[2], p.c);
-      vz += u[3];
     }
     const int64_t tok = n0 + t;
-    const f32x4_t v = {vm, va, vb, vz};
+    const f32x4_t v = {vm, va, vb, 0.f};
     if (tok < p.T) p.parts[(int64_t)s * p.T + tok] = v;
   }
 }
 
 // merge the S partials of every token and emit the five per-token outputs
-__global__ void lce_fwd_merge_kernel(const f32x4_t* parts, int S, int64_t T, float c, float rcp_tau, float* logprobs,
-                                     float* entropy, float* maximum, float* accumulate, float* entropy_b) {
+__global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, int S, int64_t T, float c, float rcp_tau,
+                                     float* logprobs, float* entropy, float* maximum, float* accumulate,
+                                     float* entropy_b) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const f32x4_t v0 = parts[t];
-  float vm = v0[0], va = v0[1], vb = v0[2], vz = v0[3];
+  float vm = v0[0], va = v0[1], vb = v0[2];
+  const float vz = xlabel[t];
   for (int s = 1; s < S; ++s) {
     const f32x4_t u = parts[(int64_t)s * T + t];
     merge_stats(vm, va, vb, u[0], u[1], u[2], c);
-    vz += u[3];
   }
   const float mz = vm * rcp_tau;
   const float lse = mz + logf(va);
@@ -234,7 +241,6 @@ struct DsArgs {
   int64_t ldS;
   TIN* dST;             // [vchunk][ldST] (vocab-major)
   int64_t ldST;
-  int dbg;              // diagnostic bit mask: 1 skip dS stores, 2 skip dS^T stores, 4 skip the epilogue
   int64_t tpad;         // tokens rounded up to the GEMM K granule: columns [T, tpad) of dST are written as zeros
   TileMap map;          // rows = token tiles, cols = vocab tiles of the chunk
 };
@@ -355,7 +361,7 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
                               !tok_ok[j] || vloc0 + row >= p.vrows);
           stage[j][rr] = d[j];
         }
-        if (tok_group_live && !(p.dbg & 2)) store_run<TIN, FN>(dst_t + (int64_t)(vloc0 + row) * p.ldST, d);
+        if (tok_group_live) store_run<TIN, FN>(dst_t + (int64_t)(vloc0 + row) * p.ldST, d);
       }
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
@@ -364,7 +370,7 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
           const int c = hh * 2 * FM + i * 2 + half, row = j * 32 + ln;
           store_run<TIN, 8>(reinterpret_cast<TIN*>(stage_lds + row * Stg::ROW_BYTES + ((c ^ Stg::swz(row)) * 16)), stage[j]);
         } else {
-          if (tok_ok[j] && !(p.dbg & 1))
+          if (tok_ok[j])
             store_run<TIN, 8>(dst_s + (tok0 + j * 32 + ln) * p.ldS + i * 16 + half * 8, stage[j]);
         }
       }
@@ -373,15 +379,13 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
   if constexpr (Stg::kEnabled) {
     // the staging tile is private to this wave: LDS operations of one wave complete in order
     const int lane = hh * 32 + ln;
-    if (!(p.dbg & 1)) {
 #pragma unroll
-      for (int it = 0; it < Stg::WAVE_BYTES / 1024; ++it) {
-        const int q = it * 64 + lane, row = q / Stg::CPR, pc = q % Stg::CPR;
-        const int c = pc ^ Stg::swz(row);
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage_lds + row * Stg::ROW_BYTES + pc * 16);
-        const int64_t tok = tok0 + row;
-        if (tok < p.T) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
-      }
+    for (int it = 0; it < Stg::WAVE_BYTES / 1024; ++it) {
+      const int q = it * 64 + lane, row = q / Stg::CPR, pc = q % Stg::CPR;
+      const int c = pc ^ Stg::swz(row);
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage_lds + row * Stg::ROW_BYTES + pc * 16);
+      const int64_t tok = tok0 + row;
+      if (tok < p.T) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
     }
   }
 }
@@ -410,10 +414,6 @@ LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
     }
   }
   const bool interior = vloc0 + Cfg::WM <= p.vrows && tok0 + Cfg::WN <= p.T;
-  if (p.dbg & 4) {
-    if (acc[0][0][0] == 123.456f) p.dS[0] = (typename Cfg::TIN)1.f;
-    return;
-  }
   __syncthreads();  // every wave's slab loads have landed and its operand reads are done: LDS is free
   char* stage_lds = lds + g.wave * DsStage<Cfg>::WAVE_BYTES;
   if (interior && __builtin_amdgcn_ballot_w64(has_label) == 0) ds_epilogue<Cfg, false>(p, acc, tok0, vloc0, hh, ln, stage_lds);
