@@ -76,6 +76,21 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                         const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream);
 
+/* Consumer of the path's outputs: the clipped PPO policy loss with dual clip, token-mean
+ * aggregation and entropy bonus.  Replaces, for the vanilla loss with token-mean aggregation,
+ * compute_policy_loss_vanilla + agg_loss (verl/trainer/ppo/core_algos.py:1140-1206, :1286-1376) and the
+ * entropy term of ppo_loss (verl/workers/utils/losses.py:134-140), and yields the upstream gradients
+ * lce_backward consumes, so no elementwise autograd graph sits between the two kernels.
+ *   all inputs fp32 [N] (flattened batch x response); entropy / g_entropy may both be NULL
+ *   token_scale: dp_size / batch_num_tokens, or <= 0 to use 1 / sum(mask)
+ *   out [8]: loss, pg_loss, entropy_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower, sum(mask), scale
+ *   g_log_prob, g_entropy [N]: d loss / d log_prob, d loss / d entropy (zero outside the mask) */
+size_t lce_ppo_loss_workspace_bytes(int64_t N);
+int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
+                 const float* mask, int64_t N, float clip_low, float clip_high, float clip_c, float entropy_coeff,
+                 float token_scale, float* out, float* g_log_prob, float* g_entropy, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
 /* Diagnostic: C[M, N] (fp32, row stride ldc) = A[M, K] . B[N, K]^T with the library's MFMA
  * mainloop (the same code that the entry points above use).  K a multiple of 64 (bf16) / 32 (fp32).
  * No counterpart in the reference; exists so the mainloop can be tested and timed on its own. */

@@ -1,0 +1,99 @@
+"""Fused PPO actor loss kernel against the oracle's restatement of compute_policy_loss_vanilla + agg_loss +
+entropy bonus (verl/trainer/ppo/core_algos.py:1140-1206,1286-1376; verl/workers/utils/losses.py:57-140)."""
+
+import pytest
+import torch
+
+from oracle import lce_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(B, L, seed, spread=0.05):
+    g = torch.Generator().manual_seed(seed)
+    lp = -torch.rand(B, L, generator=g) * 3
+    old = lp + torch.randn(B, L, generator=g) * spread
+    adv = torch.randn(B, 1, generator=g).expand(B, L).contiguous()
+    ent = torch.rand(B, L, generator=g) * 5
+    valid = torch.randint(1, L + 1, (B,), generator=g)
+    mask = (torch.arange(L)[None, :] < valid[:, None]).float()
+    return [t.to(DEV) for t in (lp, ent, old, adv, mask)]
+
+
+@pytest.mark.parametrize("spread", [0.05, 0.6, 3.0])  # 3.0 drives ratios into clip, dual-clip and the +-20 clamp
+@pytest.mark.parametrize("with_entropy", [True, False])
+def test_matches_oracle(spread, with_entropy):
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask = _case(16, 257, seed=int(spread * 100), spread=spread)
+    old = old + (torch.rand_like(old) < 0.01).float() * 25.0  # a few beyond the log-ratio clamp
+    lp1 = lp.clone().requires_grad_(True)
+    ent1 = ent.clone().requires_grad_(True) if with_entropy else None
+    loss, met = fused_ppo_loss(lp1, ent1, old, adv, mask, clip_ratio=0.2, clip_ratio_c=3.0, entropy_coeff=1e-3)
+    (loss * 1.7).backward()
+    lp2 = lp.clone().requires_grad_(True)
+    ent2 = ent.clone().requires_grad_(True) if with_entropy else None
+    rloss, rmet = O.ppo_actor_loss(lp2, ent2, old, adv, mask, clip_ratio=0.2, entropy_coeff=1e-3)
+    (rloss * 1.7).backward()
+    torch.testing.assert_close(loss, rloss, atol=1e-6, rtol=1e-5)
+    for k, v in met.items():
+        assert v.item() == pytest.approx(rmet[k], rel=1e-5, abs=1e-6), k
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-8, rtol=1e-5)
+    if with_entropy:
+        torch.testing.assert_close(ent1.grad, ent2.grad, atol=1e-9, rtol=1e-5)
+        assert (ent1.grad[mask == 0] == 0).all()
+    assert (lp1.grad[mask == 0] == 0).all()
+
+
+def test_global_batch_scaling_and_errors():
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask = _case(4, 64, seed=3)
+    loss, _ = fused_ppo_loss(lp, ent, old, adv, mask, entropy_coeff=0.01, dp_size=4, batch_num_tokens=1000)
+    pg, _ = O.policy_loss_vanilla(old, lp, adv, mask, dp_size=4, batch_num_tokens=1000)
+    want = pg - 0.01 * O.agg_loss(ent, mask, "token-mean", dp_size=4, batch_num_tokens=1000)
+    torch.testing.assert_close(loss, want, atol=1e-6, rtol=1e-5)
+    with pytest.raises(ValueError):
+        fused_ppo_loss(lp, ent, old, adv, mask, dp_size=2)
+    with pytest.raises(NotImplementedError):
+        fused_ppo_loss(lp, ent, old, adv, mask, loss_agg_mode="seq-mean-token-sum")
+    # NaNs outside the mask do not leak (masked_sum semantics, verl/utils/torch_functional.py:273-291)
+    lp_nan = lp.clone()
+    lp_nan[mask == 0] = float("nan")
+    loss_nan, _ = fused_ppo_loss(lp_nan, ent, old, adv, mask, entropy_coeff=0.01)
+    loss_ok, _ = fused_ppo_loss(lp, ent, old, adv, mask, entropy_coeff=0.01)
+    torch.testing.assert_close(loss_nan, loss_ok)
+
+
+def test_actor_step_fused_end_to_end():
+    """fused head -> fused loss -> fused backward, against the all-oracle pipeline (config-5 family, reduced)."""
+    from verl_amd import linear_cross_entropy
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    H, V, nseq, L = 1024, 32000, 8, 128
+    T = nseq * L
+    g = torch.Generator(device=DEV).manual_seed(7)
+    h = torch.randn(T, H, device=DEV, generator=g).bfloat16()
+    w = (torch.randn(V, H, device=DEV, generator=g) * 0.02).bfloat16()
+    y = torch.randint(0, V, (T,), device=DEV, generator=g)
+    valid = torch.randint(8, L + 1, (nseq,), device=DEV, generator=g)
+    mask = (torch.arange(L, device=DEV)[None, :] < valid[:, None]).float()
+    adv = torch.randn(nseq, 1, device=DEV, generator=g).expand(nseq, L).contiguous()
+    noise = torch.randn(nseq, L, device=DEV, generator=g) * 0.05
+    hh = h.clone().requires_grad_(True)
+    ww = w.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(hh, ww, y, 1.0, "none")
+    old = lp.detach().view(nseq, L) + noise
+    loss, _ = fused_ppo_loss(lp.view(nseq, L), ent.view(nseq, L), old, adv, mask, entropy_coeff=1e-3)
+    loss.backward()
+    h2 = h.clone().requires_grad_(True)
+    w2 = w.clone().requires_grad_(True)
+    z = h2.float() @ w2.float().t()
+    rlp = torch.log_softmax(z, -1).gather(-1, y[:, None]).squeeze(-1)
+    rent = torch.logsumexp(z, -1) - (torch.softmax(z, -1) * z).sum(-1)
+    rloss, _ = O.ppo_actor_loss(rlp.view(nseq, L), rent.view(nseq, L), old, adv, mask, entropy_coeff=1e-3)
+    rloss.backward()
+    torch.testing.assert_close(loss, rloss, atol=1e-4, rtol=1e-4)
+    assert (hh.grad.float() - h2.grad).abs().max() <= 2e-2 * h2.grad.abs().max()
+    assert (ww.grad.float() - w2.grad).abs().max() <= 2e-2 * w2.grad.abs().max()

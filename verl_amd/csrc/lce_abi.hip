@@ -493,6 +493,36 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   return check_launch("logits_fwd_kernel");
 }
 
+size_t lce_ppo_loss_workspace_bytes(int64_t N) {
+  (void)N;
+  return 1024 * 8 * sizeof(float);
+}
+
+int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
+                 const float* mask, int64_t N, float clip_low, float clip_high, float clip_c, float entropy_coeff,
+                 float token_scale, float* out, float* g_log_prob, float* g_entropy, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  if (N <= 0) return fail(LCE_E_ARG, "ppo loss: N must be positive");
+  if (!log_prob || !old_log_prob || !advantages || !mask || !out || !g_log_prob) return fail(LCE_E_ARG, "null pointer");
+  if ((entropy == nullptr) != (g_entropy == nullptr)) return fail(LCE_E_ARG, "entropy and g_entropy go together");
+  if (!(clip_c > 1.f)) return fail(LCE_E_ARG, "clip_ratio_c must be greater than 1");
+  if (!workspace || workspace_bytes < lce_ppo_loss_workspace_bytes(N)) return fail(LCE_E_WORKSPACE, "ppo workspace too small");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  int blocks = (int)((N + 255) / 256);
+  if (blocks > 1024) blocks = 1024;
+  PpoArgs p;
+  p.log_prob = log_prob; p.entropy = entropy; p.old_log_prob = old_log_prob; p.advantages = advantages; p.mask = mask;
+  p.N = N; p.clip_low = clip_low; p.clip_high = clip_high; p.clip_c = clip_c; p.entropy_coeff = entropy_coeff;
+  p.g_log_prob = g_log_prob; p.g_entropy = g_entropy; p.partials = static_cast<float*>(workspace);
+  hipLaunchKernelGGL(ppo_terms_kernel, dim3(blocks), dim3(256), 0, st, p);
+  int rc = check_launch("ppo_terms_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL(ppo_finish_kernel, dim3(1), dim3(64), 0, st, p.partials, blocks, token_scale, entropy_coeff, out);
+  if ((rc = check_launch("ppo_finish_kernel"))) return rc;
+  hipLaunchKernelGGL(ppo_scale_kernel, dim3(blocks), dim3(256), 0, st, g_log_prob, g_entropy, N, out);
+  return check_launch("ppo_scale_kernel");
+}
+
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                         const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream) {
   if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);

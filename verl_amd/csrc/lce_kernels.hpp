@@ -639,4 +639,100 @@ __global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// consumer of the path's outputs: clipped PPO policy loss + entropy bonus, token-mean aggregation
+// ------------------------------------------------------------------------------------------------
+struct PpoArgs {
+  const float* log_prob;
+  const float* entropy;  // may be null
+  const float* old_log_prob;
+  const float* advantages;
+  const float* mask;
+  int64_t N;
+  float clip_low, clip_high, clip_c, entropy_coeff;
+  float* g_log_prob;  // unscaled d(sum of masked losses)/d log_prob
+  float* g_entropy;   // may be null
+  float* partials;    // [blocks][8]
+};
+
+// one element; returns the masked per-token terms and the unscaled gradients
+__global__ void ppo_terms_kernel(PpoArgs p) {
+  __shared__ float sh[8][256];
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < p.N; t += (int64_t)gridDim.x * blockDim.x) {
+    const float m = p.mask[t];
+    const float lp = p.log_prob[t], A = p.advantages[t];
+    const float d = lp - p.old_log_prob[t];
+    const float nkl = fminf(fmaxf(d, -20.f), 20.f);
+    const float r = __expf(nkl);
+    const float dr = (d > -20.f && d < 20.f) ? r : 0.f;          // d ratio / d log_prob
+    const float rc = fminf(fmaxf(r, 1.f - p.clip_low), 1.f + p.clip_high);
+    const float drc = (r > 1.f - p.clip_low && r < 1.f + p.clip_high) ? dr : 0.f;
+    const float l1 = -A * r, l2 = -A * rc, l3 = -A * p.clip_c;
+    const float lc1 = fmaxf(l1, l2);
+    const float dlc1 = l1 > l2 ? -A * dr : (l2 > l1 ? -A * drc : -A * 0.5f * (dr + drc));
+    const bool dual = A < 0.f;
+    const float loss = dual ? fminf(l3, lc1) : lc1;
+    const float dloss = (dual && l3 < lc1) ? 0.f : dlc1;
+    const bool on = m != 0.f;  // values outside the mask never reach a sum (NaNs there are harmless)
+    p.g_log_prob[t] = on ? dloss * m : 0.f;
+    float ent = 0.f;
+    if (p.entropy) {
+      ent = p.entropy[t];
+      p.g_entropy[t] = on ? -p.entropy_coeff * m : 0.f;
+    }
+    if (on) {
+      s[0] += loss * m;
+      s[1] += ent * m;
+      s[2] += (l2 > l1 ? 1.f : 0.f) * m;
+      s[3] += -nkl * m;
+      s[4] += ((lc1 > l3 && dual) ? 1.f : 0.f) * m;
+    }
+    s[5] += m;
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) sh[k][threadIdx.x] = s[k];
+  __syncthreads();
+  for (int w = blockDim.x >> 1; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sh[k][threadIdx.x] += sh[k][threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x < 8) p.partials[blockIdx.x * 8 + threadIdx.x] = sh[threadIdx.x][0];
+}
+
+// out: [0] loss, [1] pg_loss, [2] entropy_loss, [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower,
+//      [6] number of masked tokens, [7] scale applied to the per-token sums
+__global__ void ppo_finish_kernel(const float* partials, int blocks, float token_scale, float entropy_coeff, float* out) {
+  __shared__ double tot[8];
+  if (threadIdx.x < 8) {
+    double a = 0.0;
+    for (int b = 0; b < blocks; ++b) a += (double)partials[b * 8 + threadIdx.x];
+    tot[threadIdx.x] = a;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const double n = tot[5];
+    const double scale = token_scale > 0.f ? (double)token_scale : 1.0 / n;  // token-mean: dp_size / batch_num_tokens
+    const double pg = tot[0] * scale, el = tot[1] * scale;
+    out[0] = (float)(pg - (double)entropy_coeff * el);
+    out[1] = (float)pg;
+    out[2] = (float)el;
+    out[3] = (float)(tot[2] / (n + 1e-8));
+    out[4] = (float)(tot[3] / (n + 1e-8));
+    out[5] = (float)(tot[4] / (n + 1e-8));
+    out[6] = (float)n;
+    out[7] = (float)scale;
+  }
+}
+
+__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t N, const float* out) {
+  const float scale = out[7];
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < N; t += (int64_t)gridDim.x * blockDim.x) {
+    g_lp[t] *= scale;
+    if (g_ent) g_ent[t] *= scale;
+  }
+}
+
 }  // namespace lce
