@@ -18,6 +18,10 @@
 
 namespace lce {
 
+#ifdef LCE_DBG_TIMING
+__device__ unsigned long long lce_dbg_times[16];
+#endif
+
 typedef __bf16 bf16_t;
 typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -239,22 +243,56 @@ struct GemmCore {
     load_frags(lds, 0, af[0], bf[0]);
     int stage = 0;
     int64_t kb_next = (int64_t)NS * Cfg::BKB;
+#ifdef LCE_DBG_TIMING
+    uint64_t dbg_compute = 0, dbg_vm = 0, dbg_bar = 0;
+    uint64_t dbg_last = __builtin_amdgcn_s_memtime();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    const uint64_t dbg_t0 = dbg_last;
+#endif
     for (int it = 0; it < nk; ++it) {
       const char* s = lds + stage * Cfg::STAGE_BYTES;
 #pragma unroll
-      for (int kk = 0; kk < KSUB - 1; ++kk)
+      for (int kk = 0; kk < KSUB - 1; ++kk) {
         substep<false>(acc, af[kk & 1], bf[kk & 1], s, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1], lds, 0, 0);
+      }
       // last substep of this slab: its fragments are in registers, so this wave is done with the stage
       const int nstage = stage + 1 == NS ? 0 : stage + 1;
+#ifdef LCE_DBG_TIMING
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      const uint64_t t1 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      wait_vm<(NS - 2) * PER>();
+      const uint64_t t2 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();
+      const uint64_t t3 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      dbg_compute += t1 - dbg_last;  // last substep of the previous slab + substeps 0..KSUB-2 of this one
+      dbg_vm += t2 - t1;
+      dbg_bar += t3 - t2;
+      dbg_last = t3;
+#else
       wait_vm<(NS - 2) * PER>();           // slab it+1 has landed (only the younger slabs may be in flight)
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of the stage have returned
       __builtin_amdgcn_s_barrier();
+#endif
       substep<true>(acc, af[(KSUB - 1) & 1], bf[(KSUB - 1) & 1], lds + nstage * Cfg::STAGE_BYTES, 0, af[0], bf[0], lds,
                     stage, kb_next < last_kbyte ? kb_next : last_kbyte);
       kb_next += Cfg::BKB;
       stage = nstage;
     }
     wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
+#ifdef LCE_DBG_TIMING
+    if (lane == 0 && (wave == 0 || wave == Cfg::NW - 1)) {
+      const uint64_t t_end = __builtin_amdgcn_s_memtime();
+      unsigned long long* d = lce_dbg_times + (wave == 0 ? 0 : 8);
+      atomicAdd(d + 0, (unsigned long long)dbg_compute);
+      atomicAdd(d + 1, (unsigned long long)dbg_vm);
+      atomicAdd(d + 2, (unsigned long long)dbg_bar);
+      atomicAdd(d + 3, (unsigned long long)(t_end - dbg_t0));
+      atomicAdd(d + 4, (unsigned long long)nk);
+    }
+#endif
   }
 
   template <int N>

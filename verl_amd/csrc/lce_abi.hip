@@ -344,6 +344,18 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
 
 extern "C" {
 
+#ifdef LCE_DBG_TIMING
+int lce_dbg_read(unsigned long long* out, int reset) {
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(lce::lce_dbg_times), 16 * sizeof(unsigned long long));
+  if (reset) {
+    unsigned long long z[16] = {0};
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(lce::lce_dbg_times), z, sizeof(z));
+  }
+  return 0;
+}
+#endif
+
 int lce_abi_version(void) { return LCE_ABI_VERSION; }
 const char* lce_last_error(void) { return g_err; }
 int lce_num_variants(void) { return kNumVariants; }
