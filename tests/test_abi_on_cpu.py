@@ -43,8 +43,11 @@ def test_abi_version_and_error_string():
     assert rc == -1 and b"dtype" in lib.lce_last_error()
     assert lib.lce_forward_workspace_bytes(16384, 3584, 152064, 0) < (64 << 20)
     # backward workspace stays far below a [T, V] tile pair: bounded d_logits chunk + transposed operands + fp32 d_hidden
-    T, H, V = 16384, 3584, 152064
-    assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) < 0.25 * T * V * 2 + 4 * V * H
+    # (at every token count: few tokens add K-split partials of d_hidden, many tokens narrow the chunk)
+    for T, H, V, dt in [(16384, 3584, 152064, 0), (8192, 2048, 152064, 0), (64, 3584, 152064, 0), (1024, 4096, 128256, 0),
+                        (4096, 3584, 152064, 1), (65536, 5120, 152064, 0), (262144, 4096, 128256, 0)]:
+        esz = 2 if dt == 0 else 4
+        assert lib.lce_backward_workspace_bytes(T, H, V, dt, 0) < 0.25 * T * V * esz + 4 * V * H, (T, H, V, dt)
 
 
 def test_signature_matches_reference():

@@ -283,6 +283,37 @@ def test_vocab_chunking_is_transparent(vchunk):
     torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
 
 
+@pytest.mark.parametrize("T,H,V,vchunk,dtype", [
+    (64, 256, 5000, 2048, torch.bfloat16),   # 16 K slices per chunk; the short last chunk leaves half of them empty
+    (100, 128, 300, 0, torch.bfloat16),      # single chunk narrower than the slices: empty slices on the first chunk
+    (1, 128, 2500, 1024, torch.float32),
+    (300, 512, 9000, 0, torch.float32),
+])
+def test_few_tokens_split_the_d_hidden_reduction(T, H, V, vchunk, dtype):
+    """With few tokens the vocabulary reduction of d_hidden is cut into K slices with one fp32 partial
+    each (summed in a fixed order at the end); results must not depend on it."""
+    from verl_amd.utils.kernel import kernels
+
+    tau = 0.8
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, dtype, seed=19)
+    try:
+        kernels.set_vocab_chunk(vchunk)
+        _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+        _, _, dh2, dw2 = _run(h, w, y, tau, g_lp, g_ent)
+    finally:
+        kernels.set_vocab_chunk(0)
+    if dtype == torch.float32:
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+        for got, want in ((dh, rdh), (dw, rdw)):
+            err = (got.double() - want).abs().max().item()
+            assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
+    else:
+        rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+        torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+        torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2)  # fixed summation order: bit-identical reruns
+
+
 def test_every_tile_variant_agrees():
     from verl_amd import _abi
 

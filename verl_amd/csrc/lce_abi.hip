@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include <mutex>
+#include <utility>
 #include <vector>
 
 #include "lce_kernels.hpp"
@@ -92,6 +93,7 @@ GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t l
   GemmArgs<typename Cfg::TIN> p;
   p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
   p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
+  p.ksplit = 1; p.kslice = K; p.cf_split_stride = 0;
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   return p;
@@ -172,21 +174,28 @@ struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
   size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, total;
   int nchunks;
+  int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
 };
 
-BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
+// The d_hidden GEMM has only ceil(T/256) * ceil(H/256) output tiles, each with a K loop as long as the
+// vocabulary chunk.  With few tokens one such tile takes longer than a CU's share of the whole launch
+// (d_logits tiles + both GEMMs) and would set the launch's duration; the K range is then cut into
+// slices, with an fp32 partial each, so that a tile takes at most about half of that share.
+int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
+  const int64_t ntt = (T + 255) / 256, nht = (H + 255) / 256, nvt = (vchunk + 255) / 256;
+  const int64_t work = ntt * nvt * H + nvt * nht * ntt * 256 + ntt * nht * vchunk;  // in K elements of 256x256 tiles
+  const int64_t share = work / 256 / 2;
+  const int64_t s = share > 0 ? (vchunk + share - 1) / share : 16;
+  return (int)(s < 1 ? 1 : s > 16 ? 16 : s);
+}
+
+// layout for a given chunk width
+BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
   BwdLayout L;
-  if (vchunk <= 0) {
-    // default: as wide as possible (fewer, longer launches) while the whole workspace stays below a
-    // quarter of one [T, V] tile plus one fp32 [V, H]:  8*T*vc*esz/2 + esz*V*H + (esz+4)*T*H  <=  0.25*T*V*esz + 4*V*H
-    const double tv = 0.25 * (double)T * V * esz, vh = (4.0 - esz) * (double)V * H, th = (esz + 4.0) * (double)T * H;
-    const double bound = (tv + vh - th) / (4.0 * esz * (double)T);
-    vchunk = bound > 16384.0 ? 16384 : (int64_t)(bound / 1024.0) * 1024;
-    if (vchunk < 2048) vchunk = 2048;
-  }
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
+  L.ksplit = dh_ksplit(T, H, vchunk);
   L.nchunks = (int)((V + vchunk - 1) / vchunk);
   // Row strides are kept away from large powers of two (+128 bytes): with a 16 or 32 KiB stride the
   // 256 rows of an operand tile would all fall into the same L2 channel.
@@ -209,9 +218,25 @@ BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk
   }
   L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
   L.off_Ht = o;    o += align256((size_t)H * L.ldHt * esz);
-  L.off_dHacc = o; o += L.nchunks > 1 ? align256((size_t)T * H * 4) : 0;
+  L.off_dHacc = o; o += (L.nchunks > 1 || L.ksplit > 1) ? (size_t)L.ksplit * align256((size_t)T * H * 4) : 0;
   L.total = o;
   return L;
+}
+
+// vchunk <= 0 picks the default chunk width: as wide as possible (fewer, longer launches) while the
+// whole workspace stays below a quarter of one [T, V] tile plus one fp32 [V, H],
+//   8*T*vc*esz/2 + esz*V*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
+// and no wider than 16384 columns or, with few tokens, than what gives the d_logits pass 512 tiles.
+// gt, gv: K-permutation groups that tokens / vocabulary are rounded up to (at most one workgroup
+// tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
+BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
+  if (vchunk <= 0) {
+    const double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
+    const int64_t ntt = (T + 255) / 256;
+    vchunk = ntt >= 8 ? 16384 : 512 * 256 / ntt;
+    while (vchunk > 2048 && (double)bwd_layout_for(T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
+  }
+  return bwd_layout_for(T, H, V, esz, vchunk, gt, gv);
 }
 
 template <typename Cfg>
@@ -244,6 +269,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   for (int c = 0; c <= L.nchunks; ++c) {
     BwdChunkArgs<TIN> p;
     p.n_gw = p.n_gh = p.n_ds = 0;
+    bool swapped = false;
     if (c < L.nchunks) {
       const int64_t v0 = (int64_t)c * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
@@ -266,16 +292,26 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
       const bool first = cc == 0, last = cc == L.nchunks - 1;
-      const int mode_h = (first ? 0 : 1) | (last ? 2 : 0);
+      const int mode_h = (first ? 0 : 1) | ((last && L.ksplit == 1) ? 2 : 0);
       p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h);
+      if (L.ksplit > 1) {
+        p.gh.ksplit = L.ksplit;
+        p.gh.kslice = round_up((kc + L.ksplit - 1) / L.ksplit, Cfg::BK);
+        p.gh.cf_split_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
+      }
       // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
       p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
-      p.n_gh = p.gh.map.total;
+      p.n_gh = p.gh.map.total * L.ksplit;
       p.n_gw = p.gw.map.total;
+      if (p.gh.kslice > p.gw.K) {  // longer tiles go first
+        std::swap(p.gh, p.gw);
+        std::swap(p.n_gh, p.n_gw);
+        swapped = true;
+      }
     }
     if (g_split_bwd) {
       const int n[3] = {p.n_gw, p.n_gh, p.n_ds};
-      const int cls[3] = {PC_GEMM_DW, PC_GEMM_DH, PC_BWD_DS};
+      const int cls[3] = {swapped ? PC_GEMM_DH : PC_GEMM_DW, swapped ? PC_GEMM_DW : PC_GEMM_DH, PC_BWD_DS};
       for (int k = 0; k < 3; ++k) {
         if (n[k] == 0) continue;
         BwdChunkArgs<TIN> q = p;
@@ -290,6 +326,15 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     ProfScope prof(PC_BWD_CHUNK, st);
     hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
+  }
+  if (L.ksplit > 1) {
+    ProfScope prof(PC_GEMM_DH, st);
+    const int64_t n = T * H;
+    int64_t blocks = (n / 4 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(splitk_reduce_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
+                       (int64_t)(align256((size_t)T * H * 4) / 4), n, d_hidden);
+    if ((rc = check_launch("splitk_reduce_kernel"))) return rc;
   }
   return LCE_OK;
 }

@@ -438,6 +438,10 @@ struct GemmArgs {
   int64_t ldct;
   int out_mode;
   TileMap map;  // rows = M tiles, cols = N tiles
+  // split K: workgroup `bid` computes tile bid % map.total over k in [s * kslice, min(K, (s + 1) * kslice)),
+  // s = bid / map.total < ksplit, into the fp32 partial Cf + s * cf_split_stride (out_mode 0 or 1 only)
+  int ksplit;
+  int64_t kslice, cf_split_stride;
 };
 
 template <typename Cfg, int MODE, bool EDGE>
@@ -470,15 +474,34 @@ LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t 
 }
 
 template <typename Cfg>
-LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
+  GemmArgs<typename Cfg::TIN> p = pin;
+  int64_t k0 = 0, k1 = p.K;
+  if (p.ksplit > 1) {
+    const int s = bid / p.map.total;
+    bid -= s * p.map.total;
+    k0 = s * p.kslice;
+    k1 = k0 + p.kslice < p.K ? k0 + p.kslice : p.K;
+    p.Cf += s * p.cf_split_stride;
+  }
   int tm, tn;
   if (!p.map.decode(bid, tm, tn)) return;
   const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
-  g.init(p.A, p.lda, m0, p.M, p.B, p.ldb, n0, p.N);
+  g.init(p.A + k0, p.lda, m0, p.M, p.B + k0, p.ldb, n0, p.N);
   f32x16_t acc[Cfg::FM][Cfg::FN];
-  g.run(lds, p.K, acc);
+  if (k0 < k1) {
+    g.run(lds, k1 - k0, acc);
+  } else {  // empty slice of a short last chunk: contributes zero (and still initialises its partial)
+    if (p.out_mode != 0) return;
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  }
   const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
 #define LCE_EPI(MODE)                                                                           \
   if (edge) gemm_epilogue<Cfg, MODE, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);         \
@@ -510,8 +533,10 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_nt_kernel(GemmArgs<typenam
 // Sub-grid sizes are multiples of 32, which keeps (block id % 8) -> XCD intact for every sub-problem.
 template <typename TIN>
 struct BwdChunkArgs {
-  GemmArgs<TIN> gw;  // d_weight[chunk c-1] = dS^T . h^T      (K = T: longest tiles)
-  GemmArgs<TIN> gh;  // d_hidden (+)= dS . W^T[chunk c-1]      (K = chunk width)
+  // the two gradient GEMMs of chunk c-1, the one with the longer K loop per tile in the first slot:
+  //   d_weight[chunk c-1] = dS^T . h^T   (K = T)   and   d_hidden (+)= dS . W^T[chunk c-1]   (K = chunk width / K splits)
+  GemmArgs<TIN> gw;
+  GemmArgs<TIN> gh;
   DsArgs<TIN> ds;    // d_logits of chunk c                     (K = H, heavy epilogue)
   int n_gw, n_gh, n_ds;
 };
@@ -523,6 +548,20 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_chunk_kernel(BwdChunkAr
   if (bid < p.n_gw) gemm_tile<Cfg>(p.gw, bid, lds);
   else if (bid < p.n_gw + p.n_gh) gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds);
   else ds_tile<Cfg>(p.ds, bid - p.n_gw - p.n_gh, lds);
+}
+
+// out[i] = (T)(sum over s < S of part[s * stride + i]), i < n (n a multiple of 4); the sum runs in the
+// fixed order s = 0, 1, ..., so the result does not depend on scheduling
+template <typename T>
+__global__ void splitk_reduce_kernel(const float* part, int S, int64_t stride, int64_t n, T* out) {
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n; i += (int64_t)gridDim.x * blockDim.x * 4) {
+    float4 a = *reinterpret_cast<const float4*>(part + i);
+    for (int s = 1; s < S; ++s) {
+      const float4 b = *reinterpret_cast<const float4*>(part + s * stride + i);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    out[i] = (T)a.x; out[i + 1] = (T)a.y; out[i + 2] = (T)a.z; out[i + 3] = (T)a.w;
+  }
 }
 
 __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
