@@ -29,11 +29,16 @@ MEASURED_TRAFFIC = {
     }
 }
 WORKLOADS = {
-    # name: (T, H, V, temperature, weight std)
-    "qwen2.5-7b-head-T16384": (16384, 3584, 152064, 1.0, 0.02),
-    "llama3-8b-head-T32768": (32768, 4096, 128256, 0.6, 0.02),
-    "qwen2.5-32b-head-T65536": (65536, 5120, 152064, 1.0, 0.015),
-    "small": (2048, 1024, 32768, 1.0, 0.02),
+    # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step)
+    # `sequences` > 0: T is that many equally long rows, each with a valid prefix of U{shortest..row}
+    # tokens; the upstream gradients are zero on the masked suffix (as a PPO response mask gives them).
+    "qwen2.5-7b-head-T16384": (16384, 3584, 152064, 1.0, 0.02, 0, 0, False),
+    "llama3-8b-head-T32768": (32768, 4096, 128256, 0.6, 0.02, 8, 512, False),
+    "qwen2.5-32b-head-T65536": (65536, 5120, 152064, 1.0, 0.015, 0, 0, False),
+    # one actor micro-step: forward, clipped PPO loss (eps 0.2, dual clip 3.0, token-mean) with entropy
+    # bonus 1e-3, backward; the loss kernel produces the upstream gradients
+    "llama3-8b-actor-step-T262144": (262144, 4096, 128256, 1.0, 0.02, 64, 256, True),
+    "small": (2048, 1024, 32768, 1.0, 0.02, 0, 0, False),
 }
 
 
@@ -109,13 +114,28 @@ def main():
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
-    T, H, V, tau, wstd = WORKLOADS[args.workload]
+    T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload]
     g = torch.Generator(device=dev).manual_seed(1234 + 2)
     h = torch.randn(T, H, device=dev, generator=g).bfloat16().requires_grad_(True)
     w = (torch.randn(V, H, device=dev, generator=g) * wstd).bfloat16().requires_grad_(True)
     y = torch.randint(0, V, (T,), device=dev, generator=g)
     g_lp = torch.randn(T, device=dev, generator=g)
     g_ent = torch.randn(T, device=dev, generator=g)
+    mask = torch.ones(T, device=dev)
+    if nseq:
+        row = T // nseq
+        valid = torch.randint(shortest, row + 1, (nseq,), device=dev, generator=g)
+        mask = (torch.arange(row, device=dev)[None, :] < valid[:, None]).float().reshape(T)
+        g_lp, g_ent = g_lp * mask, g_ent * mask
+    t_active = int(mask.sum().item())
+    if ppo:
+        from verl_amd.workers.utils.losses import fused_ppo_loss
+
+        with torch.no_grad():
+            lp0, _ = linear_cross_entropy(h, w, y, tau, "none")
+        old_lp = lp0 + 0.05 * torch.randn(T, device=dev, generator=g)
+        adv = torch.randn(nseq, device=dev, generator=g).repeat_interleave(T // nseq)
+        del lp0
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
@@ -129,7 +149,11 @@ def main():
         h.grad = None
         w.grad = None
         lp, ent = linear_cross_entropy(h, w, y, tau, "none")
-        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        if ppo:
+            loss, _ = fused_ppo_loss(lp, ent, old_lp, adv, mask, clip_ratio=0.2, clip_ratio_c=3.0, entropy_coeff=1e-3)
+            loss.backward()
+        else:
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
     for _ in range(args.warmup):
         step()
@@ -153,21 +177,21 @@ def main():
     lib.lce_profile_enable(0)
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
     # the dominant kernel (largest share of the step) and its algorithmic FLOPs per launch:
-    # every MFMA kernel of the path does 2*T*V*H per step split over its launches
     # algorithmic FLOPs per step of each MFMA kernel class (the recompute of the logits in the
-    # backward is executed but not counted): forward 2TVH; backward d_hidden + d_weight 4TVH
-    algo = {"lce_fwd_kernel": 2.0, "lce_bwd_chunk_kernel": 4.0}
+    # backward is executed but not counted): forward 2*T*V*H; backward d_hidden + d_weight 4*Ta*V*H,
+    # Ta = tokens with a non-zero upstream gradient (the others add exactly zero and are skipped)
+    algo = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": 4.0 * t_active}
     if args.split_backward:
-        algo.update({"gemm_nt_kernel(d_hidden)": 2.0, "gemm_nt_kernel(d_weight)": 2.0})
-    executed = {"lce_fwd_kernel": 2.0, "lce_bwd_chunk_kernel": 6.0, "gemm_nt_kernel(d_hidden)": 2.0,
-                "gemm_nt_kernel(d_weight)": 2.0, "lce_bwd_ds_kernel": 2.0}
+        algo.update({"gemm_nt_kernel(d_hidden)": 2.0 * t_active, "gemm_nt_kernel(d_weight)": 2.0 * t_active})
+    executed = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": 6.0 * t_active, "gemm_nt_kernel(d_hidden)": 2.0 * t_active,
+                "gemm_nt_kernel(d_weight)": 2.0 * t_active, "lce_bwd_ds_kernel": 2.0 * t_active}
     mfma = {k: v for k, v in kernels.items() if k in algo}
     dom = max(mfma, key=lambda k: mfma[k]["ms_per_step"])
-    flops_per_launch = algo[dom] * T * V * H / mfma[dom]["launches_per_step"]
+    flops_per_launch = algo[dom] * V * H / mfma[dom]["launches_per_step"]
     achieved = flops_per_launch / (mfma[dom]["avg_ms"] * 1e-3)
     for k, v in kernels.items():
         if k in executed:
-            v["executed_tflops"] = executed[k] * T * V * H / (v["ms_per_step"] * 1e-3) / 1e12
+            v["executed_tflops"] = executed[k] * V * H / (v["ms_per_step"] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
         "kernel": dom,
@@ -193,10 +217,12 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd+bwd"},
-        "algorithmic_tflops": algorithmic / 1e12,  # 6*T*V*H per step
+        "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau,
+                   "pass": "fwd+ppo_loss+bwd" if ppo else "fwd+bwd", "tokens_with_gradient": t_active},
+        "algorithmic_tflops": algorithmic / 1e12,  # 6*T*V*H per step, the reference's accounting per token
         "frac_of_bf16_peak": algorithmic / PEAK_BF16,
-        "executed_tflops": 8.0 * T * V * H / (elapsed / args.steps) / 1e12,  # one recompute of the logits
+        # what the kernels execute: forward on T tokens, recompute + two GEMMs on the tokens with gradient
+        "executed_tflops": (2.0 * T + 6.0 * t_active) * V * H / (elapsed / args.steps) / 1e12,
         "roofline": roofline,
         "kernels": kernels,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),

@@ -314,6 +314,51 @@ def test_few_tokens_split_the_d_hidden_reduction(T, H, V, vchunk, dtype):
     assert torch.equal(dh, dh2) and torch.equal(dw, dw2)  # fixed summation order: bit-identical reruns
 
 
+@pytest.mark.parametrize("pattern", ["prefix", "random", "none", "single", "entropy_only", "first_tile_empty"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_tokens_without_upstream_gradient(pattern, dtype):
+    """Prompt and padding positions of a PPO batch arrive with zero upstream gradients.  The backward
+    runs on the list of the other tokens only; the result must equal the dense computation (their
+    contribution is exactly zero) and d_hidden must be exactly zero on the skipped rows."""
+    T, H, V, tau = 1500, 256, 5000, 0.9
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, dtype, seed=23)
+    g_lp, g_ent = g_lp.float(), g_ent.float()
+    g = torch.Generator().manual_seed(29)
+    if pattern == "prefix":       # three packed sequences, each with a masked suffix
+        keep = torch.zeros(T, dtype=torch.bool)
+        for a, b in ((0, 310), (500, 777), (1000, 1001)):
+            keep[a:b] = True
+    elif pattern == "random":
+        keep = torch.rand(T, generator=g) < 0.3
+    elif pattern == "none":
+        keep = torch.zeros(T, dtype=torch.bool)
+    elif pattern == "single":
+        keep = torch.zeros(T, dtype=torch.bool)
+        keep[1234] = True
+    elif pattern == "entropy_only":  # log-prob gradient zero everywhere, entropy gradient on a few tokens
+        keep = torch.rand(T, generator=g) < 0.1
+        g_lp = torch.zeros_like(g_lp)
+    else:                          # nothing in the first 256-token tile
+        keep = torch.ones(T, dtype=torch.bool)
+        keep[:300] = False
+    keep = keep.to(DEV)
+    g_lp, g_ent = g_lp * keep, g_ent * keep
+    _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    if dtype == torch.float32:
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+        for got, want in ((dh, rdh), (dw, rdw)):
+            err = (got.double() - want).abs().max().item()
+            assert err <= 1e-5 * max(want.abs().max().item(), 1e-30), (err, want.abs().max().item())
+    else:
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+        torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+        torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    dead = ~((g_lp != 0) | (g_ent != 0))
+    assert torch.count_nonzero(dh[dead]) == 0
+    if pattern == "none":
+        assert torch.count_nonzero(dw) == 0
+
+
 def test_every_tile_variant_agrees():
     from verl_amd import _abi
 

@@ -105,15 +105,17 @@ struct GemmCore {
   int wave, lane, wave_m, wave_n;
   uint32_t a_rd, b_rd;  // LDS byte offsets (within a stage) of this lane's operand rows, swizzle folded in
 
-  // rows beyond the matrix are clamped to its last row (their results are discarded by the epilogue)
+  // rows beyond the matrix are clamped to its last row (their results are discarded by the epilogue).
+  // With `b_rows` given, row n of the B operand is B[b_rows[n]] (a gather; B is then the matrix's first
+  // row and every row's byte offset must fit 32 bits).
   LCE_DEV void init(const TIN* A, int64_t lda, int64_t m0, int64_t M, const TIN* B, int64_t ldb, int64_t n0,
-                    int64_t N) {
+                    int64_t N, const int* b_rows = nullptr) {
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     lane = threadIdx.x & 63;
     wave_m = wave / Cfg::WAVES_N;
     wave_n = wave % Cfg::WAVES_N;
     a_base = reinterpret_cast<const char*>(A + m0 * lda);
-    b_base = reinterpret_cast<const char*>(B + n0 * ldb);
+    b_base = reinterpret_cast<const char*>(b_rows ? B : B + n0 * ldb);
     const int rows_a = (int)((M - m0) < (int64_t)Cfg::BM ? (M - m0) : (int64_t)Cfg::BM);
     const int rows_b = (int)((N - n0) < (int64_t)Cfg::BN ? (N - n0) : (int64_t)Cfg::BN);
     const int lr = lane / Cfg::CH, pc = lane % Cfg::CH;
@@ -129,7 +131,8 @@ struct GemmCore {
       const int row = (j * Cfg::NW + wave) * Cfg::ROWS_PER_LOAD + lr;
       const int c = pc ^ Cfg::swz(row);
       const int crow = row < rows_b ? row : rows_b - 1;
-      lb.voff[j] = (uint32_t)((int64_t)crow * ldb * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
+      const int64_t grow = b_rows ? (int64_t)b_rows[n0 + crow] : (int64_t)crow;
+      lb.voff[j] = (uint32_t)(grow * ldb * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
     }
     const int r32 = lane & 31, hh = lane >> 5;
     const int x = (hh ^ Cfg::swz(r32)) * 16;
@@ -315,6 +318,16 @@ struct TileMap {
   int rows_fastest;            // 1: consecutive blocks walk the row dimension first
   int total;                   // launched workgroups (multiple of 8)
 
+  // shape of the 32-tile blocks that one XCD works on: up to 8 tiles along the row side
+  __host__ __device__ static int block_rows(int nrow_tiles) {
+    int br = 1;
+    while (br < 8 && br < nrow_tiles) br <<= 1;
+    return br;
+  }
+  // the same map over fewer row tiles (a count that only the device knows): its workgroups are the
+  // first `total` ids of the grid that was sized for the full map, the others have nothing to do
+  __device__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, block_rows(rows), rows_fastest); }
+
   __host__ __device__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
     TileMap t;
     t.nrow_tiles = nrow_tiles;
@@ -329,6 +342,7 @@ struct TileMap {
   }
   // returns false when the slot is padding (no tile)
   __device__ bool decode(int bid, int& rt, int& ct) const {
+    if (bid >= total) return false;
     const int per_xcd = total >> 3;
     const int vid = (bid & 7) * per_xcd + (bid >> 3);
     const int blk = vid >> 5, within = vid & 31;

@@ -30,7 +30,7 @@ int fail(int code, const char* fmt, ...) {
 }
 
 // ---- optional per-kernel-class timing with HIP events (off by default; used by the benchmark) ----
-enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_BWD_CHUNK, PC_COUNT };
+enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_BWD_CHUNK, PC_ACTIVE_ROWS, PC_DH_FINISH, PC_COUNT };
 struct ProfRec { int cls; hipEvent_t a, b; };
 std::mutex g_prof_mu;
 bool g_prof_on = false;
@@ -78,12 +78,7 @@ void allow_lds(K kernel, int bytes) {
   (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-// choose the shape of the 32-tile blocks that one XCD works on (rows = `nrow_tiles` side)
-int block_rows(int nrow_tiles) {
-  int br = 1;
-  while (br < 8 && br < nrow_tiles) br <<= 1;
-  return br;
-}
+int block_rows(int nrow_tiles) { return TileMap::block_rows(nrow_tiles); }
 
 // ---------------------------------------------------------------------------------------------
 template <typename Cfg>
@@ -94,6 +89,7 @@ GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t l
   p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
   p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
   p.ksplit = 1; p.kslice = K; p.cf_split_stride = 0;
+  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1;
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   return p;
@@ -172,7 +168,7 @@ int forward_splits_upper_bound(int64_t T) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, total;
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
 };
@@ -218,7 +214,11 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   }
   L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
   L.off_Ht = o;    o += align256((size_t)H * L.ldHt * esz);
-  L.off_dHacc = o; o += (L.nchunks > 1 || L.ksplit > 1) ? (size_t)L.ksplit * align256((size_t)T * H * 4) : 0;
+  L.off_dHacc = o; o += (size_t)L.ksplit * align256((size_t)T * H * 4);
+  // list of the tokens with a non-zero upstream gradient, its inverse, and its length
+  L.off_rows = o;  o += align256((size_t)L.tpad * 4);
+  L.off_inv = o;   o += align256((size_t)T * 4);
+  L.off_nrows = o; o += 256;
   L.total = o;
   return L;
 }
@@ -252,6 +252,20 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   TIN* Ht = reinterpret_cast<TIN*>(ws + L.off_Ht);
   float* dHacc = reinterpret_cast<float*>(ws + L.off_dHacc);
   int rc;
+  // Tokens with zero upstream gradients (prompt and padding positions of a PPO batch) add nothing to
+  // either gradient: list the others on the device and run everything below on that list.  Nothing
+  // comes back to the host, so grids are sized for all T tokens and surplus workgroups exit at once.
+  // (The gather addresses rows of `hidden` with 32-bit byte offsets; larger inputs run uncompacted.)
+  const bool compact = (uint64_t)T * (uint64_t)ldh * sizeof(TIN) < (1ull << 32);
+  int* rows = compact ? reinterpret_cast<int*>(ws + L.off_rows) : nullptr;
+  int* inv = compact ? reinterpret_cast<int*>(ws + L.off_inv) : nullptr;
+  int* n_rows = compact ? reinterpret_cast<int*>(ws + L.off_nrows) : nullptr;
+  if (compact) {
+    ProfScope prof(PC_ACTIVE_ROWS, st);
+    hipLaunchKernelGGL(active_rows_kernel<1024>, dim3(1), dim3(1024), 0, st, dlogprobs,
+                       (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), dentropy, T, rows, inv, n_rows);
+    if ((rc = check_launch("active_rows_kernel"))) return rc;
+  }
   // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
   {
     ProfScope prof(PC_TRANSPOSE, st);
@@ -259,7 +273,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                        st, W, ldw, V, H, Wt, L.ldWt, L.vpad);
     if ((rc = check_launch("transpose W"))) return rc;
     hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)(L.tpad / 64), (unsigned)((H + 63) / 64)), dim3(256), 0,
-                       st, h, ldh, T, H, Ht, L.ldHt, L.tpad);
+                       st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
     if ((rc = check_launch("transpose h"))) return rc;
   }
 
@@ -281,6 +295,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
       d.g_ent = dentropy;
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
+      d.rows = rows; d.n_rows = n_rows;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       d.map = TileMap::make(ntt, nvt, block_rows(ntt), 1);
       p.n_ds = d.map.total;
@@ -289,11 +304,10 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int cc = c - 1;
       const int64_t v0 = (int64_t)cc * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
-      // d_hidden[T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T ; rounded to the output type on the last chunk
+      // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T  (rows = listed tokens)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
-      const bool first = cc == 0, last = cc == L.nchunks - 1;
-      const int mode_h = (first ? 0 : 1) | ((last && L.ksplit == 1) ? 2 : 0);
-      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, d_hidden, H, mode_h);
+      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+      p.gh.m_dev = n_rows;
       if (L.ksplit > 1) {
         p.gh.ksplit = L.ksplit;
         p.gh.kslice = round_up((kc + L.ksplit - 1) / L.ksplit, Cfg::BK);
@@ -301,6 +315,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       }
       // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
       p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
+      p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
       p.n_gh = p.gh.map.total * L.ksplit;
       p.n_gw = p.gw.map.total;
       if (p.gh.kslice > p.gw.K) {  // longer tiles go first
@@ -327,14 +342,14 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
-  if (L.ksplit > 1) {
-    ProfScope prof(PC_GEMM_DH, st);
-    const int64_t n = T * H;
-    int64_t blocks = (n / 4 + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(splitk_reduce_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
-                       (int64_t)(align256((size_t)T * H * 4) / 4), n, d_hidden);
-    if ((rc = check_launch("splitk_reduce_kernel"))) return rc;
+  {
+    // d_hidden = ordered sum of the fp32 partials, rounded once; zero rows for tokens without gradient
+    ProfScope prof(PC_DH_FINISH, st);
+    int64_t blocks = (T * (H / 4) + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(dh_finish_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
+                       (int64_t)(align256((size_t)T * H * 4) / 4), inv, T, H, d_hidden);
+    if ((rc = check_launch("dh_finish_kernel"))) return rc;
   }
   return LCE_OK;
 }
@@ -425,7 +440,7 @@ int lce_profile_num_classes(void) { return PC_COUNT; }
 const char* lce_profile_class_name(int cls) {
   static const char* names[PC_COUNT] = {"lce_fwd_kernel", "lce_fwd_merge_kernel", "lce_bwd_ds_kernel", "gemm_nt_kernel(d_hidden)",
                                         "gemm_nt_kernel(d_weight)", "transpose_pad_kernel", "logits_fwd_kernel", "logits_bwd_kernel",
-                                        "lce_bwd_chunk_kernel"};
+                                        "lce_bwd_chunk_kernel", "active_rows_kernel", "dh_finish_kernel"};
   return (cls >= 0 && cls < PC_COUNT) ? names[cls] : "";
 }
 int lce_profile_read(double* total_ms, int64_t* launches, int reset) {

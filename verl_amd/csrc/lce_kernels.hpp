@@ -243,6 +243,11 @@ struct DsArgs {
   int64_t ldST;
   int64_t tpad;         // tokens rounded up to the GEMM K granule: columns [T, tpad) of dST are written as zeros
   TileMap map;          // rows = token tiles, cols = vocab tiles of the chunk
+  // Token compaction (both null = off): only tokens with a non-zero upstream gradient take part.
+  // rows[k] is the token behind compact position k < *n_rows; dS / dS^T are indexed by k, while
+  // hidden, labels, the statistics and the upstream gradients are read at rows[k].
+  const int* rows;
+  const int* n_rows;
 };
 
 // The two gradient GEMMs sum over the vocabulary (d_hidden) and over the tokens (d_weight); any
@@ -317,7 +322,7 @@ struct DsStage {
 
 template <typename Cfg, bool SLOW>
 LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t tok0,
-                         int vloc0, int hh, int ln, char* stage_lds) {
+                         int64_t Tc, int vloc0, int hh, int ln, char* stage_lds) {
   typedef typename Cfg::TIN TIN;
   typedef DsStage<Cfg> Stg;
   constexpr int FM = Cfg::FM, FN = Cfg::FN;
@@ -326,11 +331,12 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
   bool tok_ok[FN];
 #pragma unroll
   for (int j = 0; j < FN; ++j) {
-    const int64_t tok = tok0 + j * 32 + ln;
-    tok_ok[j] = tok < p.T;
+    const int64_t pos = tok0 + j * 32 + ln;  // position in dS / dS^T
+    tok_ok[j] = pos < Tc;
     lse2[j] = C0[j] = C1[j] = G[j] = 0.f;
     rel[j] = -1;
     if (tok_ok[j]) {
+      const int64_t tok = p.rows ? (int64_t)p.rows[pos] : pos;
       const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
       const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
       lse2[j] = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
@@ -385,19 +391,23 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
       const int c = pc ^ Stg::swz(row);
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage_lds + row * Stg::ROW_BYTES + pc * 16);
       const int64_t tok = tok0 + row;
-      if (tok < p.T) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
+      if (tok < Tc) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
     }
   }
 }
 
 template <typename Cfg>
 LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+  const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;  // tokens that take part
   int tt, vt;
-  if (!p.map.decode(bid, tt, vt)) return;
+  // with a device-side token count the XCD-aware map is rebuilt over the token tiles that exist, so
+  // that they spread evenly over the XCDs (the host's map would leave whole XCDs without work)
+  const TileMap map = p.n_rows ? p.map.with_rows((int)((Tc + Cfg::BN - 1) / Cfg::BN)) : p.map;
+  if (!map.decode(bid, tt, vt)) return;
   const int64_t n0 = (int64_t)tt * Cfg::BN, m0 = (int64_t)vt * Cfg::BM;
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
-  g.init(p.W, p.ldw, m0, p.vrows, p.h, p.ldh, n0, p.T);
+  g.init(p.W, p.ldw, m0, p.vrows, p.h, p.ldh, n0, Tc, p.rows);
   f32x16_t acc[Cfg::FM][Cfg::FN];
   g.run(lds, p.H, acc);
 
@@ -408,16 +418,16 @@ LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
     const int64_t tok = tok0 + j * 32 + ln;
-    if (tok < p.T) {
-      const int64_t y = p.labels[tok] - p.v0;
+    if (tok < Tc) {
+      const int64_t y = p.labels[p.rows ? p.rows[tok] : tok] - p.v0;
       has_label |= (y >= vloc0 && y < vloc0 + Cfg::WM);
     }
   }
-  const bool interior = vloc0 + Cfg::WM <= p.vrows && tok0 + Cfg::WN <= p.T;
+  const bool interior = vloc0 + Cfg::WM <= p.vrows && tok0 + Cfg::WN <= Tc;
   __syncthreads();  // every wave's slab loads have landed and its operand reads are done: LDS is free
   char* stage_lds = lds + g.wave * DsStage<Cfg>::WAVE_BYTES;
-  if (interior && __builtin_amdgcn_ballot_w64(has_label) == 0) ds_epilogue<Cfg, false>(p, acc, tok0, vloc0, hh, ln, stage_lds);
-  else ds_epilogue<Cfg, true>(p, acc, tok0, vloc0, hh, ln, stage_lds);
+  if (interior && __builtin_amdgcn_ballot_w64(has_label) == 0) ds_epilogue<Cfg, false>(p, acc, tok0, Tc, vloc0, hh, ln, stage_lds);
+  else ds_epilogue<Cfg, true>(p, acc, tok0, Tc, vloc0, hh, ln, stage_lds);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -442,6 +452,11 @@ struct GemmArgs {
   // s = bid / map.total < ksplit, into the fp32 partial Cf + s * cf_split_stride (out_mode 0 or 1 only)
   int ksplit;
   int64_t kslice, cf_split_stride;
+  // sizes known only on the device (null = use M / K): rows that exist, M = min(M, *m_dev), and the
+  // reduction length, K = min(K, *k_dev rounded up to k_gran); K = 0 gives C = 0
+  const int* m_dev;
+  const int* k_dev;
+  int k_gran;
 };
 
 template <typename Cfg, int MODE, bool EDGE>
@@ -476,16 +491,25 @@ LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t 
 template <typename Cfg>
 LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
   GemmArgs<typename Cfg::TIN> p = pin;
+  if (p.m_dev) {
+    const int64_t m = *p.m_dev;
+    p.M = m < p.M ? m : p.M;
+  }
+  if (p.k_dev) {
+    const int64_t k = ((int64_t)*p.k_dev + p.k_gran - 1) / p.k_gran * p.k_gran;
+    p.K = k < p.K ? k : p.K;
+  }
   int64_t k0 = 0, k1 = p.K;
   if (p.ksplit > 1) {
-    const int s = bid / p.map.total;
+    const int s = bid / p.map.total;  // (the grid holds ksplit copies of the host-sized map)
     bid -= s * p.map.total;
     k0 = s * p.kslice;
     k1 = k0 + p.kslice < p.K ? k0 + p.kslice : p.K;
     p.Cf += s * p.cf_split_stride;
   }
   int tm, tn;
-  if (!p.map.decode(bid, tm, tn)) return;
+  const TileMap map = p.m_dev ? p.map.with_rows((int)((p.M + Cfg::BM - 1) / Cfg::BM)) : p.map;
+  if (!map.decode(bid, tm, tn)) return;
   const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
@@ -493,8 +517,8 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
   f32x16_t acc[Cfg::FM][Cfg::FN];
   if (k0 < k1) {
     g.run(lds, k1 - k0, acc);
-  } else {  // empty slice of a short last chunk: contributes zero (and still initialises its partial)
-    if (p.out_mode != 0) return;
+  } else {  // empty K range: contributes zero (and still initialises what it owns)
+    if (p.out_mode == 1) return;
 #pragma unroll
     for (int i = 0; i < Cfg::FM; ++i)
 #pragma unroll
@@ -550,18 +574,56 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_chunk_kernel(BwdChunkAr
   else ds_tile<Cfg>(p.ds, bid - p.n_gw - p.n_gh, lds);
 }
 
-// out[i] = (T)(sum over s < S of part[s * stride + i]), i < n (n a multiple of 4); the sum runs in the
-// fixed order s = 0, 1, ..., so the result does not depend on scheduling
+// d_hidden[t][:] = (T)(sum over s < S of part[s * stride + pos(t) * H + :]) with pos(t) = inv[t] (t itself
+// without `inv`), or zeros where inv[t] < 0 (token without upstream gradient).  The sum runs in the
+// fixed order s = 0, 1, ..., so the result does not depend on scheduling.  H a multiple of 4.
 template <typename T>
-__global__ void splitk_reduce_kernel(const float* part, int S, int64_t stride, int64_t n, T* out) {
-  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n; i += (int64_t)gridDim.x * blockDim.x * 4) {
-    float4 a = *reinterpret_cast<const float4*>(part + i);
-    for (int s = 1; s < S; ++s) {
-      const float4 b = *reinterpret_cast<const float4*>(part + s * stride + i);
-      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+__global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, T* out) {
+  const int64_t per_row = H / 4, n = ntok * per_row;
+  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t t = q / per_row, c = (q - t * per_row) * 4;
+    const int64_t pos = inv ? (int64_t)inv[t] : t;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pos >= 0) {
+      const float* src = part + pos * H + c;
+      a = *reinterpret_cast<const float4*>(src);
+      for (int s = 1; s < S; ++s) {
+        const float4 b = *reinterpret_cast<const float4*>(src + s * stride);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+      }
     }
-    out[i] = (T)a.x; out[i + 1] = (T)a.y; out[i + 2] = (T)a.z; out[i + 3] = (T)a.w;
+    T* dst = out + t * H + c;
+    dst[0] = (T)a.x; dst[1] = (T)a.y; dst[2] = (T)a.z; dst[3] = (T)a.w;
   }
+}
+
+// Tokens whose upstream gradients are both zero add nothing to either gradient.  One workgroup lists
+// the others in order: rows[k] = k-th such token, inv[t] = its position k or -1, *n_rows = how many.
+// g_lp has stride 0 when one value is shared by all tokens (sum / mean reduction).
+template <int NT>
+__global__ __launch_bounds__(NT) void active_rows_kernel(const float* g_lp, int64_t g_lp_stride, const float* g_ent, int64_t T,
+                                                          int* rows, int* inv, int* n_rows) {
+  __shared__ int counts[NT];
+  const int64_t per = (T + NT - 1) / NT;
+  const int64_t t0 = (int64_t)threadIdx.x * per, t1 = t0 + per < T ? t0 + per : T;
+  int n = 0;
+  for (int64_t t = t0; t < t1; ++t) n += (g_lp[t * g_lp_stride] != 0.f) || (g_ent && g_ent[t] != 0.f);
+  counts[threadIdx.x] = n;
+  __syncthreads();
+  // inclusive scan (Hillis-Steele)
+  for (int off = 1; off < NT; off <<= 1) {
+    const int v = threadIdx.x >= off ? counts[threadIdx.x - off] : 0;
+    __syncthreads();
+    counts[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int pos = counts[threadIdx.x] - n;
+  for (int64_t t = t0; t < t1; ++t) {
+    const bool on = (g_lp[t * g_lp_stride] != 0.f) || (g_ent && g_ent[t] != 0.f);
+    inv[t] = on ? pos : -1;
+    if (on) rows[pos++] = (int)t;
+  }
+  if (threadIdx.x == NT - 1) *n_rows = counts[NT - 1];
 }
 
 __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
@@ -571,16 +633,22 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
 // out[c][perm(r)] = in[r][c] for r < R, c < C; out has `ldo` columns, columns perm(r) with r in
 // [R, rpad) are zero-filled (rpad a multiple of the permutation's group).  PERM: 0 none,
 // 1 KPerm::token, 2 KPerm::vocab.  Grid: (rpad/64, ceil(C/64)), 256 threads.
+// With `rows` / `n_rows` (device), row r of the input is in[rows[r]] for r < *n_rows and R = *n_rows.
 template <typename Cfg, int PERM>
 __global__ void transpose_pad_kernel(const typename Cfg::TIN* in, int64_t ldi, int64_t R, int64_t C, typename Cfg::TIN* out,
-                                     int64_t ldo, int64_t rpad) {
+                                     int64_t ldo, int64_t rpad, const int* rows = nullptr, const int* n_rows = nullptr) {
   typedef typename Cfg::TIN TIN;
   __shared__ TIN tile[64][65];
   const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (n_rows) {
+    R = *n_rows;
+    if (r0 >= (R + 255) / 256 * 256) return;  // beyond the last K granule that any GEMM reads
+  }
   for (int i = ty; i < 64; i += 4) {
     const int64_t r = r0 + i, c = c0 + tx;
-    tile[i][tx] = (r < R && c < C) ? in[r * ldi + c] : (TIN)0.f;
+    const int64_t src = (rows && r < R) ? (int64_t)rows[r] : r;
+    tile[i][tx] = (r < R && c < C) ? in[src * ldi + c] : (TIN)0.f;
   }
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
