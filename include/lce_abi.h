@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 1
+#define LCE_ABI_VERSION 2
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -68,13 +68,16 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
 /* Unfused twins on logits that already exist in memory.
  * Replaces logprobs_from_logits (verl/utils/torch_functional.py:73-107, :155-207) and
  * entropy_from_logits (:231-245) with one pass over the rows.
- *   logits [R, V] row stride ldl, dtype LCE_DTYPE_*; labels [R] int64 or NULL; logprobs / entropy [R] fp32, either may be NULL. */
+ *   logits [R, V] row stride ldl, dtype LCE_DTYPE_*; labels [R] int64 or NULL; logprobs / entropy [R] fp32, either may be NULL;
+ *   stats [R, 2] fp32 or NULL: per row logsumexp and sum softmax * logit, which let the backward skip its own reduction pass. */
 int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
-                       float* logprobs, float* entropy, void* stream);
+                       float* logprobs, float* entropy, float* stats, void* stream);
 /* d_logits [R, V] (row stride ldd, same dtype as logits) of sum(dlogprobs*logprobs) + sum(dentropy*entropy);
- * dlogprobs / dentropy [R] fp32, either may be NULL.  Autograd twin of the two functions above. */
+ * dlogprobs / dentropy [R] fp32, either may be NULL; stats as written by lce_logits_forward for the same logits, or NULL
+ * (then recomputed).  Autograd twin of the two functions above. */
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
-                        const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream);
+                        const float* stats, const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd,
+                        void* stream);
 
 /* Consumer of the path's outputs: the clipped PPO policy loss with dual clip, token-mean
  * aggregation and entropy bonus.  Replaces, for the vanilla loss with token-mean aggregation,

@@ -35,6 +35,44 @@ def test_forward_and_backward(dtype, shape):
     torch.testing.assert_close(zz.grad.float(), want, **(dict(atol=1e-5, rtol=1e-4) if dtype == torch.float32 else tol))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,ldl,off_in,off_out", [(3001, 3001, 0, 0), (4099, 4200, 3, 3), (1000, 1024, 1, 5), (70000, 70000, 0, 0), (5, 8, 1, 0)])
+def test_row_alignment_strides_and_saved_statistics(dtype, V, ldl, off_in, off_out):
+    """The kernels read rows as [head | 16-byte vectors | tail]; rows that start at any element offset,
+    padded row strides and outputs aligned differently from the inputs must give the same values, and
+    the backward must give the same result with the forward's row statistics as when it recomputes them."""
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    R = 9
+    g = torch.Generator().manual_seed(V + off_in)
+    buf = (torch.randn(R * ldl + off_in, generator=g) * 3).to(dtype).to(DEV)
+    z = buf[off_in:].view(R, ldl)[:, :V]
+    y = torch.randint(0, V, (R,), generator=g).to(DEV)
+    lp = torch.empty(R, device=DEV)
+    ent = torch.empty(R, device=DEV)
+    stats = torch.empty(R, 2, device=DEV)
+    code = _abi.dtype_code(dtype)
+    st = _abi.current_stream(torch.device(DEV))
+    _abi.check(lib.lce_logits_forward(z.data_ptr(), ldl, y.data_ptr(), R, V, code, lp.data_ptr(), ent.data_ptr(), stats.data_ptr(), st), "fwd")
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(lp, O.logprobs_from_logits(z, y).float(), **tol)
+    torch.testing.assert_close(ent, O.entropy_from_logits(z).float(), **tol)
+    g_lp = torch.randn(R, generator=g).to(DEV)
+    g_ent = torch.randn(R, generator=g).to(DEV)
+    want = O.logits_backward(z, y, g_lp, g_ent)
+    outs = []
+    for use_stats in (True, False):
+        obuf = torch.full((R * ldl + off_out,), 7.0, device=DEV, dtype=dtype)
+        d = obuf[off_out:].view(R, ldl)
+        _abi.check(lib.lce_logits_backward(z.data_ptr(), ldl, y.data_ptr(), R, V, code, stats.data_ptr() if use_stats else None,
+                                           g_lp.data_ptr(), g_ent.data_ptr(), d.data_ptr(), ldl, st), "bwd")
+        torch.testing.assert_close(d[:, :V].float(), want, **(dict(atol=1e-5, rtol=1e-4) if dtype == torch.float32 else tol))
+        assert (d[:, V:] == 7.0).all() and (obuf[:off_out] == 7.0).all()  # nothing outside the rows is written
+        outs.append(d[:, :V].clone())
+    torch.testing.assert_close(outs[0].float(), outs[1].float(), atol=1e-6, rtol=1e-5) if dtype == torch.float32 else None
+
+
 def test_extreme_logits_and_variants():
     from verl_amd.utils import torch_functional as F
 

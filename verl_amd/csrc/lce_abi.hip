@@ -550,7 +550,7 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 }
 
 int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
-                       float* logprobs, float* entropy, void* stream) {
+                       float* logprobs, float* entropy, float* stats, void* stream) {
   if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
   if (R == 0) return LCE_OK;
@@ -559,9 +559,9 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   constexpr int NT = 512;
   ProfScope prof(PC_LOGITS_FWD, st);
   if (dtype == LCE_DTYPE_BF16)
-    hipLaunchKernelGGL((logits_fwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, logprobs, entropy);
+    hipLaunchKernelGGL((logits_fwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, logprobs, entropy, stats);
   else
-    hipLaunchKernelGGL((logits_fwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, logprobs, entropy);
+    hipLaunchKernelGGL((logits_fwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, logprobs, entropy, stats);
   return check_launch("logits_fwd_kernel");
 }
 
@@ -596,7 +596,8 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
 }
 
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
-                        const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd, void* stream) {
+                        const float* stats, const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd,
+                        void* stream) {
   if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V || ldd < V) return fail(LCE_E_ARG, "bad shape");
   if (R == 0) return LCE_OK;
@@ -605,9 +606,9 @@ int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, 
   constexpr int NT = 512;
   ProfScope prof(PC_LOGITS_BWD, st);
   if (dtype == LCE_DTYPE_BF16)
-    hipLaunchKernelGGL((logits_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, dlogprobs, dentropy, (bf16_t*)d_logits, ldd);
+    hipLaunchKernelGGL((logits_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, stats, dlogprobs, dentropy, (bf16_t*)d_logits, ldd);
   else
-    hipLaunchKernelGGL((logits_bwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, dlogprobs, dentropy, (float*)d_logits, ldd);
+    hipLaunchKernelGGL((logits_bwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, stats, dlogprobs, dentropy, (float*)d_logits, ldd);
   return check_launch("logits_bwd_kernel");
 }
 

@@ -666,12 +666,31 @@ __global__ void transpose_pad_kernel(const typename Cfg::TIN* in, int64_t ldi, i
 template <typename TIN>
 LCE_DEV float load_as_float(const TIN* p, int64_t i) { return (float)p[i]; }
 
+// A row is walked as [head | 16-byte vectors | tail]: `head` elements bring the pointer to a 16-byte
+// boundary, then every lane loads whole vectors (8 bf16 / 4 fp32), two per trip so that two loads
+// are in flight per lane.
+template <typename TIN>
+struct RowSplit {
+  static constexpr int N = 16 / (int)sizeof(TIN);
+  typedef typename VecOf<TIN, N>::type vec_t;
+  int64_t head, nvec, tail0;
+  LCE_DEV RowSplit(const TIN* row, int64_t V) {
+    const uint64_t mis = reinterpret_cast<uint64_t>(row) & 15;
+    head = (int64_t)(((16 - mis) & 15) / sizeof(TIN));
+    if (head > V) head = V;
+    nvec = (V - head) / N;
+    tail0 = head + nvec * N;
+  }
+};
+
+// per-row online (max, sum exp, sum z exp): the block leaves m = max, a = sum exp(z - m), b = sum z exp(z - m)
 template <typename TIN, int NT>
 LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, float* sh) {
-  // per-thread online (max, sum exp, sum z exp) in natural-log units scaled to base 2
+  typedef RowSplit<TIN> RS;
+  typedef typename RS::vec_t vec_t;
+  constexpr int N = RS::N;
   float tm = kNegBig, ta = 0.f, tb = 0.f;
-  for (int64_t v = threadIdx.x; v < V; v += NT) {
-    const float z = load_as_float(row, v);
+  auto add_one = [&](float z) {
     if (z > tm) {
       const float sc = fast_exp2((tm - z) * kLog2e);
       ta *= sc;
@@ -681,7 +700,40 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
     const float e = fast_exp2((z - tm) * kLog2e);
     ta += e;
     tb = __builtin_fmaf(z, e, tb);
+  };
+  auto add_vec = [&](const vec_t& v) {
+    float z[N];
+    float vm = (float)v[0];
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      z[e] = (float)v[e];
+      vm = fmaxf(vm, z[e]);
+    }
+    if (vm > tm) {  // one rescale per vector
+      const float sc = fast_exp2((tm - vm) * kLog2e);
+      ta *= sc;
+      tb *= sc;
+      tm = vm;
+    }
+    const float ntm2 = -tm * kLog2e;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      const float ex = fast_exp2(__builtin_fmaf(z[e], kLog2e, ntm2));
+      ta += ex;
+      tb = __builtin_fmaf(z[e], ex, tb);
+    }
+  };
+  const RS rs(row, V);
+  for (int64_t v = threadIdx.x; v < rs.head; v += NT) add_one(load_as_float(row, v));
+  const vec_t* vp = reinterpret_cast<const vec_t*>(row + rs.head);
+  int64_t i = threadIdx.x;
+  for (; i + NT < rs.nvec; i += 2 * NT) {
+    const vec_t v0 = vp[i], v1 = vp[i + NT];
+    add_vec(v0);
+    add_vec(v1);
   }
+  if (i < rs.nvec) add_vec(vp[i]);
+  for (int64_t v = rs.tail0 + threadIdx.x; v < V; v += NT) add_one(load_as_float(row, v));
   // wave reduce
   for (int off = 32; off > 0; off >>= 1) {
     const float m2 = __shfl_xor(tm, off), a2 = __shfl_xor(ta, off), b2 = __shfl_xor(tb, off);
@@ -704,9 +756,10 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
   __syncthreads();
 }
 
+// stats (optional, [R][2]): logsumexp and sum softmax * logit of each row, kept for the backward
 template <typename TIN, int NT>
 __global__ __launch_bounds__(NT) void logits_fwd_kernel(const TIN* logits, int64_t ldl, const int64_t* labels, int64_t V,
-                                                        float* logprobs, float* entropy) {
+                                                        float* logprobs, float* entropy, float* stats) {
   __shared__ float sh[3 * NT / 64];
   const int64_t r = blockIdx.x;
   const TIN* row = logits + r * ldl;
@@ -720,30 +773,75 @@ __global__ __launch_bounds__(NT) void logits_fwd_kernel(const TIN* logits, int64
       const float zy = (y >= 0 && y < V) ? load_as_float(row, y) : 0.f;
       logprobs[r] = zy - lse;
     }
+    if (stats) {
+      stats[2 * r] = lse;
+      stats[2 * r + 1] = b / a;
+    }
   }
 }
 
 template <typename TIN, int NT>
 __global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64_t ldl, const int64_t* labels, int64_t V,
-                                                        const float* g_lp, const float* g_ent, TIN* dl, int64_t ldd) {
+                                                        const float* stats, const float* g_lp, const float* g_ent, TIN* dl,
+                                                        int64_t ldd) {
+  typedef RowSplit<TIN> RS;
+  typedef typename RS::vec_t vec_t;
+  constexpr int N = RS::N;
   __shared__ float sh[3 * NT / 64];
   const int64_t r = blockIdx.x;
   const TIN* row = logits + r * ldl;
-  float m, a, b;
-  row_stats<TIN, NT>(row, V, m, a, b, sh);
-  const float lse2 = (m + logf(a)) * kLog2e;
-  const float eb = b / a;
+  float lse, eb;
+  if (stats) {
+    lse = stats[2 * r];
+    eb = stats[2 * r + 1];
+  } else {
+    float m, a, b;
+    row_stats<TIN, NT>(row, V, m, a, b, sh);
+    lse = m + logf(a);
+    eb = b / a;
+  }
+  const float lse2 = lse * kLog2e;
   const float glp = g_lp ? g_lp[r] : 0.f;
   const float gent = g_ent ? g_ent[r] : 0.f;
   const int64_t y = (g_lp && labels) ? labels[r] : -1;
   TIN* out = dl + r * ldd;
-  for (int64_t v = threadIdx.x; v < V; v += NT) {
+  // d = p * (-glp - gent * (z - eb)) = p * (c0 + c1 * z)
+  const float c0 = -glp + gent * eb, c1 = -gent;
+  auto one = [&](int64_t v) {
     const float z = load_as_float(row, v);
-    const float pr = fast_exp2(__builtin_fmaf(z, kLog2e, -lse2));
-    float d = pr * (-glp - gent * (z - eb));
+    float d = fast_exp2(__builtin_fmaf(z, kLog2e, -lse2)) * __builtin_fmaf(z, c1, c0);
     if (v == y) d += glp;
     out[v] = (TIN)d;
+  };
+  const RS rs(row, V);
+  const bool same = ((reinterpret_cast<uint64_t>(out) ^ reinterpret_cast<uint64_t>(row)) & 15) == 0;  // vector stores line up too
+  if (!same) {
+    for (int64_t v = threadIdx.x; v < V; v += NT) one(v);
+    return;
   }
+  for (int64_t v = threadIdx.x; v < rs.head; v += NT) one(v);
+  const vec_t* vp = reinterpret_cast<const vec_t*>(row + rs.head);
+  vec_t* op = reinterpret_cast<vec_t*>(out + rs.head);
+  auto vec = [&](int64_t i, const vec_t& v) {
+    vec_t o;
+    const int64_t v0 = rs.head + i * N;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      const float z = (float)v[e];
+      float d = fast_exp2(__builtin_fmaf(z, kLog2e, -lse2)) * __builtin_fmaf(z, c1, c0);
+      if (v0 + e == y) d += glp;
+      o[e] = (TIN)d;
+    }
+    op[i] = o;
+  };
+  int64_t i = threadIdx.x;
+  for (; i + NT < rs.nvec; i += 2 * NT) {
+    const vec_t a0 = vp[i], a1 = vp[i + NT];
+    vec(i, a0);
+    vec(i + NT, a1);
+  }
+  if (i < rs.nvec) vec(i, vp[i]);
+  for (int64_t v = rs.tail0 + threadIdx.x; v < V; v += NT) one(v);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -35,6 +35,8 @@ def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool):
     dev = logits.device
     lp = torch.empty((R,), device=dev, dtype=torch.float32) if want_logprobs else None
     ent = torch.empty((R,), device=dev, dtype=torch.float32) if want_entropy else None
+    # row statistics for the backward (it then needs one pass instead of two)
+    stats = torch.empty((R, 2), device=dev, dtype=torch.float32) if (torch.is_grad_enabled() and logits.requires_grad) else None
     y = None
     if want_logprobs:
         y = labels.reshape(-1).to(torch.int64).contiguous()
@@ -42,14 +44,14 @@ def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool):
     if R > 0:
         with torch.cuda.device(dev):
             rc = _abi.load().lce_logits_forward(
-                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, code, _abi.ptr(lp), _abi.ptr(ent),
+                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, code, _abi.ptr(lp), _abi.ptr(ent), _abi.ptr(stats),
                 _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_logits_forward")
-    return rows, y, lp, ent
+    return rows, y, lp, ent, stats
 
 
-def _logits_backward(rows, y, g_lp, g_ent, out_shape, out_dtype):
+def _logits_backward(rows, y, stats, g_lp, g_ent, out_shape, out_dtype):
     R, V = rows.shape
     dev = rows.device
     d = torch.empty((R, V), device=dev, dtype=rows.dtype)
@@ -58,8 +60,8 @@ def _logits_backward(rows, y, g_lp, g_ent, out_shape, out_dtype):
     if R > 0:
         with torch.cuda.device(dev):
             rc = _abi.load().lce_logits_backward(
-                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, _abi.dtype_code(rows.dtype), _abi.ptr(g_lp),
-                _abi.ptr(g_ent), d.data_ptr(), d.stride(0), _abi.current_stream(dev),
+                rows.data_ptr(), rows.stride(0), _abi.ptr(y), R, V, _abi.dtype_code(rows.dtype), _abi.ptr(stats),
+                _abi.ptr(g_lp), _abi.ptr(g_ent), d.data_ptr(), d.stride(0), _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_logits_backward")
     return d.reshape(out_shape).to(out_dtype)
@@ -68,29 +70,29 @@ def _logits_backward(rows, y, g_lp, g_ent, out_shape, out_dtype):
 class _LogprobsFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels):
-        rows, y, lp, _ = _logits_forward(logits, labels, True, False)
-        ctx.save_for_backward(rows, y)
+        rows, y, lp, _, stats = _logits_forward(logits, labels, True, False)
+        ctx.save_for_backward(rows, y, stats)
         ctx.shape, ctx.dtype = logits.shape, logits.dtype
         return lp.reshape(logits.shape[:-1]).to(logits.dtype)
 
     @staticmethod
     def backward(ctx, g):
-        rows, y = ctx.saved_tensors
-        return _logits_backward(rows, y, g, None, ctx.shape, ctx.dtype), None
+        rows, y, stats = ctx.saved_tensors
+        return _logits_backward(rows, y, stats, g, None, ctx.shape, ctx.dtype), None
 
 
 class _EntropyFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, out_dtype):
-        rows, _, _, ent = _logits_forward(logits, None, False, True)
-        ctx.save_for_backward(rows)
+        rows, _, _, ent, stats = _logits_forward(logits, None, False, True)
+        ctx.save_for_backward(rows, stats)
         ctx.shape, ctx.dtype = logits.shape, logits.dtype
         return ent.reshape(logits.shape[:-1]).to(out_dtype)
 
     @staticmethod
     def backward(ctx, g):
-        (rows,) = ctx.saved_tensors
-        return _logits_backward(rows, None, None, g, ctx.shape, ctx.dtype), None
+        rows, stats = ctx.saved_tensors
+        return _logits_backward(rows, None, stats, None, g, ctx.shape, ctx.dtype), None
 
 
 def logprobs_from_logits(logits, labels, inplace_backward=True):
