@@ -269,10 +269,10 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
   {
     ProfScope prof(PC_TRANSPOSE, st);
-    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)(L.vpad / 64), (unsigned)((H + 63) / 64)), dim3(256), 0,
+    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((L.vpad + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
                        st, W, ldw, V, H, Wt, L.ldWt, L.vpad);
     if ((rc = check_launch("transpose W"))) return rc;
-    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)(L.tpad / 64), (unsigned)((H + 63) / 64)), dim3(256), 0,
+    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)((L.tpad + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
                        st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
     if ((rc = check_launch("transpose h"))) return rc;
   }

@@ -270,6 +270,16 @@ struct KPerm {
     const int64_t i = l / 32, w = l % 32, hh = (w >> 2) & 1, r = (w >> 3) * 4 + (w & 3);
     return v - l + hh * 16 * Cfg::FM + i * 16 + r;
   }
+  // inverses: which token / vocabulary row sits at position u
+  static __host__ __device__ int64_t token_at(int64_t u) {
+    const int64_t l = u % GT;
+    return u - l + (l % Cfg::FN) * 32 + l / Cfg::FN;
+  }
+  static __host__ __device__ int64_t vocab_at(int64_t u) {
+    const int64_t l = u % GV;
+    const int64_t hh = l / (16 * Cfg::FM), rem = l % (16 * Cfg::FM), i = rem / 16, r = rem % 16;
+    return u - l + i * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+  }
 };
 
 template <typename T, int N>
@@ -632,30 +642,63 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
 
 // out[c][perm(r)] = in[r][c] for r < R, c < C; out has `ldo` columns, columns perm(r) with r in
 // [R, rpad) are zero-filled (rpad a multiple of the permutation's group).  PERM: 0 none,
-// 1 KPerm::token, 2 KPerm::vocab.  Grid: (rpad/64, ceil(C/64)), 256 threads.
+// 1 KPerm::token, 2 KPerm::vocab.  Grid: (ceil(rpad/128), ceil(C/64)), 256 threads; a workgroup moves
+// 128 rows x 64 columns through LDS with 16-byte loads and stores on both sides.
+// `in` rows and `out` rows must be 16-byte aligned (ldi, ldo, C multiples of 16 bytes).
 // With `rows` / `n_rows` (device), row r of the input is in[rows[r]] for r < *n_rows and R = *n_rows.
 template <typename Cfg, int PERM>
-__global__ void transpose_pad_kernel(const typename Cfg::TIN* in, int64_t ldi, int64_t R, int64_t C, typename Cfg::TIN* out,
-                                     int64_t ldo, int64_t rpad, const int* rows = nullptr, const int* n_rows = nullptr) {
+__global__ __launch_bounds__(256) void transpose_pad_kernel(const typename Cfg::TIN* in, int64_t ldi, int64_t R, int64_t C,
+                                                            typename Cfg::TIN* out, int64_t ldo, int64_t rpad,
+                                                            const int* rows = nullptr, const int* n_rows = nullptr) {
   typedef typename Cfg::TIN TIN;
-  __shared__ TIN tile[64][65];
-  const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  constexpr int N = 16 / (int)sizeof(TIN);   // elements per 16-byte vector
+  constexpr int RB = 128, CB = 64;
+  constexpr int PITCH = CB + (sizeof(TIN) == 2 ? 2 : 1);  // odd number of 32-bit words per tile row
+  static_assert(KPerm<Cfg>::GT <= RB && KPerm<Cfg>::GV <= RB && RB % KPerm<Cfg>::GT == 0 && RB % KPerm<Cfg>::GV == 0, "group size");
+  typedef typename VecOf<TIN, N>::type vec_t;
+  __shared__ TIN tile[RB][PITCH];
+  const int64_t r0 = (int64_t)blockIdx.x * RB, c0 = (int64_t)blockIdx.y * CB;
   if (n_rows) {
     R = *n_rows;
     if (r0 >= (R + 255) / 256 * 256) return;  // beyond the last K granule that any GEMM reads
   }
-  for (int i = ty; i < 64; i += 4) {
-    const int64_t r = r0 + i, c = c0 + tx;
-    const int64_t src = (rows && r < R) ? (int64_t)rows[r] : r;
-    tile[i][tx] = (r < R && c < C) ? in[src * ldi + c] : (TIN)0.f;
+  {
+    constexpr int LPR = CB / N;            // lanes per row
+    constexpr int RPP = 256 / LPR;         // rows per pass
+    const int lr = threadIdx.x / LPR, lc = (threadIdx.x % LPR) * N;
+#pragma unroll
+    for (int k = 0; k < RB / RPP; ++k) {
+      const int i = k * RPP + lr;
+      const int64_t r = r0 + i, c = c0 + lc;
+      vec_t v;
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[e] = (TIN)0.f;
+      if (r < R && c < C) {
+        const int64_t src = rows ? (int64_t)rows[r] : r;
+        v = *reinterpret_cast<const vec_t*>(in + src * ldi + c);
+      }
+#pragma unroll
+      for (int e = 0; e < N; ++e) tile[i][lc + e] = v[e];
+    }
   }
   __syncthreads();
-  for (int i = ty; i < 64; i += 4) {
-    const int64_t c = c0 + i, r = r0 + tx;
-    if (c < C && r < rpad) {
-      const int64_t pr = PERM == 1 ? KPerm<Cfg>::token(r) : (PERM == 2 ? KPerm<Cfg>::vocab(r) : r);
-      out[c * ldo + pr] = tile[tx][i];
+  {
+    constexpr int LPR = RB / N;            // lanes per output row segment
+    constexpr int CPP = 256 / LPR;         // output rows per pass
+    const int q = (threadIdx.x % LPR) * N, lc = threadIdx.x / LPR;
+#pragma unroll
+    for (int k = 0; k < CB / CPP; ++k) {
+      const int ci = k * CPP + lc;
+      const int64_t c = c0 + ci, u0 = r0 + q;
+      if (c >= C || u0 >= rpad) continue;
+      vec_t v;
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        const int64_t u = u0 + e;
+        const int64_t r = PERM == 1 ? KPerm<Cfg>::token_at(u) : (PERM == 2 ? KPerm<Cfg>::vocab_at(u) : u);
+        v[e] = tile[(int)(r - r0)][ci];
+      }
+      *reinterpret_cast<vec_t*>(out + c * ldo + u0) = v;
     }
   }
 }
