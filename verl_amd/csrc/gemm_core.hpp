@@ -326,7 +326,7 @@ struct TileMap {
   }
   // the same map over fewer row tiles (a count that only the device knows): its workgroups are the
   // first `total` ids of the grid that was sized for the full map, the others have nothing to do
-  __device__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, block_rows(rows), rows_fastest); }
+  __device__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, rows >= br ? br : block_rows(rows), rows_fastest); }
 
   __host__ __device__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
     TileMap t;
