@@ -24,8 +24,8 @@ PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
 # (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt); counters cannot be read from inside this process.
 MEASURED_TRAFFIC = {
     "qwen2.5-7b-head-T16384": {
-        "lce_bwd_chunk_kernel": 3962132 * 1024 * 2.0 + 1115442 * 1024 * 1.0,
-        "lce_fwd_kernel": 13898456 * 1024 * 2.0 + 460800 * 1024 * 1.0,
+        "lce_bwd_chunk_kernel": 3872942 * 1024 * 2.0 + 1115384 * 1024 * 1.0,
+        "lce_fwd_kernel": 13823881 * 1024 * 2.0 + 8184 * 1024 * 1.0,
     }
 }
 WORKLOADS = {
@@ -94,6 +94,7 @@ def main():
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
     ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
+    ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -111,6 +112,8 @@ def main():
         _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
     if args.split_backward:
         _abi.check(lib.lce_set_option(1, 1), "lce_set_option")
+    if args.dlogits_tokens_first:
+        _abi.check(lib.lce_set_option(2, 1), "lce_set_option")
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")

@@ -104,8 +104,10 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 int lce_set_variant(int variant);
 int lce_num_variants(void);
 /* Diagnostic options (process-wide).  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and
- * the two gradient GEMMs of a backward chunk as three kernels instead of one (for per-phase timing). */
-enum { LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1 };
+ * the two gradient GEMMs of a backward chunk as three kernels instead of one (for per-phase timing).
+ * LCE_OPT_DLOGITS_TOKENS_FIRST: order in which an XCD's consecutive blocks of d_logits tiles walk the
+ * chunk: -1 = chosen by size (default), 0 = along the vocabulary, 1 = along the tokens. */
+enum { LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1, LCE_OPT_DLOGITS_TOKENS_FIRST = 2 };
 int lce_set_option(int key, int64_t value);
 
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every kernel

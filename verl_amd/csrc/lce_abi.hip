@@ -19,6 +19,7 @@ namespace {
 thread_local char g_err[512] = "";
 int g_variant = 3;
 int g_split_bwd = 0;
+int g_ds_tokens_first = -1;  // -1: by size
   // diagnostic: launch the three sub-problems of a backward chunk separately
 
 int fail(int code, const char* fmt, ...) {
@@ -297,9 +298,12 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       d.rows = rows; d.n_rows = n_rows;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
-      // consecutive blocks of an XCD walk the vocabulary first: the token tiles' rows of `hidden`, the
-      // larger operand, stay in its L2 while W's chunk streams (measured 2% on the launch vs tokens first)
-      d.map = TileMap::make(ntt, nvt, block_rows(ntt), 0);
+      // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
+      // faster on the launch while `hidden` is small enough to stay in the memory-side cache next to the
+      // chunk's other operands (T=16384, H=3584: 117 MB), along the tokens is 2% faster beyond that
+      // (T=32768, H=4096 and T=65536, H=5120).
+      const int tokens_first = g_ds_tokens_first >= 0 ? g_ds_tokens_first : ((size_t)T * H * sizeof(TIN) > ((size_t)128 << 20));
+      d.map = TileMap::make(ntt, nvt, block_rows(ntt), tokens_first);
       p.n_ds = d.map.total;
     }
     if (c > 0) {
@@ -429,6 +433,7 @@ int lce_set_variant(int variant) {
 int lce_set_option(int key, int64_t value) {
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
+    case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
 }
