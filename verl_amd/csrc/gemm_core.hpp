@@ -40,6 +40,10 @@ struct Mma;
 template <>
 struct Mma<bf16_t> {
   static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
+#ifdef LCE_DBG_NO_MFMA
+    asm volatile("" ::"v"(a), "v"(b));  // keeps the operand reads alive
+    return;
+#endif
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
                                                   acc, 0, 0, 0);
   }
@@ -56,10 +60,15 @@ struct Mma<float> {
   }
 };
 
-template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_>
+// SPLIT_ (needs BM == BN): the ring holds NSTAGE_ HALF stages, one operand's slab each, in the order
+// A0 B0 A1 B1 A2 ...; with five of them a barrier still hands back one A and one B half per slab, but
+// the odd half lets the A operand of the slab after next stay in flight ACROSS the barrier, so half of
+// the loads get two barrier periods to land instead of one.
+template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0>
 struct GemmCfg {
   typedef TIN_ TIN;
   static constexpr int BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
+  static constexpr int SPLIT = SPLIT_;  // 0 whole stages; 1 split ring, A operand early; 2 split ring, B operand early
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NTHREADS = NW * 64;
@@ -72,13 +81,14 @@ struct GemmCfg {
   static constexpr int A_LOADS = BM / ROWS_PER_LOAD / NW;
   static constexpr int B_LOADS = BN / ROWS_PER_LOAD / NW;
   static constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int STAGE_BYTES = SPLIT ? A_BYTES : A_BYTES + B_BYTES;  // one ring slot
   static constexpr int LDS_BYTES = STAGE_BYTES * NSTAGE;
+  static_assert(!SPLIT || (BM == BN && NSTAGE == 5), "split ring: equal halves, five slots");
   static_assert(BKB == 128 || BKB == 64, "slab rows are 64 or 128 bytes");
   static_assert(BM % (ROWS_PER_LOAD * NW) == 0 && BN % (ROWS_PER_LOAD * NW) == 0, "tile/loader mismatch");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be whole 32x32 blocks");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-  static_assert(KSUB % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 4, "pipeline shape");
+  static_assert(KSUB % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 5, "pipeline shape");
 
   // XOR pattern applied to the chunk index of a row (uses row bits 0..3 only, so it is the same
   // for rows that differ by a multiple of 32).
@@ -137,7 +147,7 @@ struct GemmCore {
     const int r32 = lane & 31, hh = lane >> 5;
     const int x = (hh ^ Cfg::swz(r32)) * 16;
     a_rd = (uint32_t)((wave_m * Cfg::WM + r32) * Cfg::BKB + x);
-    b_rd = (uint32_t)(Cfg::A_BYTES + (wave_n * Cfg::WN + r32) * Cfg::BKB + x);
+    b_rd = (uint32_t)((Cfg::SPLIT ? 0 : Cfg::A_BYTES) + (wave_n * Cfg::WN + r32) * Cfg::BKB + x);
   }
 
   static constexpr int PER = Cfg::A_LOADS + Cfg::B_LOADS;  // wave-wide DMA loads per slab
@@ -159,48 +169,63 @@ struct GemmCore {
                                        (lptr_t)(sa + Cfg::A_BYTES + (j * Cfg::NW + wave) * 1024), 16, 0, 0);
     }
   }
+  // split ring: load j of one operand's half slab into ring slot `slot`
+  LCE_DEV void dma_half(char* lds, int slot, int64_t kbyte, bool is_b, int j) const {
+#ifdef LCE_DBG_NO_DMA
+    if (kbyte > 0) return;
+#endif
+    char* sa = lds + slot * Cfg::STAGE_BYTES + (j * Cfg::NW + wave) * 1024;
+    if (is_b) __builtin_amdgcn_global_load_lds((gptr_t)(b_base + kbyte + lb.voff[j]), (lptr_t)sa, 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)(a_base + kbyte + la.voff[j]), (lptr_t)sa, 16, 0, 0);
+  }
   LCE_DEV void issue_slab(char* lds, int stage, int64_t kbyte) const {
 #pragma unroll
     for (int i = 0; i < PER; ++i) dma_one(lds, stage, kbyte, i);
   }
 
   // one of the N_READS operand reads of k-substep kk, in the order a0, b0..b(FN-1), a1..a(FM-1)
-  LCE_DEV void read_one(const char* s, int kk, int idx, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
+  // (sa, sb: the ring slots holding the A and the B operand; the same pointer unless the ring is split)
+  LCE_DEV void read_one(const char* sa, const char* sb, int kk, int idx, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
 #ifdef LCE_DBG_NO_READS
     if (kk > 0) return;
 #endif
     const uint32_t ao = a_rd ^ (uint32_t)(kk * 32);
     const uint32_t bo = b_rd ^ (uint32_t)(kk * 32);
-    if (idx == 0) af[0] = *reinterpret_cast<const u32x4_t*>(s + ao);
-    else if (idx <= Cfg::FN) bf[idx - 1] = *reinterpret_cast<const u32x4_t*>(s + bo + (idx - 1) * 32 * Cfg::BKB);
-    else af[idx - Cfg::FN] = *reinterpret_cast<const u32x4_t*>(s + ao + (idx - Cfg::FN) * 32 * Cfg::BKB);
+    if (idx == 0) af[0] = *reinterpret_cast<const u32x4_t*>(sa + ao);
+    else if (idx <= Cfg::FN) bf[idx - 1] = *reinterpret_cast<const u32x4_t*>(sb + bo + (idx - 1) * 32 * Cfg::BKB);
+    else af[idx - Cfg::FN] = *reinterpret_cast<const u32x4_t*>(sa + ao + (idx - Cfg::FN) * 32 * Cfg::BKB);
   }
-  LCE_DEV void load_frags(const char* s, int kk, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
+  LCE_DEV void load_frags(const char* sa, const char* sb, int kk, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
 #pragma unroll
-    for (int i = 0; i < N_READS; ++i) read_one(s, kk, i, af, bf);
+    for (int i = 0; i < N_READS; ++i) read_one(sa, sb, kk, i, af, bf);
   }
 
   // One k-substep with a hand-placed instruction order (pinned by scheduling barriers): the MFMAs
   // of this substep, with the operand reads of the NEXT substep (from `s_next`, substep `kk_next`)
   // and, when DMA is set, the global->LDS loads of a future slab dealt out between them.
-  template <bool DMA>
+  // DMA: 0 none; 1 the loads of a whole stage (unsplit ring); 2 / 3 (split ring) loads [J0, J1) of a B / A half
+  template <int DMA, int J0 = 0, int J1 = 0>
   LCE_DEV void substep(f32x16_t (&acc)[Cfg::FM][Cfg::FN], const u32x4_t (&af)[Cfg::FM], const u32x4_t (&bf)[Cfg::FN],
-                       const char* s_next, int kk_next, u32x4_t (&af_n)[Cfg::FM], u32x4_t (&bf_n)[Cfg::FN],
-                       char* lds, int dma_stage, int64_t dma_kbyte) const {
+                       const char* sa_next, const char* sb_next, int kk_next, u32x4_t (&af_n)[Cfg::FM],
+                       u32x4_t (&bf_n)[Cfg::FN], char* lds, int dma_stage, int64_t dma_kbyte) const {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int b = 0; b < N_BLK; ++b) {
       Mma<TIN>::run(acc[b / Cfg::FN][b % Cfg::FN], af[b / Cfg::FN], bf[b % Cfg::FN]);
       // reads: spread over the first blocks, one read after every `rstep`-th MFMA
       constexpr int rstep = 1;
-      if ((b % rstep) == rstep - 1 && b / rstep < N_READS) read_one(s_next, kk_next, b / rstep, af_n, bf_n);
+      if ((b % rstep) == rstep - 1 && b / rstep < N_READS) read_one(sa_next, sb_next, kk_next, b / rstep, af_n, bf_n);
       if (N_BLK < N_READS && b == N_BLK - 1) {
 #pragma unroll
-        for (int r = N_BLK; r < N_READS; ++r) read_one(s_next, kk_next, r, af_n, bf_n);
+        for (int r = N_BLK; r < N_READS; ++r) read_one(sa_next, sb_next, kk_next, r, af_n, bf_n);
       }
-      if (DMA) {
+      if constexpr (DMA == 1) {
 #pragma unroll
         for (int d = b * PER / N_BLK; d < (b + 1) * PER / N_BLK; ++d) dma_one(lds, dma_stage, dma_kbyte, d);
+      } else if constexpr (DMA == 2 || DMA == 3) {
+        constexpr int NJ = J1 - J0;
+#pragma unroll
+        for (int d = b * NJ / N_BLK; d < (b + 1) * NJ / N_BLK; ++d) dma_half(lds, dma_stage, dma_kbyte, DMA == 2, J0 + d);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -216,6 +241,16 @@ struct GemmCore {
   LCE_DEV void prologue(char* lds, int64_t K) const {
     const int nk = (int)(K / Cfg::BK);
     const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
+    if constexpr (Cfg::SPLIT) {
+      // half slabs 0..3 = E0 L0 E1 L1 (E: the early operand) into slots 0..3
+#pragma unroll
+      for (int hf = 0; hf < 4; ++hf) {
+        const int64_t kb = (int64_t)(hf / 2) * Cfg::BKB;
+#pragma unroll
+        for (int j = 0; j < Cfg::A_LOADS; ++j) dma_half(lds, hf, kb < last_kbyte ? kb : last_kbyte, (hf & 1) == (Cfg::SPLIT == 1), j);
+      }
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < Cfg::NSTAGE; ++s) {
       const int64_t kb = (int64_t)s * Cfg::BKB;
@@ -231,6 +266,10 @@ struct GemmCore {
   // The K loop proper; prologue() must have been called for this tile (no other vector memory
   // loads may have been issued by this wave in between: the waits count outstanding loads).
   LCE_DEV void main(char* lds, int64_t K, f32x16_t (&acc)[Cfg::FM][Cfg::FN]) const {
+    if constexpr (Cfg::SPLIT) {
+      main_split(lds, K, acc);
+      return;
+    }
     constexpr int NS = Cfg::NSTAGE, KSUB = Cfg::KSUB;
     const int nk = (int)(K / Cfg::BK);
     const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
@@ -243,7 +282,7 @@ struct GemmCore {
     wait_vm<(NS - 1) * PER>();
     __builtin_amdgcn_s_barrier();
     u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];
-    load_frags(lds, 0, af[0], bf[0]);
+    load_frags(lds, lds, 0, af[0], bf[0]);
     int stage = 0;
     int64_t kb_next = (int64_t)NS * Cfg::BKB;
 #ifdef LCE_DBG_TIMING
@@ -256,7 +295,7 @@ struct GemmCore {
       const char* s = lds + stage * Cfg::STAGE_BYTES;
 #pragma unroll
       for (int kk = 0; kk < KSUB - 1; ++kk) {
-        substep<false>(acc, af[kk & 1], bf[kk & 1], s, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1], lds, 0, 0);
+        substep<0>(acc, af[kk & 1], bf[kk & 1], s, s, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1], lds, 0, 0);
       }
       // last substep of this slab: its fragments are in registers, so this wave is done with the stage
       const int nstage = stage + 1 == NS ? 0 : stage + 1;
@@ -279,10 +318,91 @@ struct GemmCore {
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of the stage have returned
       __builtin_amdgcn_s_barrier();
 #endif
-      substep<true>(acc, af[(KSUB - 1) & 1], bf[(KSUB - 1) & 1], lds + nstage * Cfg::STAGE_BYTES, 0, af[0], bf[0], lds,
-                    stage, kb_next < last_kbyte ? kb_next : last_kbyte);
+      substep<1>(acc, af[(KSUB - 1) & 1], bf[(KSUB - 1) & 1], lds + nstage * Cfg::STAGE_BYTES,
+                    lds + nstage * Cfg::STAGE_BYTES, 0, af[0], bf[0], lds, stage, kb_next < last_kbyte ? kb_next : last_kbyte);
       kb_next += Cfg::BKB;
       stage = nstage;
+    }
+    wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
+#ifdef LCE_DBG_TIMING
+    if (lane == 0 && (wave == 0 || wave == Cfg::NW - 1)) {
+      const uint64_t t_end = __builtin_amdgcn_s_memtime();
+      unsigned long long* d = lce_dbg_times + (wave == 0 ? 0 : 8);
+      atomicAdd(d + 0, (unsigned long long)dbg_compute);
+      atomicAdd(d + 1, (unsigned long long)dbg_vm);
+      atomicAdd(d + 2, (unsigned long long)dbg_bar);
+      atomicAdd(d + 3, (unsigned long long)(t_end - dbg_t0));
+      atomicAdd(d + 4, (unsigned long long)nk);
+    }
+#endif
+  }
+
+  // K loop over the split ring.  One operand is "early" (E: A with SPLIT = 1, B with SPLIT = 2), the
+  // other "late" (L).  Slab i reads E(i) from slot (2i) % 5 and L(i) from slot (2i+1) % 5.  While slab i
+  // computes, its first two k-substeps issue the loads of E(i+2) into the slot that L(i-1) left
+  // (slot (2i+4) % 5); after the barrier that ends slab i, its last substep issues L(i+2) into E(i)'s
+  // slot.  The barrier needs E(i+1), L(i+1): everything except the youngest A_LOADS loads, E(i+2),
+  // which stay in flight across it.  So the burst after the barrier is half as long and half of the
+  // loads get two barrier periods to land.  Measured against the 2-stage ring of whole slabs: the
+  // load-only loop drops from 1.37 to 1.10 ms (16384 x 16384 x 3584), the full GEMM from 1.59 to 1.54.
+  LCE_DEV void main_split(char* lds, int64_t K, f32x16_t (&acc)[Cfg::FM][Cfg::FN]) const {
+    constexpr int KSUB = Cfg::KSUB, HL = Cfg::A_LOADS;
+    constexpr bool A_EARLY = Cfg::SPLIT == 1;
+    constexpr int EARLY = A_EARLY ? 3 : 2, LATE = A_EARLY ? 2 : 3;  // substep DMA modes: 3 loads an A half, 2 a B half
+    static_assert(Cfg::A_LOADS == Cfg::B_LOADS && KSUB == 4 && HL % 2 == 0, "equal halves, four k-substeps");
+    const int nk = (int)(K / Cfg::BK);
+    const int64_t last_kbyte = (int64_t)(nk - 1) * Cfg::BKB;
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    wait_vm<2 * HL>();  // E0, L0 have landed
+    __builtin_amdgcn_s_barrier();
+    u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];
+    load_frags(lds + (A_EARLY ? 0 : Cfg::STAGE_BYTES), lds + (A_EARLY ? Cfg::STAGE_BYTES : 0), 0, af[0], bf[0]);
+    int sa = 0;  // slot of this slab's early half; the late half is in the next slot
+#ifdef LCE_DBG_TIMING
+    uint64_t dbg_compute = 0, dbg_vm = 0, dbg_bar = 0;
+    uint64_t dbg_last = __builtin_amdgcn_s_memtime();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    const uint64_t dbg_t0 = dbg_last;
+#endif
+    for (int it = 0; it < nk; ++it) {
+      const int sb = sa + 1 >= 5 ? sa + 1 - 5 : sa + 1;
+      const int na = sa + 2 >= 5 ? sa + 2 - 5 : sa + 2;
+      const int nb = sa + 3 >= 5 ? sa + 3 - 5 : sa + 3;
+      const int fa = sa + 4 >= 5 ? sa + 4 - 5 : sa + 4;  // free slot: takes E(it+2)
+      const char* pa = lds + (A_EARLY ? sa : sb) * Cfg::STAGE_BYTES;
+      const char* pb = lds + (A_EARLY ? sb : sa) * Cfg::STAGE_BYTES;
+      const int64_t kb2 = (int64_t)(it + 2) * Cfg::BKB;
+      const int64_t kb = kb2 < last_kbyte ? kb2 : last_kbyte;
+      substep<EARLY, 0, HL / 2>(acc, af[0], bf[0], pa, pb, 1, af[1], bf[1], lds, fa, kb);
+      substep<EARLY, HL / 2, HL>(acc, af[1], bf[1], pa, pb, 2, af[0], bf[0], lds, fa, kb);
+      substep<0>(acc, af[0], bf[0], pa, pb, 3, af[1], bf[1], lds, 0, 0);
+#ifdef LCE_DBG_TIMING
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      const uint64_t t1 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      wait_vm<HL>();
+      const uint64_t t2 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();
+      const uint64_t t3 = __builtin_amdgcn_s_memtime();
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      dbg_compute += t1 - dbg_last;
+      dbg_vm += t2 - t1;
+      dbg_bar += t3 - t2;
+      dbg_last = t3;
+#else
+      wait_vm<HL>();                       // slab it+1 has landed; E(it+2) may still be in flight
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of both slots have returned
+      __builtin_amdgcn_s_barrier();
+#endif
+      substep<LATE, 0, HL>(acc, af[1], bf[1], lds + (A_EARLY ? na : nb) * Cfg::STAGE_BYTES, lds + (A_EARLY ? nb : na) * Cfg::STAGE_BYTES, 0,
+                           af[0], bf[0], lds, sa, kb);
+      sa = na;
     }
     wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
 #ifdef LCE_DBG_TIMING

@@ -17,7 +17,8 @@ using namespace lce;
 namespace {
 
 thread_local char g_err[512] = "";
-int g_variant = 3;
+constexpr int kDefaultVariant = 2;
+int g_variant = kDefaultVariant;
 int g_split_bwd = 0;
 int g_ds_tokens_first = -1;  // -1: by size
   // diagnostic: launch the three sub-problems of a backward chunk separately
@@ -67,8 +68,8 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // tile configurations of the mainloop, selectable for tuning
 //            TIN     BM   BN   BKB NSTAGE WAVES_M WAVES_N
 template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 2, 2, 2> Cfg; };
-template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 64, 4, 2, 2> Cfg; };
-template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 64, 4, 4, 2> Cfg; };
+template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 1> Cfg; };  // split ring of five half stages, A early
+template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 2> Cfg; };  // split ring of five half stages, B early
 template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };
 template <typename TIN> struct Variant4 { typedef GemmCfg<TIN, 256, 128, 128, 3, 2, 2> Cfg; };
 constexpr int kNumVariants = 5;
@@ -426,8 +427,8 @@ int lce_abi_version(void) { return LCE_ABI_VERSION; }
 const char* lce_last_error(void) { return g_err; }
 int lce_num_variants(void) { return kNumVariants; }
 int lce_set_variant(int variant) {
-  if (variant < 0 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
-  g_variant = variant;
+  if (variant < -1 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
+  g_variant = variant < 0 ? kDefaultVariant : variant;
   return LCE_OK;
 }
 int lce_set_option(int key, int64_t value) {
