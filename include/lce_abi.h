@@ -100,8 +100,8 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
 int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
                 int64_t K, int dtype, int variant, void* stream);
 
-/* Tuning hook: selects the tile / LDS-ring configuration used by the mainloops, 0 <= variant <
- * lce_num_variants(); -1 restores the default.  Process-wide. */
+/* Tuning hook: selects the tile / LDS-ring configuration used by the mainloops of forward and backward,
+ * 0 <= variant < lce_num_variants(); -1 restores the defaults (which differ between the two).  Process-wide. */
 int lce_set_variant(int variant);
 int lce_num_variants(void);
 /* Diagnostic options (process-wide).  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and

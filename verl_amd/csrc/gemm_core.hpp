@@ -279,7 +279,7 @@ struct GemmCore {
       for (int j = 0; j < Cfg::FN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    wait_vm<(NS - 1) * PER>();
+    wait_vm<Cfg::SPLIT ? 0 : (NS - 1) * PER>();  // (the split ring has its own loop; this body is still instantiated)
     __builtin_amdgcn_s_barrier();
     u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];
     load_frags(lds, lds, 0, af[0], bf[0]);
@@ -303,7 +303,7 @@ struct GemmCore {
       __builtin_amdgcn_s_waitcnt(0xC07F);
       const uint64_t t1 = __builtin_amdgcn_s_memtime();
       __builtin_amdgcn_s_waitcnt(0xC07F);
-      wait_vm<(NS - 2) * PER>();
+      wait_vm<Cfg::SPLIT ? 0 : (NS - 2) * PER>();
       const uint64_t t2 = __builtin_amdgcn_s_memtime();
       __builtin_amdgcn_s_waitcnt(0xC07F);
       __builtin_amdgcn_s_barrier();
@@ -314,7 +314,7 @@ struct GemmCore {
       dbg_bar += t3 - t2;
       dbg_last = t3;
 #else
-      wait_vm<(NS - 2) * PER>();           // slab it+1 has landed (only the younger slabs may be in flight)
+      wait_vm<Cfg::SPLIT ? 0 : (NS - 2) * PER>();  // slab it+1 has landed (only the younger slabs may be in flight)
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of the stage have returned
       __builtin_amdgcn_s_barrier();
 #endif

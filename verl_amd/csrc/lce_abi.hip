@@ -17,8 +17,10 @@ using namespace lce;
 namespace {
 
 thread_local char g_err[512] = "";
-constexpr int kDefaultVariant = 2;
-int g_variant = kDefaultVariant;
+// Defaults: the backward's long-K GEMMs gain 3% from the split ring; the forward does not and fetches
+// twice as much through the fabric with it (the XCD's workgroups drift apart and lose L2 sharing).
+constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2;
+int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 int g_split_bwd = 0;
 int g_ds_tokens_first = -1;  // -1: by size
   // diagnostic: launch the three sub-problems of a backward chunk separately
@@ -67,7 +69,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // tile configurations of the mainloop, selectable for tuning
 //            TIN     BM   BN   BKB NSTAGE WAVES_M WAVES_N
-template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 2, 2, 2> Cfg; };
+template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 5, 2, 2, 2> Cfg; };  // 4 waves of 128x128, split ring
 template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 1> Cfg; };  // split ring of five half stages, A early
 template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 2> Cfg; };  // split ring of five half stages, B early
 template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };
@@ -428,7 +430,8 @@ const char* lce_last_error(void) { return g_err; }
 int lce_num_variants(void) { return kNumVariants; }
 int lce_set_variant(int variant) {
   if (variant < -1 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
-  g_variant = variant < 0 ? kDefaultVariant : variant;
+  g_variant_fwd = variant < 0 ? kDefaultVariantFwd : variant;
+  g_variant_bwd = variant < 0 ? kDefaultVariantBwd : variant;
   return LCE_OK;
 }
 int lce_set_option(int key, int64_t value) {
@@ -493,7 +496,7 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
     return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
   char* ws = static_cast<char*>(workspace);
 #define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st)
-  switch (g_variant) {
+  switch (g_variant_fwd) {
     case 1: return LCE_FWD(Variant1);
     case 2: return LCE_FWD(Variant2);
     case 3: return LCE_FWD(Variant3);
@@ -530,7 +533,7 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
     return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, lce_backward_workspace_bytes(T, H, V, dtype, vchunk));
   char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
 #define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st)
-  switch (g_variant) {
+  switch (g_variant_bwd) {
     case 1: return LCE_BWD(Variant1);
     case 2: return LCE_BWD(Variant2);
     case 3: return LCE_BWD(Variant3);
