@@ -2,8 +2,9 @@
 //
 // Both operands are K-contiguous in memory ("NT" GEMM).  One workgroup owns a BM x BN tile of C;
 // its waves are arranged WAVES_M x WAVES_N and each wave owns (BM/WAVES_M) x (BN/WAVES_N) as
-// 32x32 MFMA blocks.  K is streamed in slabs of BKB bytes per row through an NSTAGE-deep LDS ring
-// that is filled by direct global->LDS loads (16 bytes per lane, no VGPR staging).
+// 32x32 MFMA blocks.  K is streamed in slabs of BKB bytes per row through an LDS ring that is filled
+// by direct global->LDS loads (16 bytes per lane, no VGPR staging): NSTAGE whole slabs, or NSTAGE half
+// slabs (one operand each) in the split layout described at GemmCfg.
 //
 // LDS layout of one operand slab: row-major, BKB bytes per row, the 16-byte chunk index of every
 // row XOR-ed with a function of the row number so that the 16-byte MFMA operand reads of 32
@@ -201,7 +202,7 @@ struct GemmCore {
   }
 
   // One k-substep with a hand-placed instruction order (pinned by scheduling barriers): the MFMAs
-  // of this substep, with the operand reads of the NEXT substep (from `s_next`, substep `kk_next`)
+  // of this substep, with the operand reads of the NEXT substep (from `sa_next` / `sb_next`, substep `kk_next`)
   // and, when DMA is set, the global->LDS loads of a future slab dealt out between them.
   // DMA: 0 none; 1 the loads of a whole stage (unsplit ring); 2 / 3 (split ring) loads [J0, J1) of a B / A half
   template <int DMA, int J0 = 0, int J1 = 0>
