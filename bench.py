@@ -84,12 +84,90 @@ def cpu_baseline(seconds_budget: float = 20.0):
     }
 
 
+PEAK_HBM = 8e12  # MI355X HBM3E peak, bytes/s
+
+LOGITS_WORKLOADS = {
+    # name: (rows, vocabulary): logits that already exist in HBM, bf16
+    "logits-twins-R8192-V152064": (8192, 152064),
+}
+
+
+def run_logits_workload(args, name):
+    """The unfused twins on given logits (logprobs_from_logits + entropy_from_logits): HBM-bound row
+    reductions; one step = both forward passes and both backward passes over one [R, V] bf16 tensor."""
+    import torch
+
+    from verl_amd import _abi
+    from verl_amd.utils import torch_functional as F
+
+    lib = _abi.load()
+    dev = torch.device("cuda:0")
+    R, V = LOGITS_WORKLOADS[name]
+    g = torch.Generator(device=dev).manual_seed(1234 + 6)
+    z = (torch.randn(R, V, device=dev, generator=g) * 3).bfloat16().requires_grad_(True)
+    y = torch.randint(0, V, (R,), device=dev, generator=g)
+    g_lp = torch.randn(R, device=dev, generator=g).bfloat16()
+    g_ent = torch.randn(R, device=dev, generator=g).bfloat16()
+
+    def step():
+        z.grad = None
+        lp = F.logprobs_from_logits(z, y)
+        ent = F.entropy_from_logits(z)
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    lib.lce_profile_enable(1)
+    _abi.profile_read(reset=True)
+    nprof = max(2, min(args.steps, 5))
+    for _ in range(nprof):
+        step()
+    torch.cuda.synchronize()
+    prof = _abi.profile_read(reset=True)
+    lib.lce_profile_enable(0)
+    kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
+    # algorithmic bytes per launch: forward reads the logits once; backward reads them once and writes d_logits once
+    bytes_per_launch = {"logits_fwd_kernel": R * V * 2.0, "logits_bwd_kernel": 2.0 * R * V * 2.0}
+    for k, v in kernels.items():
+        if k in bytes_per_launch:
+            v["achieved_GBps"] = bytes_per_launch[k] / (v["avg_ms"] * 1e-3) / 1e9
+    dom = max((k for k in kernels if k in bytes_per_launch), key=lambda k: kernels[k]["ms_per_step"])
+    achieved = bytes_per_launch[dom] / (kernels[dom]["avg_ms"] * 1e-3)
+    out = {
+        "metric": "rows/s, logprobs_from_logits + entropy_from_logits forward and backward on given logits",
+        "value": R / (elapsed / args.steps),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": name, "R": R, "V": V, "pass": "2 x fwd + 2 x bwd (+ torch's accumulation of the two d_logits)"},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": achieved / PEAK_HBM, "traffic": None, "avg_launch_ms": kernels[dom]["avg_ms"],
+                     "bytes_per_launch": bytes_per_launch[dom]},
+        "kernels": kernels,
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS) + sorted(LOGITS_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
@@ -101,6 +179,9 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload in LOGITS_WORKLOADS:
+        run_logits_workload(args, args.workload)
+        return
 
     import torch
 

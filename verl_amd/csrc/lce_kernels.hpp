@@ -289,8 +289,9 @@ struct VecOf<float, N> { typedef float type __attribute__((ext_vector_type(N)));
 template <int N>
 struct VecOf<bf16_t, N> { typedef bf16_t type __attribute__((ext_vector_type(N))); };
 
-// store N consecutive elements (N * sizeof(T) <= 16 bytes per store; wider runs are split)
-template <typename T, int N>
+// store N consecutive elements (N * sizeof(T) <= 16 bytes per store; wider runs are split);
+// STREAM: non-temporal stores, for data that this kernel does not read back
+template <typename T, int N, bool STREAM = false>
 LCE_DEV void store_run(T* dst, const float (&v)[N]) {
   constexpr int PER = (16 / (int)sizeof(T)) < N ? (16 / (int)sizeof(T)) : N;
   typedef typename VecOf<T, PER>::type vec_t;
@@ -299,7 +300,8 @@ LCE_DEV void store_run(T* dst, const float (&v)[N]) {
     vec_t out;
 #pragma unroll
     for (int e = 0; e < PER; ++e) out[e] = (T)v[k + e];
-    *reinterpret_cast<vec_t*>(dst + k) = out;
+    if (STREAM) __builtin_nontemporal_store(out, reinterpret_cast<vec_t*>(dst + k));
+    else *reinterpret_cast<vec_t*>(dst + k) = out;
   }
 }
 
@@ -698,7 +700,7 @@ __global__ __launch_bounds__(256) void transpose_pad_kernel(const typename Cfg::
         const int64_t r = PERM == 1 ? KPerm<Cfg>::token_at(u) : (PERM == 2 ? KPerm<Cfg>::vocab_at(u) : u);
         v[e] = tile[(int)(r - r0)][ci];
       }
-      *reinterpret_cast<vec_t*>(out + c * ldo + u0) = v;
+      __builtin_nontemporal_store(v, reinterpret_cast<vec_t*>(out + c * ldo + u0));  // read back only by later launches
     }
   }
 }
@@ -875,15 +877,17 @@ __global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64
       if (v0 + e == y) d += glp;
       o[e] = (TIN)d;
     }
-    op[i] = o;
+    __builtin_nontemporal_store(o, &op[i]);  // written once, never re-read by this kernel
   };
   int64_t i = threadIdx.x;
-  for (; i + NT < rs.nvec; i += 2 * NT) {
-    const vec_t a0 = vp[i], a1 = vp[i + NT];
+  for (; i + 3 * NT < rs.nvec; i += 4 * NT) {  // four loads in flight per lane
+    const vec_t a0 = vp[i], a1 = vp[i + NT], a2 = vp[i + 2 * NT], a3 = vp[i + 3 * NT];
     vec(i, a0);
     vec(i + NT, a1);
+    vec(i + 2 * NT, a2);
+    vec(i + 3 * NT, a3);
   }
-  if (i < rs.nvec) vec(i, vp[i]);
+  for (; i < rs.nvec; i += NT) vec(i, vp[i]);
   for (int64_t v = rs.tail0 + threadIdx.x; v < V; v += NT) one(v);
 }
 
