@@ -17,10 +17,12 @@ using namespace lce;
 namespace {
 
 thread_local char g_err[512] = "";
-// Defaults: the backward's long-K GEMMs gain 3% from the split ring; the forward does not and fetches
-// twice as much through the fabric with it (the XCD's workgroups drift apart and lose L2 sharing).
+// Defaults: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it only up
+// to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed
+// (the XCD's workgroups drift apart and lose L2 sharing), so large forwards keep the 2-stage ring.
 constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2;
 int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
+bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
 int g_split_bwd = 0;
 int g_ds_tokens_first = -1;  // -1: by size
   // diagnostic: launch the three sub-problems of a backward chunk separately
@@ -73,6 +75,9 @@ template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 5,
 template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 1> Cfg; };  // split ring of five half stages, A early
 template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 2> Cfg; };  // split ring of five half stages, B early
 template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };
+// forward with few tokens (one pass over W, HBM-bound): narrow token tiles leave LDS for a deeper ring
+template <typename TIN> struct VariantT64 { typedef GemmCfg<TIN, 256, 64, 128, 4, 4, 2> Cfg; };
+template <typename TIN> struct VariantT128 { typedef GemmCfg<TIN, 256, 128, 128, 3, 4, 2> Cfg; };
 template <typename TIN> struct Variant4 { typedef GemmCfg<TIN, 256, 128, 128, 3, 2, 2> Cfg; };
 constexpr int kNumVariants = 5;
 
@@ -161,7 +166,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
 // upper bound of the number of vocabulary splits forward_impl picks, over the token-tile widths in use
 int forward_splits_upper_bound(int64_t T) {
   int best = 1;
-  for (int bn = 128; bn <= 256; bn <<= 1) {
+  for (int bn = 64; bn <= 256; bn <<= 1) {
     const int ntt = (int)((T + bn - 1) / bn);
     const int br = block_rows(ntt), bc = 32 / br, nrb = (ntt + br - 1) / br;
     const int S = bc * ((8 + nrb - 1) / nrb);
@@ -430,6 +435,7 @@ const char* lce_last_error(void) { return g_err; }
 int lce_num_variants(void) { return kNumVariants; }
 int lce_set_variant(int variant) {
   if (variant < -1 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
+  g_variant_forced = variant >= 0;
   g_variant_fwd = variant < 0 ? kDefaultVariantFwd : variant;
   g_variant_bwd = variant < 0 ? kDefaultVariantBwd : variant;
   return LCE_OK;
@@ -496,6 +502,10 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
     return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
   char* ws = static_cast<char*>(workspace);
 #define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st)
+  if (!g_variant_forced && T <= 64) return LCE_FWD(VariantT64);
+  if (!g_variant_forced && T <= 128) return LCE_FWD(VariantT128);
+  if (!g_variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
+  if (!g_variant_forced && T <= 8192) return LCE_FWD(Variant2);  // measured 4-7% faster than the 2-stage ring up to here, equal beyond
   switch (g_variant_fwd) {
     case 1: return LCE_FWD(Variant1);
     case 2: return LCE_FWD(Variant2);
