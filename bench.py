@@ -29,7 +29,7 @@ MEASURED_TRAFFIC = {
     }
 }
 WORKLOADS = {
-    # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step)
+    # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step[, forward only])
     # `sequences` > 0: T is that many equally long rows, each with a valid prefix of U{shortest..row}
     # tokens; the upstream gradients are zero on the masked suffix (as a PPO response mask gives them).
     "qwen2.5-7b-head-T16384": (16384, 3584, 152064, 1.0, 0.02, 0, 0, False),
@@ -38,6 +38,8 @@ WORKLOADS = {
     # one actor micro-step: forward, clipped PPO loss (eps 0.2, dual clip 3.0, token-mean) with entropy
     # bonus 1e-3, backward; the loss kernel produces the upstream gradients
     "llama3-8b-actor-step-T262144": (262144, 4096, 128256, 1.0, 0.02, 64, 256, True),
+    # log-prob pass with few tokens: one streaming read of W, HBM-bound
+    "qwen2.5-7b-head-T64-fwd": (64, 3584, 152064, 1.0, 0.02, 0, 0, False, True),
     "small": (2048, 1024, 32768, 1.0, 0.02, 0, 0, False),
 }
 
@@ -198,7 +200,8 @@ def main():
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
-    T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload]
+    T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload][:8]
+    fwd_only = len(WORKLOADS[args.workload]) > 8 and WORKLOADS[args.workload][8]
     g = torch.Generator(device=dev).manual_seed(1234 + 2)
     h = torch.randn(T, H, device=dev, generator=g).bfloat16().requires_grad_(True)
     w = (torch.randn(V, H, device=dev, generator=g) * wstd).bfloat16().requires_grad_(True)
@@ -232,6 +235,10 @@ def main():
     def step():
         h.grad = None
         w.grad = None
+        if fwd_only:
+            with torch.no_grad():
+                linear_cross_entropy(h, w, y, tau, "none")
+            return
         lp, ent = linear_cross_entropy(h, w, y, tau, "none")
         if ppo:
             loss, _ = fused_ppo_loss(lp, ent, old_lp, adv, mask, clip_ratio=0.2, clip_ratio_c=3.0, entropy_coeff=1e-3)
@@ -276,6 +283,24 @@ def main():
     for k, v in kernels.items():
         if k in executed:
             v["executed_tflops"] = executed[k] * V * H / (v["ms_per_step"] * 1e-3) / 1e12
+    if fwd_only:
+        # one pass over W: the HBM roofline bounds it
+        k = kernels["lce_fwd_kernel"]
+        nbytes = (V * H + T * H) * 2.0
+        out = {
+            "metric": "tokens/s, forward (log-prob + entropy) with few tokens; % of HBM peak",
+            "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic",
+            "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
+            "roofline": {"bound": "hbm", "kernel": "lce_fwd_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
+                         "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM, "traffic": None,
+                         "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes},
+            "kernels": kernels,
+            "cpu_baseline": None,
+        }
+        print(json.dumps(out), flush=True)
+        return
     roofline = {
         "bound": "mfma",
         "kernel": dom,

@@ -150,8 +150,15 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   if (rc) return rc;
   {
     ProfScope prof(PC_FWD_MERGE, st);
-    hipLaunchKernelGGL(lce_fwd_merge_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T, p.c,
-                       1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
+    if (S >= 64)
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+                         p.c, 1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
+    else if (S >= 8)
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+                         p.c, 1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
+    else
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T, p.c,
+                         1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
     rc = check_launch("lce_fwd_merge_kernel");
   }
   if (rc) return rc;

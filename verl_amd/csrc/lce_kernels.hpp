@@ -178,19 +178,31 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
   }
 }
 
-// merge the S partials of every token and emit the five per-token outputs
+// merge the S partials of every token and emit the five per-token outputs; LANES (a power of two up
+// to 64) threads share a token: each merges every LANES-th partial, then a fixed shuffle tree joins
+// them (with few tokens there are hundreds of splits per token and only a handful of tokens)
+template <int LANES>
 __global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, int S, int64_t T, float c, float rcp_tau,
                                      float* logprobs, float* entropy, float* maximum, float* accumulate,
                                      float* entropy_b) {
-  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
-  const f32x4_t v0 = parts[t];
-  float vm = v0[0], va = v0[1], vb = v0[2];
-  const float vz = xlabel[t];
-  for (int s = 1; s < S; ++s) {
-    const f32x4_t u = parts[(int64_t)s * T + t];
-    merge_stats(vm, va, vb, u[0], u[1], u[2], c);
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t t = gid / LANES;
+  const int sub = (int)(gid % LANES);
+  const bool live = t < T;
+  float vm = kNegBig, va = 0.f, vb = 0.f;
+  if (live) {
+    for (int s = sub; s < S; s += LANES) {
+      const f32x4_t u = parts[(int64_t)s * T + t];
+      merge_stats(vm, va, vb, u[0], u[1], u[2], c);
+    }
   }
+#pragma unroll
+  for (int off = LANES / 2; off > 0; off >>= 1) {
+    const float m2 = __shfl_xor(vm, off), a2 = __shfl_xor(va, off), b2 = __shfl_xor(vb, off);
+    merge_stats(vm, va, vb, m2, a2, b2, c);
+  }
+  if (!live || sub != 0) return;
+  const float vz = xlabel[t];
   const float mz = vm * rcp_tau;
   const float lse = mz + logf(va);
   const float eb = (vb / va) * rcp_tau;
