@@ -1,0 +1,93 @@
+"""Direct calls of the C ABI (no Python wrapper in between): row strides larger than H, a workspace
+placed at an odd offset, error codes for bad arguments on the device, and a non-default stream."""
+
+import pytest
+import torch
+
+from oracle import lce_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _call(lib, _abi, h, ldh, w, ldw, y, T, H, V, dtype, tau, g_lp, g_ent, stream, vchunk=0, ws_shift=0):
+    code = _abi.dtype_code(dtype)
+    f32 = dict(device=DEV, dtype=torch.float32)
+    lp, ent, mx, acc, eb = (torch.empty(T, **f32) for _ in range(5))
+    nf = lib.lce_forward_workspace_bytes(T, H, V, code)
+    ws = torch.empty(nf + 256, device=DEV, dtype=torch.uint8)
+    rc = lib.lce_forward(h.data_ptr(), ldh, w.data_ptr(), ldw, y.data_ptr(), T, H, V, code, tau, 0, lp.data_ptr(), ent.data_ptr(),
+                         mx.data_ptr(), acc.data_ptr(), eb.data_ptr(), ws.data_ptr(), nf, stream)
+    _abi.check(rc, "lce_forward")
+    dh = torch.empty(T, H, device=DEV, dtype=dtype)
+    dw = torch.empty(V, H, device=DEV, dtype=dtype)
+    nb = lib.lce_backward_workspace_bytes(T, H, V, code, vchunk)
+    wsb = torch.empty(nb + 512, device=DEV, dtype=torch.uint8)
+    rc = lib.lce_backward(h.data_ptr(), ldh, w.data_ptr(), ldw, y.data_ptr(), T, H, V, code, tau, 0, mx.data_ptr(), acc.data_ptr(),
+                          eb.data_ptr(), g_lp.data_ptr(), g_ent.data_ptr(), dh.data_ptr(), dw.data_ptr(),
+                          wsb.data_ptr() + ws_shift, nb, vchunk, stream)
+    _abi.check(rc, "lce_backward")
+    return lp, ent, dh, dw
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_padded_row_strides_side_stream_and_shifted_workspace(dtype):
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V, tau = 333, 256, 3001, 0.7
+    pad_h, pad_w = 64, 8
+    g = torch.Generator().manual_seed(5)
+    hbuf = (torch.rand(T, H + pad_h, generator=g) - 0.5).to(dtype).to(DEV)
+    wbuf = (torch.rand(V, H + pad_w, generator=g) - 0.5).to(dtype).to(DEV)
+    h, w = hbuf[:, :H], wbuf[:, :H]
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = (torch.rand(T, generator=g) * 2 - 1).to(DEV)
+    g_ent = (torch.rand(T, generator=g) - 0.5).to(DEV)
+    side = torch.cuda.Stream(device=DEV)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        lp, ent, dh, dw = _call(lib, _abi, hbuf, H + pad_h, wbuf, H + pad_w, y, T, H, V, dtype, tau, g_lp, g_ent, side.cuda_stream,
+                                vchunk=1024, ws_shift=16)
+    side.synchronize()
+    if dtype == torch.float32:
+        rlp, rent = O.lce_forward(h, w, y, tau, compute_dtype=torch.float64)
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+        for got, want in ((lp, rlp), (ent, rent), (dh, rdh), (dw, rdw)):
+            err = (got.double() - want).abs().max().item()
+            assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
+    else:
+        rlp, rent = O.lce_forward(h, w, y, tau)
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+        torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+        torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+        torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+        torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
+def test_error_codes_leave_the_device_untouched():
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V = 8, 128, 100
+    h = torch.zeros(T, H, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(V, H, device=DEV, dtype=torch.bfloat16)
+    y = torch.zeros(T, device=DEV, dtype=torch.int64)
+    out = torch.full((5, T), 7.0, device=DEV)
+    ws = torch.empty(lib.lce_forward_workspace_bytes(T, H, V, 0), device=DEV, dtype=torch.uint8)
+    st = _abi.current_stream(torch.device(DEV))
+    args = lambda **kw: [kw.get("h", h.data_ptr()), kw.get("ldh", H), w.data_ptr(), kw.get("ldw", H), y.data_ptr(), T, H, V, 0,
+                         kw.get("tau", 1.0), kw.get("red", 0), out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr(),
+                         out[3].data_ptr(), out[4].data_ptr(), ws.data_ptr(), kw.get("nws", ws.numel()), st]
+    assert lib.lce_forward(*args(ldh=H - 8)) == -1           # row stride shorter than a row
+    assert lib.lce_forward(*args(ldw=H + 3)) == -1           # row stride not a multiple of 16 bytes
+    assert lib.lce_forward(*args(h=h.data_ptr() + 2)) == -1  # misaligned pointer
+    assert lib.lce_forward(*args(tau=0.0)) == -1
+    assert lib.lce_forward(*args(red=9)) == -1
+    assert lib.lce_forward(*args(nws=16)) == -2              # workspace too small
+    assert b"workspace" in lib.lce_last_error()
+    torch.cuda.synchronize()
+    assert (out == 7.0).all()
+    assert lib.lce_forward(*args()) == 0
+    torch.cuda.synchronize()
+    assert not (out == 7.0).any()
