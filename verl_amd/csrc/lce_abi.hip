@@ -512,7 +512,10 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
   if (!g_variant_forced && T <= 64) return LCE_FWD(VariantT64);
   if (!g_variant_forced && T <= 128) return LCE_FWD(VariantT128);
   if (!g_variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
-  if (!g_variant_forced && T <= 8192) return LCE_FWD(Variant2);  // measured 4-7% faster than the 2-stage ring up to here, equal beyond
+  // the split ring: measured 4-7% faster than the 2-stage ring up to 8192 tokens, equal (+-1%) beyond, and
+  // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
+  if (!g_variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * (dtype == LCE_DTYPE_BF16 ? 2 : 4) > (512ull << 20)))
+    return LCE_FWD(Variant2);
   switch (g_variant_fwd) {
     case 1: return LCE_FWD(Variant1);
     case 2: return LCE_FWD(Variant2);
