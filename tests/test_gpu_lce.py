@@ -234,6 +234,23 @@ def test_config2_full_size_properties_and_sampled_parity():
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2) and torch.equal(dh, dh2) and torch.equal(dw, dw2)
 
 
+def test_wide_hidden_and_256k_vocabulary():
+    """H = 8192 and V = 262144 (the largest vocabularies in use): 4.3 GB of weights, row offsets beyond
+    2^31 bytes inside W, 128 K-slabs per logit tile; a quarter of the tokens without gradient."""
+    T, H, V, tau = 2048, 8192, 262144, 0.9
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.01, seed=1241)
+    keep = (torch.arange(T, device=DEV) % 4) != 3
+    g_lp, g_ent = g_lp * keep, g_ent * keep
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau, chunk=512)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, chunk=512)
+    torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+    torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+    assert_bf16_bar(dh, rdh)
+    assert_bf16_bar(dw, rdw)
+    assert (dh[~keep] == 0).all()
+
+
 def test_config3_masked_rows_temperature_06():
     """Llama-3-8B-shaped head, tau = 0.6, a response mask zeroing a random suffix of each row
     (reduced token count; upstream gradients are zero on masked positions)."""
