@@ -23,9 +23,8 @@ thread_local char g_err[512] = "";
 constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2;
 int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
-int g_split_bwd = 0;
-int g_ds_tokens_first = -1;  // -1: by size
-  // diagnostic: launch the three sub-problems of a backward chunk separately
+int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
+int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
