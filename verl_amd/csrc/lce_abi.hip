@@ -216,7 +216,7 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   L.vpad = round_up(V, gv);
   L.ldS = vchunk + 64;
   L.ldST = L.tpad + 64;
-  L.ldWt = L.vpad + 64;
+  L.ldWt = vchunk + 64;  // one chunk of W^T at a time
   L.ldHt = L.tpad + 64;
   size_t o = 0;
   // the d_logits pair is double buffered when there is more than one chunk: chunk c is produced
@@ -240,15 +240,15 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
 
 // vchunk <= 0 picks the default chunk width: as wide as possible (fewer, longer launches) while the
 // whole workspace stays below a quarter of one [T, V] tile plus one fp32 [V, H],
-//   8*T*vc*esz/2 + esz*V*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
-// and no wider than 16384 columns or, with few tokens, than what gives the d_logits pass 512 tiles.
+//   8*T*vc*esz/2 + esz*vc*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
+// and no wider than 32768 columns or, with few tokens, than what gives the d_logits pass 512 tiles.
 // gt, gv: K-permutation groups that tokens / vocabulary are rounded up to (at most one workgroup
 // tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
 BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
     const double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
     const int64_t ntt = (T + 255) / 256;
-    vchunk = ntt >= 8 ? 16384 : 512 * 256 / ntt;
+    vchunk = ntt >= 8 ? 32768 : 512 * 256 / ntt;
     while (vchunk > 2048 && (double)bwd_layout_for(T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
   }
   return bwd_layout_for(T, H, V, esz, vchunk, gt, gv);
@@ -281,12 +281,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                        (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), dentropy, T, rows, inv, n_rows);
     if ((rc = check_launch("active_rows_kernel"))) return rc;
   }
-  // K-contiguous copies of the second operands of the two gradient GEMMs: W^T [H][V], h^T [H][T]
+  // K-contiguous copy of the d_weight GEMM's second operand: h^T [H][T] (W^T follows chunk by chunk)
   {
     ProfScope prof(PC_TRANSPOSE, st);
-    hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((L.vpad + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
-                       st, W, ldw, V, H, Wt, L.ldWt, L.vpad);
-    if ((rc = check_launch("transpose W"))) return rc;
     hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)((L.tpad + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
                        st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
     if ((rc = check_launch("transpose h"))) return rc;
@@ -324,9 +321,16 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int cc = c - 1;
       const int64_t v0 = (int64_t)cc * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
-      // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . Wt[H][v0 : v0 + Kc]^T  (rows = listed tokens)
+      // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . Wt[H][Kc]^T  (rows = listed tokens), Wt = this chunk of W,
+      // transposed just before the launch (the previous launch, the last reader of the buffer, is complete by then)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
-      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt + v0, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+      {
+        ProfScope prof(PC_TRANSPOSE, st);
+        hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((kc + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
+                           st, W + v0 * ldw, ldw, vrows, H, Wt, L.ldWt, kc);
+        if ((rc = check_launch("transpose W"))) return rc;
+      }
+      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
       p.gh.m_dev = n_rows;
       if (L.ksplit > 1) {
         p.gh.ksplit = L.ksplit;
