@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 2
+#define LCE_ABI_VERSION 3
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -64,6 +64,32 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
                  const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                  void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
                  void* stream);
+
+/* Vocabulary-parallel building blocks: what one rank of a tensor-parallel lm-head runs on its shard
+ * W[vocab_offset : vocab_offset + V_local, :] of the vocabulary.  The exchange between the ranks (an
+ * all-gather of the partials, a sum of d_hidden) is the caller's.  Replaces the per-rank part of the
+ * reference's tensor-parallel branch: the mainloop matching labels against `rank * vocab_size`
+ * (verl/utils/kernel/kernels.py:328, :343-344), its all-reduced statistics and TP epilogue (:444-566, :705-757)
+ * and the backward's label mask with the same offset (:1503).  labels are GLOBAL vocabulary ids.
+ *   lce_forward_shard: partials [T, 4] fp32 = per token (max logit, sum exp(logit - max),
+ *     sum logit * exp(logit - max), label logit or 0 if the label is not in the shard), logits = h.w / temperature.
+ *     Workspace as lce_forward_workspace_bytes(T, H, V_local, dtype).
+ *   lce_merge_shards: partials [R, T, 4] (shard-major, e.g. straight out of an all-gather) -> the five outputs of
+ *     lce_forward for the whole vocabulary, merged in the fixed order r = 0..R-1.  Workspace: 4*T bytes for
+ *     reduction sum / mean, else unused.
+ *   lce_backward_shard: as lce_backward with the merged statistics; d_weight_shard [V_local, H] is complete,
+ *     d_hidden_partial [T, H] is this shard's contribution (the ranks' partials add up to d_hidden).
+ *     Workspace as lce_backward_workspace_bytes(T, H, V_local, dtype, vchunk). */
+int lce_forward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
+                      int64_t H, int64_t V_local, int64_t vocab_offset, int dtype, float temperature, float* partials,
+                      void* workspace, size_t workspace_bytes, void* stream);
+int lce_merge_shards(const float* partials, int R, int64_t T, int reduction, float* logprobs, float* entropy, float* maximum,
+                     float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes, void* stream);
+int lce_backward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
+                       int64_t H, int64_t V_local, int64_t vocab_offset, int dtype, float temperature, int reduction,
+                       const float* maximum, const float* accumulate, const float* entropy_b, const float* dlogprobs,
+                       const float* dentropy, void* d_hidden_partial, void* d_weight_shard, void* workspace,
+                       size_t workspace_bytes, int64_t vchunk, void* stream);
 
 /* Unfused twins on logits that already exist in memory.
  * Replaces logprobs_from_logits (verl/utils/torch_functional.py:73-107, :155-207) and

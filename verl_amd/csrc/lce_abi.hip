@@ -120,7 +120,10 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                  int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* logprobs, float* entropy,
-                 float* maximum, float* accumulate, float* entropy_b, char* ws, hipStream_t st) {
+                 float* maximum, float* accumulate, float* entropy_b, char* ws, hipStream_t st, int64_t label_offset = 0,
+                 float* shard_out = nullptr) {
+  // shard_out: W is one shard of a larger vocabulary starting at row label_offset; instead of the five
+  // outputs the per-token partial (max, sum exp, sum logit*exp, label logit) goes to shard_out [T][4]
   typedef typename Cfg::TIN TIN;
   const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
   const int nvt = (int)((V + Cfg::BM - 1) / Cfg::BM);
@@ -135,6 +138,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.parts = reinterpret_cast<f32x4_t*>(ws);
   p.xlabel = reinterpret_cast<float*>(ws + align256((size_t)S * T * 16));
   p.S = S; p.nvt = nvt;
+  p.label_offset = label_offset;
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
   allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
@@ -147,6 +151,20 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
     rc = check_launch("lce_fwd_kernel");
   }
   if (rc) return rc;
+  if (shard_out) {
+    ProfScope prof(PC_FWD_MERGE, st);
+    f32x4_t* out = reinterpret_cast<f32x4_t*>(shard_out);
+    if (S >= 64)
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S,
+                         T, p.c, 1.0f / temperature, out);
+    else if (S >= 8)
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+                         p.c, 1.0f / temperature, out);
+    else
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+                         p.c, 1.0f / temperature, out);
+    return check_launch("lce_fwd_shard_merge_kernel");
+  }
   {
     ProfScope prof(PC_FWD_MERGE, st);
     if (S >= 64)
@@ -258,7 +276,9 @@ template <typename Cfg>
 int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                   int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
                   const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
-                  typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st) {
+                  typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st,
+                  int64_t vocab_offset = 0) {
+  // vocab_offset: W is the shard [vocab_offset, vocab_offset + V) of a larger vocabulary (labels are global ids)
   typedef typename Cfg::TIN TIN;
   const BwdLayout L = bwd_layout(T, H, V, sizeof(TIN), vchunk, KPerm<Cfg>::GT, KPerm<Cfg>::GV);
   TIN* dS[2] = {reinterpret_cast<TIN*>(ws + L.off_dS[0]), reinterpret_cast<TIN*>(ws + L.off_dS[1])};
@@ -301,7 +321,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
       DsArgs<TIN>& d = p.ds;
       d.W = W + v0 * ldw; d.ldw = ldw; d.h = h; d.ldh = ldh; d.labels = labels; d.T = T; d.H = H;
-      d.v0 = v0; d.vrows = vrows; d.rcp_tau = 1.0f / temperature; d.c = kLog2e / temperature;
+      d.v0 = vocab_offset + v0; d.vrows = vrows; d.rcp_tau = 1.0f / temperature; d.c = kLog2e / temperature;
       d.maximum = maximum; d.accumulate = accumulate; d.entropy_b = entropy_b;
       d.g_lp = dlogprobs; d.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
       d.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
@@ -381,24 +401,26 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
 template <template <typename> class Vt>
 int dispatch_dtype_forward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
                            int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* lp, float* ent,
-                           float* mx, float* ac, float* eb, char* ws, hipStream_t st) {
+                           float* mx, float* ac, float* eb, char* ws, hipStream_t st, int64_t label_offset = 0,
+                           float* shard_out = nullptr) {
   if (dtype == LCE_DTYPE_BF16)
     return forward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
-                                                  reduction, lp, ent, mx, ac, eb, ws, st);
+                                                  reduction, lp, ent, mx, ac, eb, ws, st, label_offset, shard_out);
   return forward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
-                                               reduction, lp, ent, mx, ac, eb, ws, st);
+                                               reduction, lp, ent, mx, ac, eb, ws, st, label_offset, shard_out);
 }
 
 template <template <typename> class Vt>
 int dispatch_dtype_backward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
                             int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* mx,
                             const float* ac, const float* eb, const float* glp, const float* gent, void* dh, void* dw,
-                            char* ws, int64_t vchunk, hipStream_t st) {
+                            char* ws, int64_t vchunk, hipStream_t st, int64_t vocab_offset = 0) {
   if (dtype == LCE_DTYPE_BF16)
     return backward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
-                                                   reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st);
+                                                   reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st,
+                                                   vocab_offset);
   return backward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
-                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st);
+                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st, vocab_offset);
 }
 
 template <template <typename> class Vt>
@@ -493,25 +515,26 @@ size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
   return align256((size_t)forward_splits_upper_bound(T) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
 }
 
-int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
-                int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
-                float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
-                void* stream) {
+// shared body of lce_forward and lce_forward_shard
+static int forward_entry(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                         int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                         float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                         void* stream, int64_t label_offset, float* shard_out) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if (T == 0) {
-    if (reduction != LCE_REDUCTION_NONE && logprobs) {
+    if (!shard_out && reduction != LCE_REDUCTION_NONE && logprobs) {
       hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t*>(logprobs), (int64_t)1);
       return check_launch("fill_zero_kernel");
     }
     return LCE_OK;
   }
-  if (!logprobs || !entropy || !maximum || !accumulate || !entropy_b) return fail(LCE_E_ARG, "null output pointer");
+  if (!shard_out && (!logprobs || !entropy || !maximum || !accumulate || !entropy_b)) return fail(LCE_E_ARG, "null output pointer");
   if (!workspace || workspace_bytes < lce_forward_workspace_bytes(T, H, V, dtype))
     return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
   char* ws = static_cast<char*>(workspace);
-#define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st)
+#define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st, label_offset, shard_out)
   if (!g_variant_forced && T <= 64) return LCE_FWD(VariantT64);
   if (!g_variant_forced && T <= 128) return LCE_FWD(VariantT128);
   if (!g_variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
@@ -529,16 +552,64 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
 #undef LCE_FWD
 }
 
+int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                void* stream) {
+  return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
+                       accumulate, entropy_b, workspace, workspace_bytes, stream, 0, nullptr);
+}
+
+int lce_forward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
+                      int64_t H, int64_t V_local, int64_t vocab_offset, int dtype, float temperature, float* partials,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!partials && T > 0) return fail(LCE_E_ARG, "null partials pointer");
+  if (vocab_offset < 0) return fail(LCE_E_ARG, "vocab_offset must be >= 0");
+  return forward_entry(hidden, ldh, weight_shard, ldw, labels, T, H, V_local, dtype, temperature, LCE_REDUCTION_NONE, nullptr,
+                       nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, stream, vocab_offset, partials);
+}
+
+int lce_merge_shards(const float* partials, int R, int64_t T, int reduction, float* logprobs, float* entropy, float* maximum,
+                     float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes, void* stream) {
+  if (R <= 0 || T < 0) return fail(LCE_E_ARG, "bad shard count or token count");
+  if (reduction < 0 || reduction > 2) return fail(LCE_E_ARG, "Invalid reduction: %d", reduction);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (T == 0) {
+    if (reduction != LCE_REDUCTION_NONE && logprobs) {
+      hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<uint32_t*>(logprobs), (int64_t)1);
+      return check_launch("fill_zero_kernel");
+    }
+    return LCE_OK;
+  }
+  if (!partials || !logprobs || !entropy || !maximum || !accumulate || !entropy_b) return fail(LCE_E_ARG, "null pointer");
+  float* lp_tok = logprobs;
+  if (reduction != LCE_REDUCTION_NONE) {
+    if (!workspace || workspace_bytes < (size_t)T * 4) return fail(LCE_E_WORKSPACE, "merge workspace too small: need %zu bytes", (size_t)T * 4);
+    lp_tok = static_cast<float*>(workspace);
+  }
+  hipLaunchKernelGGL(lce_merge_shards_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<const f32x4_t*>(partials), R, T, lp_tok, entropy, maximum, accumulate, entropy_b);
+  int rc = check_launch("lce_merge_shards_kernel");
+  if (rc) return rc;
+  if (reduction != LCE_REDUCTION_NONE) {
+    const float scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
+    hipLaunchKernelGGL(lce_reduce_sum_kernel, dim3(1), dim3(1024), 0, st, lp_tok, T, scale, logprobs);
+    rc = check_launch("lce_reduce_sum_kernel");
+  }
+  return rc;
+}
+
 size_t lce_backward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype, int64_t vchunk) {
   if (T <= 0 || H <= 0 || V <= 0) return 256;
   return bwd_layout(T, H, V, dtype == LCE_DTYPE_BF16 ? 2 : 4, vchunk).total + 256;
 }
 
-int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
-                 int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
-                 const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
-                 void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
-                 void* stream) {
+// shared body of lce_backward and lce_backward_shard
+static int backward_entry(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                          int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                          const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                          void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                          void* stream, int64_t vocab_offset) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -555,7 +626,7 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
   if (!workspace || workspace_bytes < lce_backward_workspace_bytes(T, H, V, dtype, vchunk))
     return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, lce_backward_workspace_bytes(T, H, V, dtype, vchunk));
   char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
-#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st)
+#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st, vocab_offset)
   switch (g_variant_bwd) {
     case 1: return LCE_BWD(Variant1);
     case 2: return LCE_BWD(Variant2);
@@ -564,6 +635,26 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
     default: return LCE_BWD(Variant0);
   }
 #undef LCE_BWD
+}
+
+int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                 int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                 const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                 void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                 void* stream) {
+  return backward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, maximum, accumulate, entropy_b,
+                        dlogprobs, dentropy, d_hidden, d_weight, workspace, workspace_bytes, vchunk, stream, 0);
+}
+
+int lce_backward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
+                       int64_t H, int64_t V_local, int64_t vocab_offset, int dtype, float temperature, int reduction,
+                       const float* maximum, const float* accumulate, const float* entropy_b, const float* dlogprobs,
+                       const float* dentropy, void* d_hidden_partial, void* d_weight_shard, void* workspace,
+                       size_t workspace_bytes, int64_t vchunk, void* stream) {
+  if (vocab_offset < 0) return fail(LCE_E_ARG, "vocab_offset must be >= 0");
+  return backward_entry(hidden, ldh, weight_shard, ldw, labels, T, H, V_local, dtype, temperature, reduction, maximum, accumulate,
+                        entropy_b, dlogprobs, dentropy, d_hidden_partial, d_weight_shard, workspace, workspace_bytes, vchunk, stream,
+                        vocab_offset);
 }
 
 int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,

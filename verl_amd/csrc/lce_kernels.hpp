@@ -46,6 +46,7 @@ struct FwdArgs {
   int S;             // vocabulary splits; split s owns vocab tiles s, s+S, s+2S, ...
   int nvt;           // vocabulary tiles
   TileMap map;       // rows = token tiles, cols = splits
+  int64_t label_offset;  // W holds vocabulary rows [label_offset, label_offset + V) of a larger vocabulary (0 = all of it)
 };
 
 template <typename Cfg>
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       a[j] = 0.f;
       b[j] = 0.f;
       const int64_t t = n0 + wave_n * Cfg::WN + j * 32 + ln;
-      const int64_t y = t < p.T ? p.labels[t] : -1;
+      const int64_t y = t < p.T ? p.labels[t] - p.label_offset : -1;
       lab[j] = (y >= 0 && y < p.V) ? (int)y : -1;
     }
   }
@@ -213,6 +214,54 @@ __global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, 
   logprobs[t] = vz * rcp_tau - lse;
 }
 
+// Vocabulary-parallel building block: the same merge, but the result stays a partial for exchange
+// between the owners of the vocabulary shards: out[t] = (max logit, sum exp(logit - max),
+// sum logit * exp(logit - max), label logit or 0), in logit units (after the division by temperature).
+template <int LANES>
+__global__ void lce_fwd_shard_merge_kernel(const f32x4_t* parts, const float* xlabel, int S, int64_t T, float c, float rcp_tau,
+                                           f32x4_t* out) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t t = gid / LANES;
+  const int sub = (int)(gid % LANES);
+  const bool live = t < T;
+  float vm = kNegBig, va = 0.f, vb = 0.f;
+  if (live) {
+    for (int s = sub; s < S; s += LANES) {
+      const f32x4_t u = parts[(int64_t)s * T + t];
+      merge_stats(vm, va, vb, u[0], u[1], u[2], c);
+    }
+  }
+#pragma unroll
+  for (int off = LANES / 2; off > 0; off >>= 1) {
+    const float m2 = __shfl_xor(vm, off), a2 = __shfl_xor(va, off), b2 = __shfl_xor(vb, off);
+    merge_stats(vm, va, vb, m2, a2, b2, c);
+  }
+  if (!live || sub != 0) return;
+  const f32x4_t v = {vm * rcp_tau, va, vb * rcp_tau, xlabel[t] * rcp_tau};
+  out[t] = v;
+}
+
+// merges the partials of R vocabulary shards (shard-major [R][T]) in the fixed order r = 0, 1, ... and
+// emits the five per-token outputs
+__global__ void lce_merge_shards_kernel(const f32x4_t* partials, int R, int64_t T, float* logprobs, float* entropy,
+                                        float* maximum, float* accumulate, float* entropy_b) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  float vm = kNegBig, va = 0.f, vb = 0.f, vz = 0.f;
+  for (int r = 0; r < R; ++r) {
+    const f32x4_t u = partials[(int64_t)r * T + t];
+    merge_stats(vm, va, vb, u[0], u[1], u[2], kLog2e);
+    vz += u[3];  // the label lives in at most one shard; the others hold 0
+  }
+  const float lse = vm + logf(va);
+  const float eb = vb / va;
+  maximum[t] = vm;
+  accumulate[t] = va;
+  entropy_b[t] = eb;
+  entropy[t] = lse - eb;
+  logprobs[t] = vz - lse;
+}
+
 // deterministic single-workgroup sum of x[0..n) * scale -> out[0]
 __global__ void lce_reduce_sum_kernel(const float* x, int64_t n, float scale, float* out) {
   __shared__ double sh[1024];
@@ -239,7 +288,7 @@ struct DsArgs {
   int64_t ldh;
   const int64_t* labels;
   int64_t T, H;
-  int64_t v0;     // vocabulary index of the chunk's first row
+  int64_t v0;     // vocabulary index of the chunk's first row (global: labels are matched against v0 + row)
   int64_t vrows;  // valid rows in the chunk
   float c, rcp_tau;
   const float* maximum;
