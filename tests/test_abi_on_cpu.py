@@ -113,3 +113,14 @@ def test_fused_linear_for_ppo_constructor():
     m = FusedLinearForPPO(chunk_size=3)
     with pytest.raises(ValueError):
         m(torch.zeros(2, 3, 4, 8), torch.zeros(5, 8), torch.zeros(2, 3, 4, dtype=torch.long))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message instead of pretending."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr
