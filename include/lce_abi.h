@@ -126,6 +126,11 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
 int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
                 int64_t K, int dtype, int variant, void* stream);
 
+/* Diagnostic twin for K-major operands (bf16 only): C[M, N] = A[K, M]^T . B[K, N], the layout of the d_weight GEMM
+ * (A = d_logits [tokens, vocab], B = hidden [tokens, H]).  K a multiple of 64; lda >= M and ldb >= N rounded up to 256. */
+int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                void* stream);
+
 /* Tuning hook: selects the tile / LDS-ring configuration used by the mainloops of forward and backward,
  * 0 <= variant < lce_num_variants(); -1 restores the defaults (which differ between the two).  Process-wide. */
 int lce_set_variant(int variant);

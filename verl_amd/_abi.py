@@ -36,6 +36,7 @@ SYMBOLS = {
     "lce_ppo_loss_workspace_bytes": (_sz, [_i64]),
     "lce_ppo_loss": (_i, [_p, _p, _p, _p, _p, _i64, _f, _f, _f, _f, _f, _p, _p, _p, _p, _sz, _p]),
     "lce_gemm_nt": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _i, _p]),
+    "lce_gemm_tn": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),
     "lce_set_variant": (_i, [_i]),
     "lce_num_variants": (_i, []),
     "lce_set_option": (_i, [_i, _i64]),

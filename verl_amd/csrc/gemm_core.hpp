@@ -28,11 +28,25 @@ typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
 #define LCE_DEV __device__ __forceinline__
 
 typedef const void __attribute__((address_space(1))) * gptr_t;
 typedef void __attribute__((address_space(3))) * lptr_t;
+
+// transposing LDS read of four 16-bit elements per lane (see GemmCore::init_tn for the lane mapping).
+// Issued as inline assembly with a 32-bit LDS address: through the builtin the compiler waits for ALL
+// outstanding global->LDS loads before every such read (it cannot tell that they do not alias), which
+// serialises the ring.  The price: the compiler does not know that the result arrives later, so the
+// consumer places the lgkmcnt waits itself (GemmCore::substep).
+template <int OFF>
+LCE_DEV u32x2_t tr_read(uint32_t lds_addr) {
+  u32x2_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFF));
+  return v;
+}
 
 template <typename T>
 struct Mma;
@@ -65,11 +79,16 @@ struct Mma<float> {
 // A0 B0 A1 B1 A2 ...; with five of them a barrier still hands back one A and one B half per slab, but
 // the odd half lets the A operand of the slab after next stay in flight ACROSS the barrier, so half of
 // the loads get two barrier periods to land instead of one.
-template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0>
+// TRANS_ (split ring, 16-bit elements only): both operands are stored K-major in memory, A[k][m] and B[k][n]
+// (C = A^T . B); a ring slot holds 64 k-rows of 256 columns and the MFMA operand fragments are fetched with the
+// transposing LDS read (ds_read_b64_tr_b16, two per fragment).
+template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0, bool TRANS_ = false>
 struct GemmCfg {
   typedef TIN_ TIN;
   static constexpr int BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
   static constexpr int SPLIT = SPLIT_;  // 0 whole stages; 1 split ring, A operand early; 2 split ring, B operand early
+  static constexpr bool TRANS = TRANS_;
+  static_assert(!TRANS_ || (SPLIT_ != 0 && sizeof(TIN_) == 2 && BM_ == 256 && BN_ == 256 && BKB_ == 128), "transposed operands: split ring, 16-bit, 256x256");
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NTHREADS = NW * 64;
@@ -115,6 +134,7 @@ struct GemmCore {
   SlabLoader<Cfg::B_LOADS> lb;
   int wave, lane, wave_m, wave_n;
   uint32_t a_rd, b_rd;  // LDS byte offsets (within a stage) of this lane's operand rows, swizzle folded in
+  int64_t a_slab, b_slab;  // bytes from one K slab to the next in memory (BKB, or 64 rows for K-major operands)
 
   // rows beyond the matrix are clamped to its last row (their results are discarded by the epilogue).
   // With `b_rows` given, row n of the B operand is B[b_rows[n]] (a gather; B is then the matrix's first
@@ -127,6 +147,7 @@ struct GemmCore {
     wave_n = wave % Cfg::WAVES_N;
     a_base = reinterpret_cast<const char*>(A + m0 * lda);
     b_base = reinterpret_cast<const char*>(b_rows ? B : B + n0 * ldb);
+    a_slab = b_slab = Cfg::BKB;
     const int rows_a = (int)((M - m0) < (int64_t)Cfg::BM ? (M - m0) : (int64_t)Cfg::BM);
     const int rows_b = (int)((N - n0) < (int64_t)Cfg::BN ? (N - n0) : (int64_t)Cfg::BN);
     const int lr = lane / Cfg::CH, pc = lane % Cfg::CH;
@@ -149,6 +170,35 @@ struct GemmCore {
     const int x = (hh ^ Cfg::swz(r32)) * 16;
     a_rd = (uint32_t)((wave_m * Cfg::WM + r32) * Cfg::BKB + x);
     b_rd = (uint32_t)((Cfg::SPLIT ? 0 : Cfg::A_BYTES) + (wave_n * Cfg::WN + r32) * Cfg::BKB + x);
+  }
+
+  // K-major operands: A[k][m0 + 0..BM), B[k][n0 + 0..BN), row strides lda / ldb (elements).  A ring slot
+  // holds 64 k-rows x 512 bytes; the 16-byte chunk c of row r sits at chunk position c ^ ((r % 4) * 4), so the
+  // four rows that one transposing read touches fall into different banks.
+  LCE_DEV void init_tn(const TIN* A, int64_t lda, int64_t m0, const TIN* B, int64_t ldb, int64_t n0) {
+    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    lane = threadIdx.x & 63;
+    wave_m = wave / Cfg::WAVES_N;
+    wave_n = wave % Cfg::WAVES_N;
+    a_base = reinterpret_cast<const char*>(A + m0);
+    b_base = reinterpret_cast<const char*>(B + n0);
+    a_slab = 64 * lda * (int64_t)sizeof(TIN);
+    b_slab = 64 * ldb * (int64_t)sizeof(TIN);
+#pragma unroll
+    for (int j = 0; j < Cfg::A_LOADS; ++j) {
+      const int row = (j * Cfg::NW + wave) * 2 + lane / 32;  // one wave-wide load covers two 512-byte rows
+      const int c = (lane % 32) ^ ((row % 4) * 4);
+      la.voff[j] = (uint32_t)((int64_t)row * lda * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
+      lb.voff[j] = (uint32_t)((int64_t)row * ldb * (int64_t)sizeof(TIN)) + (uint32_t)(c * 16);
+    }
+    // transposing read: in each group of 16 lanes, lane 4e + q supplies the address of X[k0 + e][x0 + 4q ..]
+    // and lane i receives X[k0 .. k0+3][x0 + i]; groups 0/1 take the two 16-column halves of a 32-column
+    // block, groups 2/3 the upper half (k + 8) of the 16 k-values of a substep
+    const int g = lane / 16, e = (lane % 16) / 4, q = lane % 4;
+    const int ma = wave_m * Cfg::WM + 16 * (g % 2) + 4 * q, nb = wave_n * Cfg::WN + 16 * (g % 2) + 4 * q;
+    const uint32_t row_off = (uint32_t)((8 * (g / 2) + e) * 512);
+    a_rd = row_off + (uint32_t)((((ma / 8) ^ (4 * e)) * 16) + (ma % 8) * 2);
+    b_rd = row_off + (uint32_t)((((nb / 8) ^ (4 * e)) * 16) + (nb % 8) * 2);
   }
 
   static constexpr int PER = Cfg::A_LOADS + Cfg::B_LOADS;  // wave-wide DMA loads per slab
@@ -176,8 +226,10 @@ struct GemmCore {
     if (kbyte > 0) return;
 #endif
     char* sa = lds + slot * Cfg::STAGE_BYTES + (j * Cfg::NW + wave) * 1024;
-    if (is_b) __builtin_amdgcn_global_load_lds((gptr_t)(b_base + kbyte + lb.voff[j]), (lptr_t)sa, 16, 0, 0);
-    else __builtin_amdgcn_global_load_lds((gptr_t)(a_base + kbyte + la.voff[j]), (lptr_t)sa, 16, 0, 0);
+    // kbyte counts BKB bytes per slab; K-major operands advance by 64 rows per slab instead
+    const int64_t off = Cfg::TRANS ? (kbyte / Cfg::BKB) * (is_b ? b_slab : a_slab) : kbyte;
+    if (is_b) __builtin_amdgcn_global_load_lds((gptr_t)(b_base + off + lb.voff[j]), (lptr_t)sa, 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)(a_base + off + la.voff[j]), (lptr_t)sa, 16, 0, 0);
   }
   LCE_DEV void issue_slab(char* lds, int stage, int64_t kbyte) const {
 #pragma unroll
@@ -190,6 +242,22 @@ struct GemmCore {
 #ifdef LCE_DBG_NO_READS
     if (kk > 0) return;
 #endif
+    if constexpr (Cfg::TRANS) {
+      // block i of A / j of B: 32 columns further = 4 chunks = bit 6 / bits 6-7 of the byte offset, which the
+      // swizzle XORs; substep kk: 16 rows further; second half of the fragment: 4 rows further
+      const bool is_a = idx == 0 || idx > Cfg::FN;
+      const int blk = idx == 0 ? 0 : (idx <= Cfg::FN ? idx - 1 : idx - Cfg::FN);
+      const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(is_a ? sa : sb) + ((is_a ? a_rd : b_rd) ^ (uint32_t)(blk * 64));
+      u32x2_t lo, hi;
+      if (kk == 0) { lo = tr_read<0>(base); hi = tr_read<2048>(base); }
+      else if (kk == 1) { lo = tr_read<8192>(base); hi = tr_read<8192 + 2048>(base); }
+      else if (kk == 2) { lo = tr_read<16384>(base); hi = tr_read<16384 + 2048>(base); }
+      else { lo = tr_read<24576>(base); hi = tr_read<24576 + 2048>(base); }
+      const u32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
+      if (is_a) af[blk] = v;
+      else bf[blk] = v;
+      return;
+    }
     const uint32_t ao = a_rd ^ (uint32_t)(kk * 32);
     const uint32_t bo = b_rd ^ (uint32_t)(kk * 32);
     if (idx == 0) af[0] = *reinterpret_cast<const u32x4_t*>(sa + ao);
@@ -212,6 +280,21 @@ struct GemmCore {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int b = 0; b < N_BLK; ++b) {
+      if constexpr (Cfg::TRANS) {
+        // The operand reads are inline assembly (see tr_read), so the waits are placed by hand.  Reads are issued
+        // in the order a0, b0 .. b(FN-1), a1 .., two instructions each, one operand after each of the first MFMAs,
+        // and LDS reads return in order.  Before MFMA b of this substep, 2*min(b, N_READS) reads of the NEXT
+        // substep are in flight behind this substep's 2*N_READS; it needs its A block (b / FN) and B block (b % FN).
+        constexpr int ALL = 2 * N_READS;
+        const int ia = b / Cfg::FN, ib = b % Cfg::FN;
+        const int last = ia == 0 ? 1 + ib : N_READS - Cfg::FM + ia;  // index of the last operand read it depends on
+        const int done = 2 * (last + 1);
+        const int issued = 2 * (b < N_READS ? b : N_READS);
+        const int allow = (ALL - done) + issued;
+        static_assert(ALL <= 15, "lgkmcnt range");
+        wait_lgkm(allow);
+        __builtin_amdgcn_sched_barrier(0);  // the wait stays in front of the MFMA
+      }
       Mma<TIN>::run(acc[b / Cfg::FN][b % Cfg::FN], af[b / Cfg::FN], bf[b % Cfg::FN]);
       // reads: spread over the first blocks, one read after every `rstep`-th MFMA
       constexpr int rstep = 1;
@@ -417,6 +500,17 @@ struct GemmCore {
       atomicAdd(d + 4, (unsigned long long)nk);
     }
 #endif
+  }
+
+  // s_waitcnt lgkmcnt(n) only; n is a constant after unrolling, the switch folds away
+  static LCE_DEV void wait_lgkm(int n) {
+#define LCE_LGKM(N) case N: __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8)); break;
+    switch (n) {
+      LCE_LGKM(0) LCE_LGKM(1) LCE_LGKM(2) LCE_LGKM(3) LCE_LGKM(4) LCE_LGKM(5) LCE_LGKM(6) LCE_LGKM(7)
+      LCE_LGKM(8) LCE_LGKM(9) LCE_LGKM(10) LCE_LGKM(11) LCE_LGKM(12) LCE_LGKM(13) LCE_LGKM(14)
+      default: __builtin_amdgcn_s_waitcnt(0xC07F | (15 << 8)); break;
+    }
+#undef LCE_LGKM
   }
 
   template <int N>

@@ -674,6 +674,20 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 #undef LCE_GEMM
 }
 
+int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                void* stream) {
+  typedef GemmCfg<bf16_t, 256, 256, 128, 5, 4, 2, 2, true> Cfg;
+  if (!A || !B || !C || !aligned16(A) || !aligned16(B)) return fail(LCE_E_ARG, "bad pointer");
+  if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || lda % 8 != 0 || ldb % 8 != 0) return fail(LCE_E_ARG, "gemm_tn: bad shape");
+  if (lda < round_up(M, 256) || ldb < round_up(N, 256)) return fail(LCE_E_ARG, "gemm_tn: rows must be allocated in whole 256-column tiles");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  GemmArgs<bf16_t> p = make_gemm_args<Cfg>((const bf16_t*)A, lda, (const bf16_t*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0);
+  allow_lds(gemm_tn_kernel<Cfg>, Cfg::LDS_BYTES);
+  ProfScope prof(PC_GEMM_DW, st);
+  hipLaunchKernelGGL(gemm_tn_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  return check_launch("gemm_tn_kernel");
+}
+
 int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                        float* logprobs, float* entropy, float* stats, void* stream) {
   if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);

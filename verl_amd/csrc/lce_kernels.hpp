@@ -612,6 +612,29 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
 #undef LCE_EPI
 }
 
+// C[m][n] = sum_k A[k][m] * B[k][n]: both operands K-major (Cfg::TRANS); M, N whole tiles of the operands'
+// allocated width, K a multiple of 64
+template <typename Cfg>
+LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+  int tm, tn;
+  if (!p.map.decode(bid, tm, tn)) return;
+  const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
+  GemmCore<Cfg> g;
+  g.init_tn(p.A, p.lda, m0, p.B, p.ldb, n0);
+  f32x16_t acc[Cfg::FM][Cfg::FN];
+  g.run(lds, p.K, acc);
+  const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
+  if (edge) gemm_epilogue<Cfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  else gemm_epilogue<Cfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+}
+
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(GemmArgs<typename Cfg::TIN> p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  gemm_tn_tile<Cfg>(p, blockIdx.x, lds);
+}
+
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_ds_kernel(DsArgs<typename Cfg::TIN> p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
