@@ -175,6 +175,7 @@ def main():
     ap.add_argument("--vchunk", type=int, default=-1)
     ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
     ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
+    ap.add_argument("--no-transposed-reads", action="store_true", help="diagnostic: d_weight GEMM from a vocab-major copy of the d_logits")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -195,6 +196,8 @@ def main():
         _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
     if args.split_backward:
         _abi.check(lib.lce_set_option(1, 1), "lce_set_option")
+    if args.no_transposed_reads:
+        _abi.check(lib.lce_set_option(3, 0), "lce_set_option")
     if args.dlogits_tokens_first:
         _abi.check(lib.lce_set_option(2, 1), "lce_set_option")
     if args.vchunk >= 0:

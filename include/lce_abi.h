@@ -138,8 +138,11 @@ int lce_num_variants(void);
 /* Diagnostic options (process-wide).  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and
  * the two gradient GEMMs of a backward chunk as three kernels instead of one (for per-phase timing).
  * LCE_OPT_DLOGITS_TOKENS_FIRST: order in which an XCD's consecutive blocks of d_logits tiles walk the
- * chunk: -1 = chosen by size (default), 0 = along the vocabulary, 1 = along the tokens. */
-enum { LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1, LCE_OPT_DLOGITS_TOKENS_FIRST = 2 };
+ * chunk: -1 = chosen by size (default), 0 = along the vocabulary, 1 = along the tokens.
+ * LCE_OPT_DW_TRANSPOSED_READS (default 1, bf16 only): the d_weight GEMM reads the token-major d_logits with
+ * transposing LDS reads; 0 builds a second, vocab-major copy of the d_logits for it (changes the workspace size:
+ * set it before querying lce_backward_workspace_bytes). */
+enum { LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1, LCE_OPT_DLOGITS_TOKENS_FIRST = 2, LCE_OPT_DW_TRANSPOSED_READS = 3 };
 int lce_set_option(int key, int64_t value);
 
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every kernel

@@ -25,6 +25,7 @@ int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
 int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
 int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
+int g_dw_transposed_reads = 1;  // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -97,7 +98,7 @@ GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t l
   p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
   p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
   p.ksplit = 1; p.kslice = K; p.cf_split_stride = 0;
-  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1;
+  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1; p.tn = 0;
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   return p;
@@ -204,7 +205,13 @@ struct BwdLayout {
   size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, total;
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
+  bool tn;     // the d_weight GEMM reads dS (token-major) and a compact copy of hidden, both K-major: no dS^T, no h^T
 };
+
+// The d_weight GEMM can take the token-major d_logits and hidden as they are (transposing LDS reads exist
+// for 16-bit elements and are wired for the 8-wave 256 x 256 tile variants 1-3); otherwise a vocab-major copy of the
+// d_logits and a transposed hidden are built for it.
+bool dw_transposed_reads(size_t esz) { return esz == 2 && g_dw_transposed_reads && g_variant_bwd >= 1 && g_variant_bwd <= 3; }
 
 // The d_hidden GEMM has only ceil(T/256) * ceil(H/256) output tiles, each with a K loop as long as the
 // vocabulary chunk.  With few tokens one such tile takes longer than a CU's share of the whole launch
@@ -221,6 +228,7 @@ int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
 // layout for a given chunk width
 BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
   BwdLayout L;
+  L.tn = dw_transposed_reads(esz);
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
@@ -235,18 +243,18 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   L.ldS = vchunk + 64;
   L.ldST = L.tpad + 64;
   L.ldWt = vchunk + 64;  // one chunk of W^T at a time
-  L.ldHt = L.tpad + 64;
+  L.ldHt = L.tn ? round_up(H, 256) + 64 : L.tpad + 64;  // tn: row stride of the compact copy of hidden [tpad][.]
   size_t o = 0;
   // the d_logits pair is double buffered when there is more than one chunk: chunk c is produced
   // while the GEMMs of chunk c-1 consume the other pair
   for (int b = 0; b < 2; ++b) {
     L.off_dS[b] = o;
-    if (b == 0 || L.nchunks > 1) o += align256((size_t)T * L.ldS * esz);
+    if (b == 0 || L.nchunks > 1) o += align256((size_t)L.tpad * L.ldS * esz);
     L.off_dST[b] = o;
-    if (b == 0 || L.nchunks > 1) o += align256((size_t)vchunk * L.ldST * esz);
+    if (!L.tn && (b == 0 || L.nchunks > 1)) o += align256((size_t)vchunk * L.ldST * esz);
   }
   L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
-  L.off_Ht = o;    o += align256((size_t)H * L.ldHt * esz);
+  L.off_Ht = o;    o += L.tn ? align256((size_t)L.tpad * L.ldHt * esz) : align256((size_t)H * L.ldHt * esz);
   L.off_dHacc = o; o += (size_t)L.ksplit * align256((size_t)T * H * 4);
   // list of the tokens with a non-zero upstream gradient, its inverse, and its length
   L.off_rows = o;  o += align256((size_t)L.tpad * 4);
@@ -258,7 +266,7 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
 
 // vchunk <= 0 picks the default chunk width: as wide as possible (fewer, longer launches) while the
 // whole workspace stays below a quarter of one [T, V] tile plus one fp32 [V, H],
-//   8*T*vc*esz/2 + esz*vc*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
+//   (2 or 4)*T*vc*esz + esz*vc*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
 // and no wider than 32768 columns or, with few tokens, than what gives the d_logits pass 512 tiles.
 // gt, gv: K-permutation groups that tokens / vocabulary are rounded up to (at most one workgroup
 // tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
@@ -301,8 +309,13 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                        (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), dentropy, T, rows, inv, n_rows);
     if ((rc = check_launch("active_rows_kernel"))) return rc;
   }
-  // K-contiguous copy of the d_weight GEMM's second operand: h^T [H][T] (W^T follows chunk by chunk)
-  {
+  // second operand of the d_weight GEMM (W^T for d_hidden follows chunk by chunk): the listed rows of hidden,
+  // as they are (K-major, for the transposing reads), or transposed to h^T [H][T]
+  if (L.tn) {
+    ProfScope prof(PC_TRANSPOSE, st);
+    hipLaunchKernelGGL(gather_rows_kernel<TIN>, dim3(2048), dim3(256), 0, st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
+    if ((rc = check_launch("gather_rows_kernel"))) return rc;
+  } else {
     ProfScope prof(PC_TRANSPOSE, st);
     hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 1>), dim3((unsigned)((L.tpad + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
                        st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
@@ -310,7 +323,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   }
 
   const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
-  allow_lds(lce_bwd_chunk_kernel<Cfg>, Cfg::LDS_BYTES);
+  // (the K-major d_weight tiles use the 160 KB split ring whatever ring the variant itself uses)
+  const int chunk_lds = L.tn && Cfg::LDS_BYTES < 160 * 1024 ? 160 * 1024 : Cfg::LDS_BYTES;
+  allow_lds(lce_bwd_chunk_kernel<Cfg>, chunk_lds);
   // launch c (0 <= c <= nchunks): d_logits of chunk c (if any) + the two gradient GEMMs of chunk c-1 (if any)
   for (int c = 0; c <= L.nchunks; ++c) {
     BwdChunkArgs<TIN> p;
@@ -326,7 +341,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_lp = dlogprobs; d.g_lp_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
       d.g_lp_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f;
       d.g_ent = dentropy;
-      d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
+      d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = L.tn ? nullptr : dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       d.rows = rows; d.n_rows = n_rows;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
@@ -358,8 +373,15 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         p.gh.cf_split_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
       }
       // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
-      p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
-      p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
+      if (L.tn) {
+        // d_weight[v0 : v0 + vrows][H] = dS[tokens][vrows]^T . hidden[tokens][H], both operands K-major
+        p.gw = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Ht, L.ldHt, vrows, H, round_up(T, 64), nullptr, 0, d_weight + v0 * H, H, 2);
+        p.gw.tn = 1;
+        p.gw.k_dev = n_rows; p.gw.k_gran = 64;
+      } else {
+        p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
+        p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
+      }
       p.n_gh = p.gh.map.total * L.ksplit;
       p.n_gw = p.gw.map.total;
       if (p.gh.kslice > p.gw.K) {  // longer tiles go first
@@ -377,13 +399,13 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         if (k == 1) q.gw = p.gh;  // sub-problem k is moved to the front slot of a single-problem launch
         if (k == 2) { q.n_gw = 0; q.n_gh = 0; } else { q.n_gw = n[k]; q.n_gh = 0; q.n_ds = 0; }
         ProfScope prof(cls[k], st);
-        hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, q);
+        hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, q);
         if ((rc = check_launch("lce_bwd_chunk_kernel(split)"))) return rc;
       }
       continue;
     }
     ProfScope prof(PC_BWD_CHUNK, st);
-    hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
   {
@@ -475,6 +497,7 @@ int lce_set_variant(int variant) {
 int lce_set_option(int key, int64_t value) {
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
+    case LCE_OPT_DW_TRANSPOSED_READS: g_dw_transposed_reads = value != 0; return LCE_OK;
     case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }

@@ -300,9 +300,9 @@ struct DsArgs {
   const float* g_ent;   // [T] or null
   TIN* dS;              // [T][ldS]      (token-major)
   int64_t ldS;
-  TIN* dST;             // [vchunk][ldST] (vocab-major)
+  TIN* dST;             // [vchunk][ldST] (vocab-major); null when the d_weight GEMM reads dS with transposing LDS reads
   int64_t ldST;
-  int64_t tpad;         // tokens rounded up to the GEMM K granule: columns [T, tpad) of dST are written as zeros
+  int64_t tpad;         // tokens rounded up to the GEMM K granule: columns [T, tpad) of dST / rows [T, tpad) of dS are written as zeros
   TileMap map;          // rows = token tiles, cols = vocab tiles of the chunk
   // Token compaction (both null = off): only tokens with a non-zero upstream gradient take part.
   // rows[k] is the token behind compact position k < *n_rows; dS / dS^T are indexed by k, while
@@ -420,7 +420,7 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
       rel[j] = (y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
     }
   }
-  const bool tok_group_live = tok0 < p.tpad;                 // the whole token group is inside dS^T's columns
+  const bool tok_group_live = p.dST != nullptr && tok0 < p.tpad;  // the whole token group is inside dS^T's columns
   TIN* dst_t = p.dST + (tok0 + (int64_t)ln * FN);            // + vocab row * ldST   (token order: ln*FN + j)
   TIN* dst_s = p.dS + (vloc0 + hh * 16 * FM);                // + token * ldS + i*16 + r (vocab order: hh, i, r)
 #pragma unroll
@@ -464,7 +464,8 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
       const int c = pc ^ Stg::swz(row);
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(stage_lds + row * Stg::ROW_BYTES + pc * 16);
       const int64_t tok = tok0 + row;
-      if (tok < Tc) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
+      // rows of tokens that do not take part are zeros (the staged values are); they pad the d_weight GEMM's K
+      if (tok < p.tpad) *reinterpret_cast<u32x4_t*>(p.dS + tok * p.ldS + vloc0 + c * 8) = v;
     }
   }
 }
@@ -530,6 +531,9 @@ struct GemmArgs {
   const int* m_dev;
   const int* k_dev;
   int k_gran;
+  // operands K-major, A[k][m] and B[k][n] (gemm_tn_tile); the rows of C are then A's columns, which the d_logits
+  // epilogue leaves in KPerm::vocab order: row u of the tile is written to row KPerm::vocab_at(u) of C
+  int tn;
 };
 
 template <typename Cfg, int MODE, bool EDGE>
@@ -612,10 +616,39 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
 #undef LCE_EPI
 }
 
-// C[m][n] = sum_k A[k][m] * B[k][n]: both operands K-major (Cfg::TRANS); M, N whole tiles of the operands'
-// allocated width, K a multiple of 64
-template <typename Cfg>
-LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+// C[m][n] = sum_k A[k][m] * B[k][n]: both operands K-major (Cfg::TRANS); A and B are allocated in whole
+// 256-column tiles, K (or *k_dev rounded up to k_gran) a multiple of 64.  out_mode 0: Cf = acc;
+// out_mode 2: Ct[KPerm::vocab_at(m)][n] = (TIN)acc (see GemmArgs::tn).
+template <typename Cfg, typename PermCfg, int MODE, bool EDGE>
+LCE_DEV void gemm_tn_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t m0, int64_t n0,
+                              int wave_m, int wave_n, int hh, int ln) {
+  typedef typename Cfg::TIN TIN;
+#pragma unroll
+  for (int j = 0; j < Cfg::FN; ++j) {
+    const int64_t n = n0 + wave_n * Cfg::WN + j * 32 + ln;
+    if (EDGE && n >= p.N) continue;
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i) {
+      __builtin_amdgcn_sched_barrier(0);  // one 32x32 block at a time (register pressure)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int u = acc_row(i, r, hh);  // row inside the wave tile
+        const int64_t m = m0 + wave_m * Cfg::WM + (MODE == 2 ? (int)KPerm<PermCfg>::vocab_at(u) : u);
+        if (EDGE && m >= p.M) continue;
+        if (MODE == 2) p.Ct[m * p.ldct + n] = (TIN)acc[i][j][r];
+        else p.Cf[m * p.ldcf + n] = acc[i][j][r];
+      }
+    }
+  }
+}
+
+template <typename Cfg, typename PermCfg>
+LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
+  GemmArgs<typename Cfg::TIN> p = pin;
+  if (p.k_dev) {
+    const int64_t k = ((int64_t)*p.k_dev + p.k_gran - 1) / p.k_gran * p.k_gran;
+    p.K = k < p.K ? k : p.K;
+  }
   int tm, tn;
   if (!p.map.decode(bid, tm, tn)) return;
   const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
@@ -623,16 +656,30 @@ LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* l
   GemmCore<Cfg> g;
   g.init_tn(p.A, p.lda, m0, p.B, p.ldb, n0);
   f32x16_t acc[Cfg::FM][Cfg::FN];
-  g.run(lds, p.K, acc);
+  if (p.K > 0) {
+    g.run(lds, p.K, acc);
+  } else {
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  }
   const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
-  if (edge) gemm_epilogue<Cfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
-  else gemm_epilogue<Cfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  if (p.out_mode == 2) {
+    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 2, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_tn_epilogue<Cfg, PermCfg, 2, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  } else {
+    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_tn_epilogue<Cfg, PermCfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  }
 }
 
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NTHREADS) void gemm_tn_kernel(GemmArgs<typename Cfg::TIN> p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  gemm_tn_tile<Cfg>(p, blockIdx.x, lds);
+  gemm_tn_tile<Cfg, Cfg>(p, blockIdx.x, lds);
 }
 
 template <typename Cfg>
@@ -661,12 +708,29 @@ struct BwdChunkArgs {
   int n_gw, n_gh, n_ds;
 };
 
+// the mainloop configuration for K-major operands that goes with Cfg (same tile and wave layout, split ring)
+template <typename Cfg>
+struct TransOf {
+  typedef GemmCfg<typename Cfg::TIN, Cfg::BM, Cfg::BN, 128, 5, Cfg::WAVES_M, Cfg::WAVES_N, 2, true> type;
+};
+
+template <typename Cfg>
+LCE_DEV void any_gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+  if constexpr (sizeof(typename Cfg::TIN) == 2 && Cfg::BM == 256 && Cfg::BN == 256 && Cfg::WAVES_M == 4 && Cfg::WAVES_N == 2) {
+    if (p.tn) {
+      gemm_tn_tile<typename TransOf<Cfg>::type, Cfg>(p, bid, lds);
+      return;
+    }
+  }
+  gemm_tile<Cfg>(p, bid, lds);
+}
+
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_chunk_kernel(BwdChunkArgs<typename Cfg::TIN> p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int bid = blockIdx.x;
-  if (bid < p.n_gw) gemm_tile<Cfg>(p.gw, bid, lds);
-  else if (bid < p.n_gw + p.n_gh) gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds);
+  if (bid < p.n_gw) any_gemm_tile<Cfg>(p.gw, bid, lds);
+  else if (bid < p.n_gw + p.n_gh) any_gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds);
   else ds_tile<Cfg>(p.ds, bid - p.n_gw - p.n_gh, lds);
 }
 
@@ -724,6 +788,26 @@ __global__ __launch_bounds__(NT) void active_rows_kernel(const float* g_lp, int6
 
 __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+// out[r][:C] = in[rows[r]][:C] (in[r] without `rows`) for r < R = *n_rows (R without), zeros for the rows up to the next
+// multiple of 64 (the K granule of the d_weight GEMM); one 16-byte chunk per thread, C a multiple of 16 bytes
+template <typename T>
+__global__ void gather_rows_kernel(const T* in, int64_t ldi, int64_t R, int64_t C, T* out, int64_t ldo, int64_t rpad, const int* rows,
+                                   const int* n_rows) {
+  constexpr int N = 16 / (int)sizeof(T);
+  typedef typename VecOf<T, N>::type vec_t;
+  if (n_rows) R = *n_rows;
+  const int64_t rend = (R + 63) / 64 * 64 < rpad ? (R + 63) / 64 * 64 : rpad;
+  const int64_t per_row = C / N, n = rend * per_row;
+  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = q / per_row, c = (q - r * per_row) * N;
+    vec_t v;
+#pragma unroll
+    for (int e = 0; e < N; ++e) v[e] = (T)0.f;
+    if (r < R) v = *reinterpret_cast<const vec_t*>(in + (rows ? (int64_t)rows[r] : r) * ldi + c);
+    *reinterpret_cast<vec_t*>(out + r * ldo + c) = v;
+  }
 }
 
 // out[c][perm(r)] = in[r][c] for r < R, c < C; out has `ldo` columns, columns perm(r) with r in
