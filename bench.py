@@ -24,8 +24,8 @@ PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
 # (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt); counters cannot be read from inside this process.
 MEASURED_TRAFFIC = {
     "qwen2.5-7b-head-T16384": {
-        "lce_bwd_chunk_kernel": 4754751 * 1024 * 2.0 + 1413682 * 1024 * 1.0,
-        "lce_fwd_kernel": 13262378 * 1024 * 2.0 + 8184 * 1024 * 1.0,
+        "lce_bwd_chunk_kernel": 8471482 * 1024 * 2.0 + 1383069 * 1024 * 1.0,
+        "lce_fwd_kernel": 13773737 * 1024 * 2.0 + 8184 * 1024 * 1.0,
     }
 }
 WORKLOADS = {
