@@ -376,6 +376,22 @@ def test_tokens_without_upstream_gradient(pattern, dtype):
         assert torch.count_nonzero(dw) == 0
 
 
+@pytest.mark.parametrize("T", [8192, 8193, 9001])
+def test_d_hidden_operand_mode_switches_with_token_count(T):
+    """Up to 8192 tokens the bf16 d_hidden GEMM reads W as it lies in memory; beyond that it reads a
+    transposed copy of each chunk.  Both sides of the switch, ragged and with masked tokens."""
+    H, V, tau = 128, 1300, 0.7
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=37)
+    g_lp, g_ent = g_lp.float(), g_ent.float()
+    keep = (torch.rand(T, generator=torch.Generator().manual_seed(41)) < 0.6).to(DEV)
+    g_lp, g_ent = g_lp * keep, g_ent * keep
+    _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    assert torch.count_nonzero(dh[~keep]) == 0
+
+
 def test_every_tile_variant_agrees():
     from verl_amd import _abi
 

@@ -48,6 +48,14 @@ LCE_DEV u32x2_t tr_read(uint32_t lds_addr) {
   return v;
 }
 
+// plain 16-byte LDS read as inline assembly, for loops that place their lgkmcnt waits by hand
+template <int OFF>
+LCE_DEV u32x4_t lds_read16(uint32_t lds_addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_addr), "n"(OFF));
+  return v;
+}
+
 template <typename T>
 struct Mma;
 
@@ -79,16 +87,18 @@ struct Mma<float> {
 // A0 B0 A1 B1 A2 ...; with five of them a barrier still hands back one A and one B half per slab, but
 // the odd half lets the A operand of the slab after next stay in flight ACROSS the barrier, so half of
 // the loads get two barrier periods to land instead of one.
-// TRANS_ (split ring, 16-bit elements only): both operands are stored K-major in memory, A[k][m] and B[k][n]
-// (C = A^T . B); a ring slot holds 64 k-rows of 256 columns and the MFMA operand fragments are fetched with the
-// transposing LDS read (ds_read_b64_tr_b16, two per fragment).
-template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0, bool TRANS_ = false>
+// TRANS_ (split ring, 16-bit elements only): 1 = both operands are stored K-major in memory, A[k][m] and B[k][n]
+// (C = A^T . B); 2 = only B is (C = A . B with A[m][k], B[k][n]).  A ring slot of a K-major operand holds 64 k-rows
+// of 256 columns and its MFMA operand fragments are fetched with the transposing LDS read (ds_read_b64_tr_b16,
+// two per fragment).
+template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0, int TRANS_ = 0>
 struct GemmCfg {
   typedef TIN_ TIN;
   static constexpr int BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
   static constexpr int SPLIT = SPLIT_;  // 0 whole stages; 1 split ring, A operand early; 2 split ring, B operand early
-  static constexpr bool TRANS = TRANS_;
-  static_assert(!TRANS_ || (SPLIT_ != 0 && sizeof(TIN_) == 2 && BM_ == 256 && BN_ == 256 && BKB_ == 128), "transposed operands: split ring, 16-bit, 256x256");
+  static constexpr int TRANS = TRANS_;
+  static constexpr bool TRANS_A = TRANS_ == 1, TRANS_B = TRANS_ != 0;
+  static_assert(TRANS_ == 0 || (SPLIT_ != 0 && sizeof(TIN_) == 2 && BM_ == 256 && BN_ == 256 && BKB_ == 128), "transposed operands: split ring, 16-bit, 256x256");
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NTHREADS = NW * 64;
@@ -135,6 +145,9 @@ struct GemmCore {
   int wave, lane, wave_m, wave_n;
   uint32_t a_rd, b_rd;  // LDS byte offsets (within a stage) of this lane's operand rows, swizzle folded in
   int64_t a_slab, b_slab;  // bytes from one K slab to the next in memory (BKB, or 64 rows for K-major operands)
+  // mixed mode (only B K-major): memory row inside a slab and chunk offset of each load, rows clamped per slab
+  int b_row[Cfg::B_LOADS];
+  int64_t b_ld_bytes, b_kvalid;
 
   // rows beyond the matrix are clamped to its last row (their results are discarded by the epilogue).
   // With `b_rows` given, row n of the B operand is B[b_rows[n]] (a gather; B is then the matrix's first
@@ -201,6 +214,31 @@ struct GemmCore {
     b_rd = row_off + (uint32_t)((((nb / 8) ^ (4 * e)) * 16) + (nb % 8) * 2);
   }
 
+  // A[m][k] row-major as in init(); B[k][n0 + 0..BN) K-major with row stride ldb.  LDS row r of a slab is memory row
+  // perm(r) of the slab (perm: a permutation of 0..63, the order in which A's columns were stored), and memory rows at
+  // or beyond `kvalid` are replaced by row kvalid-1 (A is zero there).  B has `ncols` columns from n0 on.
+  template <typename Perm>
+  LCE_DEV void init_mixed(const TIN* A, int64_t lda, int64_t m0, int64_t M, const TIN* B, int64_t ldb, int64_t n0, int64_t ncols,
+                          int64_t kvalid, Perm perm) {
+    init(A, lda, m0, M, B, ldb, 0, Cfg::BN);
+    b_base = reinterpret_cast<const char*>(B + n0);
+    b_slab = 64;  // rows per slab (the byte offset is formed per load, see dma_half)
+    b_ld_bytes = ldb * (int64_t)sizeof(TIN);
+    b_kvalid = kvalid;
+#pragma unroll
+    for (int j = 0; j < Cfg::B_LOADS; ++j) {
+      const int row = (j * Cfg::NW + wave) * 2 + lane / 32;
+      const int c = (lane % 32) ^ ((row % 4) * 4);
+      b_row[j] = (int)perm(row);
+      // columns beyond the matrix (last N tile of a width that is no multiple of the tile) are fetched from the
+      // row's first chunk instead: in bounds, and they only feed output columns that are discarded
+      lb.voff[j] = (uint32_t)(((int64_t)c * (16 / (int)sizeof(TIN)) < ncols ? c : 0) * 16);
+    }
+    const int g = lane / 16, e = (lane % 16) / 4, q = lane % 4;
+    const int nb = wave_n * Cfg::WN + 16 * (g % 2) + 4 * q;
+    b_rd = (uint32_t)((8 * (g / 2) + e) * 512) + (uint32_t)((((nb / 8) ^ (4 * e)) * 16) + (nb % 8) * 2);
+  }
+
   static constexpr int PER = Cfg::A_LOADS + Cfg::B_LOADS;  // wave-wide DMA loads per slab
   static constexpr int N_READS = Cfg::FM + Cfg::FN;       // LDS operand reads per k-substep
   static constexpr int N_BLK = Cfg::FM * Cfg::FN;         // 32x32 blocks per wave
@@ -227,9 +265,19 @@ struct GemmCore {
 #endif
     char* sa = lds + slot * Cfg::STAGE_BYTES + (j * Cfg::NW + wave) * 1024;
     // kbyte counts BKB bytes per slab; K-major operands advance by 64 rows per slab instead
-    const int64_t off = Cfg::TRANS ? (kbyte / Cfg::BKB) * (is_b ? b_slab : a_slab) : kbyte;
-    if (is_b) __builtin_amdgcn_global_load_lds((gptr_t)(b_base + off + lb.voff[j]), (lptr_t)sa, 16, 0, 0);
-    else __builtin_amdgcn_global_load_lds((gptr_t)(a_base + off + la.voff[j]), (lptr_t)sa, 16, 0, 0);
+    if (is_b) {
+      int64_t off = kbyte;
+      if constexpr (Cfg::TRANS == 1) off = (kbyte / Cfg::BKB) * b_slab;
+      if constexpr (Cfg::TRANS == 2) {
+        int64_t row = (kbyte / Cfg::BKB) * 64 + b_row[j];
+        row = row < b_kvalid ? row : b_kvalid - 1;
+        off = row * b_ld_bytes;
+      }
+      __builtin_amdgcn_global_load_lds((gptr_t)(b_base + off + lb.voff[j]), (lptr_t)sa, 16, 0, 0);
+    } else {
+      const int64_t off = Cfg::TRANS_A ? (kbyte / Cfg::BKB) * a_slab : kbyte;
+      __builtin_amdgcn_global_load_lds((gptr_t)(a_base + off + la.voff[j]), (lptr_t)sa, 16, 0, 0);
+    }
   }
   LCE_DEV void issue_slab(char* lds, int stage, int64_t kbyte) const {
 #pragma unroll
@@ -242,18 +290,28 @@ struct GemmCore {
 #ifdef LCE_DBG_NO_READS
     if (kk > 0) return;
 #endif
-    if constexpr (Cfg::TRANS) {
-      // block i of A / j of B: 32 columns further = 4 chunks = bit 6 / bits 6-7 of the byte offset, which the
-      // swizzle XORs; substep kk: 16 rows further; second half of the fragment: 4 rows further
+    if constexpr (Cfg::TRANS != 0) {
       const bool is_a = idx == 0 || idx > Cfg::FN;
       const int blk = idx == 0 ? 0 : (idx <= Cfg::FN ? idx - 1 : idx - Cfg::FN);
-      const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(is_a ? sa : sb) + ((is_a ? a_rd : b_rd) ^ (uint32_t)(blk * 64));
-      u32x2_t lo, hi;
-      if (kk == 0) { lo = tr_read<0>(base); hi = tr_read<2048>(base); }
-      else if (kk == 1) { lo = tr_read<8192>(base); hi = tr_read<8192 + 2048>(base); }
-      else if (kk == 2) { lo = tr_read<16384>(base); hi = tr_read<16384 + 2048>(base); }
-      else { lo = tr_read<24576>(base); hi = tr_read<24576 + 2048>(base); }
-      const u32x4_t v = {lo[0], lo[1], hi[0], hi[1]};
+      u32x4_t v;
+      if ((is_a && Cfg::TRANS_A) || (!is_a && Cfg::TRANS_B)) {
+        // block i of A / j of B: 32 columns further = 4 chunks = bit 6 / bits 6-7 of the byte offset, which the
+        // swizzle XORs; substep kk: 16 rows further; second half of the fragment: 4 rows further
+        const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(is_a ? sa : sb) + ((is_a ? a_rd : b_rd) ^ (uint32_t)(blk * 64));
+        u32x2_t lo, hi;
+        if (kk == 0) { lo = tr_read<0>(base); hi = tr_read<2048>(base); }
+        else if (kk == 1) { lo = tr_read<8192>(base); hi = tr_read<8192 + 2048>(base); }
+        else if (kk == 2) { lo = tr_read<16384>(base); hi = tr_read<16384 + 2048>(base); }
+        else { lo = tr_read<24576>(base); hi = tr_read<24576 + 2048>(base); }
+        v = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+      } else {
+        // row-major operand: block i is 32 rows = 4096 bytes further, substep kk flips chunk bits (see the plain path)
+        const uint32_t base = (uint32_t)reinterpret_cast<uintptr_t>(is_a ? sa : sb) + ((is_a ? a_rd : b_rd) ^ (uint32_t)(kk * 32));
+        if (blk == 0) v = lds_read16<0>(base);
+        else if (blk == 1) v = lds_read16<4096>(base);
+        else if (blk == 2) v = lds_read16<8192>(base);
+        else v = lds_read16<12288>(base);
+      }
       if (is_a) af[blk] = v;
       else bf[blk] = v;
       return;
@@ -280,17 +338,19 @@ struct GemmCore {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int b = 0; b < N_BLK; ++b) {
-      if constexpr (Cfg::TRANS) {
+      if constexpr (Cfg::TRANS != 0) {
         // The operand reads are inline assembly (see tr_read), so the waits are placed by hand.  Reads are issued
-        // in the order a0, b0 .. b(FN-1), a1 .., two instructions each, one operand after each of the first MFMAs,
-        // and LDS reads return in order.  Before MFMA b of this substep, 2*min(b, N_READS) reads of the NEXT
-        // substep are in flight behind this substep's 2*N_READS; it needs its A block (b / FN) and B block (b % FN).
-        constexpr int ALL = 2 * N_READS;
+        // in the order a0, b0 .. b(FN-1), a1 .. (two instructions for a K-major operand, one for a row-major one),
+        // one operand after each of the first MFMAs, and LDS reads return in order.  Before MFMA b of this
+        // substep, the reads of the NEXT substep issued so far are in flight behind this substep's; the MFMA
+        // needs its A block (b / FN) and its B block (b % FN).
+        constexpr int CA = Cfg::TRANS_A ? 2 : 1, CB = Cfg::TRANS_B ? 2 : 1;
+        constexpr int ALL = CA * Cfg::FM + CB * Cfg::FN;
+        // instructions issued up to and including operand read number `idx` of the order above
+        auto upto = [](int idx) { return idx < 0 ? 0 : (idx == 0 ? CA : (idx <= Cfg::FN ? CA + CB * idx : CA + CB * Cfg::FN + CA * (idx - Cfg::FN))); };
         const int ia = b / Cfg::FN, ib = b % Cfg::FN;
-        const int last = ia == 0 ? 1 + ib : N_READS - Cfg::FM + ia;  // index of the last operand read it depends on
-        const int done = 2 * (last + 1);
-        const int issued = 2 * (b < N_READS ? b : N_READS);
-        const int allow = (ALL - done) + issued;
+        const int last = ia == 0 ? 1 + ib : Cfg::FN + ia;  // the last operand read it depends on
+        const int allow = (ALL - upto(last)) + upto((b < N_READS ? b : N_READS) - 1);
         static_assert(ALL <= 15, "lgkmcnt range");
         wait_lgkm(allow);
         __builtin_amdgcn_sched_barrier(0);  // the wait stays in front of the MFMA

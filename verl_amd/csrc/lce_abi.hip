@@ -98,7 +98,7 @@ GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t l
   p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
   p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
   p.ksplit = 1; p.kslice = K; p.cf_split_stride = 0;
-  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1; p.tn = 0;
+  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1; p.tn = 0; p.b_rows_valid = 0;
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   return p;
@@ -205,7 +205,9 @@ struct BwdLayout {
   size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, total;
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
-  bool tn;     // the d_weight GEMM reads dS (token-major) and a compact copy of hidden, both K-major: no dS^T, no h^T
+  bool tn;     // the gradient GEMMs read dS, a compact copy of hidden and W as they lie in memory (transposing LDS
+               // reads for the K-major operands): no dS^T, no h^T
+  bool tn_dh;  // ... and the d_hidden GEMM reads W as it lies in memory too: no W^T
 };
 
 // The d_weight GEMM can take the token-major d_logits and hidden as they are (transposing LDS reads exist
@@ -229,6 +231,11 @@ int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
 BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
   BwdLayout L;
   L.tn = dw_transposed_reads(esz);
+  // Measured: reading W through the transposing LDS reads costs the d_hidden GEMM about 2% of its rate, and
+  // saves one transpose of W per call.  The transpose is the larger cost up to some thousands of tokens
+  // (T=64: 1.95 -> 1.43 ms per forward + backward, T=4096: 15.7 -> 14.7 ms at H=3584, V=152064), the GEMM
+  // rate beyond that (T=16384: +0.5 ms).
+  L.tn_dh = L.tn && T <= 8192;
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
@@ -253,7 +260,7 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
     L.off_dST[b] = o;
     if (!L.tn && (b == 0 || L.nchunks > 1)) o += align256((size_t)vchunk * L.ldST * esz);
   }
-  L.off_Wt = o;    o += align256((size_t)H * L.ldWt * esz);
+  L.off_Wt = o;    o += L.tn_dh ? 0 : align256((size_t)H * L.ldWt * esz);
   L.off_Ht = o;    o += L.tn ? align256((size_t)L.tpad * L.ldHt * esz) : align256((size_t)H * L.ldHt * esz);
   L.off_dHacc = o; o += (size_t)L.ksplit * align256((size_t)T * H * 4);
   // list of the tokens with a non-zero upstream gradient, its inverse, and its length
@@ -356,16 +363,22 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int cc = c - 1;
       const int64_t v0 = (int64_t)cc * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
-      // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . Wt[H][Kc]^T  (rows = listed tokens), Wt = this chunk of W,
-      // transposed just before the launch (the previous launch, the last reader of the buffer, is complete by then)
+      // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . W[v0 : v0 + Kc][H]  (rows = listed tokens)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
-      {
+      if (L.tn_dh) {
+        // W as it lies in memory (K-major for this product), fetched with transposing LDS reads
+        p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, W + v0 * ldw, ldw, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+        p.gh.tn = 2;
+        p.gh.b_rows_valid = vrows;
+      } else {
+        // Wt = this chunk of W, transposed just before the launch (the previous launch, the last reader of the
+        // buffer, is complete by then)
         ProfScope prof(PC_TRANSPOSE, st);
         hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((kc + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
                            st, W + v0 * ldw, ldw, vrows, H, Wt, L.ldWt, kc);
         if ((rc = check_launch("transpose W"))) return rc;
+        p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
       }
-      p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
       p.gh.m_dev = n_rows;
       if (L.ksplit > 1) {
         p.gh.ksplit = L.ksplit;
@@ -699,7 +712,7 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 
 int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
                 void* stream) {
-  typedef GemmCfg<bf16_t, 256, 256, 128, 5, 4, 2, 2, true> Cfg;
+  typedef GemmCfg<bf16_t, 256, 256, 128, 5, 4, 2, 2, 1> Cfg;
   if (!A || !B || !C || !aligned16(A) || !aligned16(B)) return fail(LCE_E_ARG, "bad pointer");
   if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || lda % 8 != 0 || ldb % 8 != 0) return fail(LCE_E_ARG, "gemm_tn: bad shape");
   if (lda < round_up(M, 256) || ldb < round_up(N, 256)) return fail(LCE_E_ARG, "gemm_tn: rows must be allocated in whole 256-column tiles");

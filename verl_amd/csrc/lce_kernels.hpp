@@ -533,7 +533,8 @@ struct GemmArgs {
   int k_gran;
   // operands K-major, A[k][m] and B[k][n] (gemm_tn_tile); the rows of C are then A's columns, which the d_logits
   // epilogue leaves in KPerm::vocab order: row u of the tile is written to row KPerm::vocab_at(u) of C
-  int tn;
+  int tn;  // 0 NT (gemm_tile); 1 both operands K-major (gemm_tn_tile); 2 only B K-major, its rows in KPerm::vocab order (gemm_nb_tile)
+  int64_t b_rows_valid;  // tn == 2: rows of B that exist (K may be rounded up beyond them; A is zero there)
 };
 
 template <typename Cfg, int MODE, bool EDGE>
@@ -708,17 +709,71 @@ struct BwdChunkArgs {
   int n_gw, n_gh, n_ds;
 };
 
+// C[m][n] (+)= sum_k A[m][k] * B[k][n]: A row-major, B K-major as it lies in memory (Cfg::TRANS == 2).  Column k of A
+// holds the product partner of B's row KPerm::vocab_at(k) (the order the d_logits epilogue stores its columns in).
+// Split K, device-side M and the fp32 output modes 0 / 1 as in gemm_tile.
+template <typename Cfg, typename PermCfg>
+LCE_DEV void gemm_nb_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
+  GemmArgs<typename Cfg::TIN> p = pin;
+  if (p.m_dev) {
+    const int64_t m = *p.m_dev;
+    p.M = m < p.M ? m : p.M;
+  }
+  int64_t k0 = 0, k1 = p.K;
+  if (p.ksplit > 1) {
+    const int s = bid / p.map.total;
+    bid -= s * p.map.total;
+    k0 = s * p.kslice;
+    k1 = k0 + p.kslice < p.K ? k0 + p.kslice : p.K;
+    p.Cf += s * p.cf_split_stride;
+  }
+  int tm, tn;
+  const TileMap map = p.m_dev ? p.map.with_rows((int)((p.M + Cfg::BM - 1) / Cfg::BM)) : p.map;
+  if (!map.decode(bid, tm, tn)) return;
+  const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
+  const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
+  GemmCore<Cfg> g;
+  f32x16_t acc[Cfg::FM][Cfg::FN];
+  if (k0 < k1 && k0 < p.b_rows_valid) {
+    g.init_mixed(p.A + k0, p.lda, m0, p.M, p.B + k0 * p.ldb, p.ldb, n0, p.N - n0, p.b_rows_valid - k0,
+                 [](int r) { return KPerm<PermCfg>::vocab_at(r); });
+    g.run(lds, k1 - k0, acc);
+  } else {  // empty K range: contributes zero (and still initialises what it owns)
+    if (p.out_mode == 1) return;
+    g.init(p.A, p.lda, m0, p.M, p.A, p.lda, 0, Cfg::BN);  // (wave_m / wave_n for the epilogue)
+#pragma unroll
+    for (int i = 0; i < Cfg::FM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  }
+  const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
+  if (p.out_mode == 0) {
+    if (edge) gemm_epilogue<Cfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_epilogue<Cfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  } else {
+    if (edge) gemm_epilogue<Cfg, 1, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_epilogue<Cfg, 1, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+  }
+}
+
 // the mainloop configuration for K-major operands that goes with Cfg (same tile and wave layout, split ring)
 template <typename Cfg>
 struct TransOf {
-  typedef GemmCfg<typename Cfg::TIN, Cfg::BM, Cfg::BN, 128, 5, Cfg::WAVES_M, Cfg::WAVES_N, 2, true> type;
+  typedef GemmCfg<typename Cfg::TIN, Cfg::BM, Cfg::BN, 128, 5, Cfg::WAVES_M, Cfg::WAVES_N, 2, 1> type;   // A and B K-major
+  typedef GemmCfg<typename Cfg::TIN, Cfg::BM, Cfg::BN, 128, 5, Cfg::WAVES_M, Cfg::WAVES_N, 2, 2> mixed;  // only B
 };
 
 template <typename Cfg>
 LCE_DEV void any_gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   if constexpr (sizeof(typename Cfg::TIN) == 2 && Cfg::BM == 256 && Cfg::BN == 256 && Cfg::WAVES_M == 4 && Cfg::WAVES_N == 2) {
-    if (p.tn) {
+    if (p.tn == 1) {
       gemm_tn_tile<typename TransOf<Cfg>::type, Cfg>(p, bid, lds);
+      return;
+    }
+    if (p.tn == 2) {
+      gemm_nb_tile<typename TransOf<Cfg>::mixed, Cfg>(p, bid, lds);
       return;
     }
   }
