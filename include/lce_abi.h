@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 3
+#define LCE_ABI_VERSION 4
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -104,6 +104,12 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                         const float* stats, const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd,
                         void* stream);
+
+/* Replaces calculate_sum_pi_squared_from_logits (verl/utils/torch_functional.py:687-703; called on the actor's
+ * logits at verl/workers/engine/fsdp/transformer_impl.py:1413,1513): out[r] = sum_v softmax(logits[r])_v ^ 2
+ * = exp(logsumexp(2 z) - 2 logsumexp(z)), one pass over the row, fp32 arithmetic.  logits [R, V] row stride ldl;
+ * out [R] fp32. */
+int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream);
 
 /* Consumer of the path's outputs: the clipped PPO policy loss with dual clip, token-mean
  * aggregation and entropy bonus.  Replaces, for the vanilla loss with token-mean aggregation,

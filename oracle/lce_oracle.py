@@ -15,6 +15,7 @@ What each function follows in the reference tree (paths relative to the referenc
                              verl/utils/experimental/torch_functional.py:61-93 (same math)
 * ``logprobs_from_logits``   verl/utils/torch_functional.py:155-207
 * ``entropy_from_logits``    verl/utils/torch_functional.py:231-245
+* ``sum_pi_squared_from_logits`` verl/utils/torch_functional.py:687-703
 * ``logits_backward``        autograd of the two functions above, spelled out
 * ``masked_sum/masked_mean`` verl/utils/torch_functional.py:273-308
 * ``agg_loss``               verl/trainer/ppo/core_algos.py:1140-1206
@@ -25,7 +26,9 @@ How each is pinned (see tests/test_oracle_*.py): the reference's own known-answe
 padded-vocab regression (tests/utils/test_linear_cross_entropy.py:352-395, closed form
 ``3 - log(e^3 + (V-1)e^-15)``), uniform-logit closed forms (entropy ``log V``), shift invariance,
 fp64 brute force in pure Python on tiny inputs, ``torch.autograd`` and central finite differences
-for the gradients, the invariant ``sum_v dz = 0``, the independent C restatement in
+for the gradients, the invariant ``sum_v dz = 0``, for ``sum_pi_squared_from_logits`` the closed forms
+``1/V`` (uniform), ``(1 + (V-1) r^2) / (1 + (V-1) r)^2`` (one logit raised by ``log(1/r)``) and a pure-Python
+``sum(softmax**2)``, the independent C restatement in
 ``lce_oracle.c``, and the reference's known answers for ``agg_loss`` / ``masked_mean``
 (tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-65, tests/utils/test_torch_functional.py:61-72).
 No function here is "parity unpinned".
@@ -150,6 +153,12 @@ def entropy_from_logits(logits: torch.Tensor, compute_dtype=torch.float32):
     z = logits.to(compute_dtype)
     pd = torch.softmax(z, dim=-1)
     return torch.logsumexp(z, dim=-1) - torch.sum(pd * z, dim=-1)
+
+
+def sum_pi_squared_from_logits(logits: torch.Tensor, compute_dtype=torch.float32):
+    """sum_v softmax(z)_v^2, stated as in the reference: exp(logsumexp(2 z) - 2 logsumexp(z))."""
+    z = logits.to(compute_dtype)
+    return torch.exp(torch.logsumexp(2.0 * z, dim=-1) - 2.0 * torch.logsumexp(z, dim=-1))
 
 
 def logits_backward(

@@ -102,3 +102,38 @@ def test_masked_reductions_known_answers():
     m = torch.tensor([0.0, 1.0, 1.0, 0.0], device=DEV)
     assert F.masked_mean(v, m).item() == pytest.approx(2.5)
     assert F.masked_mean(torch.tensor([float("nan"), 2.0, 3.0, float("nan")], device=DEV), m).item() == pytest.approx(2.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 6, 50), (33, 152064), (2, 7, 4099), (1, 1), (0, 16)])
+def test_sum_pi_squared(dtype, shape):
+    """calculate_sum_pi_squared_from_logits (verl/utils/torch_functional.py:687-703) in one pass."""
+    from verl_amd.utils import torch_functional as F
+
+    g = torch.Generator().manual_seed(shape[-1] + 1)
+    z = (torch.randn(*shape, generator=g) * 3).to(dtype).to(DEV)
+    got = F.calculate_sum_pi_squared_from_logits(z)
+    assert got.shape == shape[:-1] and got.dtype == dtype
+    want = O.sum_pi_squared_from_logits(z, torch.float64)
+    tol = dict(atol=1e-7, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(got.double(), want, **tol)
+
+
+def test_sum_pi_squared_closed_forms_strides_and_errors():
+    from verl_amd.utils import torch_functional as F
+
+    V = 70001
+    z = torch.full((3, V), 4.25, device=DEV)
+    torch.testing.assert_close(F.calculate_sum_pi_squared_from_logits(z), torch.full((3,), 1.0 / V, device=DEV), rtol=1e-5, atol=0)
+    big = torch.tensor([[1000.0, -1000.0, 0.0], [-1e4, -1e4, -1e4]], device=DEV)
+    torch.testing.assert_close(F.calculate_sum_pi_squared_from_logits(big), torch.tensor([1.0, 1.0 / 3], device=DEV), rtol=1e-5, atol=0)
+    # rows that start at every 2-byte alignment inside a padded buffer
+    buf = torch.randn(6, 1031, device=DEV).bfloat16()
+    for off in range(8):
+        view = buf[:, off:off + 1000]
+        torch.testing.assert_close(F.calculate_sum_pi_squared_from_logits(view).float(),
+                                   O.sum_pi_squared_from_logits(view), atol=2e-2, rtol=2e-2)
+    with pytest.raises(NotImplementedError):
+        F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))
+    with torch.no_grad():
+        F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))

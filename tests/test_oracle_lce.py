@@ -244,3 +244,31 @@ def test_logits_functions():
     torch.testing.assert_close(O.logits_backward(z, y, g_lp, g_ent, torch.float64), zz.grad)
     torch.testing.assert_close(O.logits_backward(z, y, g_lp, None, torch.float64).sum(-1), torch.zeros(4, 6,
                                dtype=torch.float64), atol=1e-12, rtol=0)
+
+
+def test_sum_pi_squared_closed_forms_and_brute_force():
+    """Pins ``sum_pi_squared_from_logits`` (verl/utils/torch_functional.py:687-703) without retyping its
+    formula: uniform logits give 1/V, one logit raised by log(1/r) over V-1 equal ones gives
+    (1 + (V-1) r^2) / (1 + (V-1) r)^2, a dominant logit gives 1, and small random rows are summed in pure Python."""
+    import math
+
+    for V in (1, 2, 7, 1000):
+        z = torch.full((3, V), 4.25, dtype=torch.float64)
+        torch.testing.assert_close(O.sum_pi_squared_from_logits(z, torch.float64), torch.full((3,), 1.0 / V, dtype=torch.float64))
+    V, r = 50, 0.125
+    z = torch.full((1, V), -2.0, dtype=torch.float64)
+    z[0, 17] += math.log(1 / r)
+    want = (1 + (V - 1) * r * r) / (1 + (V - 1) * r) ** 2
+    assert O.sum_pi_squared_from_logits(z, torch.float64).item() == pytest.approx(want, rel=1e-12)
+    big = torch.tensor([[1000.0, -1000.0, 0.0]])
+    assert O.sum_pi_squared_from_logits(big).item() == pytest.approx(1.0, abs=1e-6)
+    g = torch.Generator().manual_seed(31)
+    z = torch.randn(5, 9, generator=g, dtype=torch.float64) * 2
+    for row, got in zip(z.tolist(), O.sum_pi_squared_from_logits(z, torch.float64).tolist()):
+        mx = max(row)
+        e = [math.exp(v - mx) for v in row]
+        s = sum(e)
+        assert got == pytest.approx(sum((v / s) ** 2 for v in e), rel=1e-12)
+    # shift invariance, and the shape contract (last dimension reduced)
+    torch.testing.assert_close(O.sum_pi_squared_from_logits(z + 3.0, torch.float64), O.sum_pi_squared_from_logits(z, torch.float64))
+    assert O.sum_pi_squared_from_logits(torch.zeros(2, 3, 4)).shape == (2, 3)

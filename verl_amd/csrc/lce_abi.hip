@@ -740,6 +740,21 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   return check_launch("logits_fwd_kernel");
 }
 
+int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream) {
+  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
+  if (R == 0) return LCE_OK;
+  if (!logits || !out) return fail(LCE_E_ARG, "null pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  constexpr int NT = 512;
+  ProfScope prof(PC_LOGITS_FWD, st);
+  if (dtype == LCE_DTYPE_BF16)
+    hipLaunchKernelGGL((logits_pi2_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, V, out);
+  else
+    hipLaunchKernelGGL((logits_pi2_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, V, out);
+  return check_launch("logits_pi2_kernel");
+}
+
 size_t lce_ppo_loss_workspace_bytes(int64_t N) {
   (void)N;
   return 1024 * 8 * sizeof(float);

@@ -951,8 +951,9 @@ struct RowSplit {
   }
 };
 
-// per-row online (max, sum exp, sum z exp): the block leaves m = max, a = sum exp(z - m), b = sum z exp(z - m)
-template <typename TIN, int NT>
+// per-row online (max, sum exp, sum z exp): the block leaves m = max, a = sum exp(z - m), b = sum z exp(z - m);
+// with SQ the third sum is sum exp(z - m)^2 instead (it rescales with the square of the factor)
+template <typename TIN, int NT, bool SQ = false>
 LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, float* sh) {
   typedef RowSplit<TIN> RS;
   typedef typename RS::vec_t vec_t;
@@ -962,12 +963,12 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
     if (z > tm) {
       const float sc = fast_exp2((tm - z) * kLog2e);
       ta *= sc;
-      tb *= sc;
+      tb *= SQ ? sc * sc : sc;
       tm = z;
     }
     const float e = fast_exp2((z - tm) * kLog2e);
     ta += e;
-    tb = __builtin_fmaf(z, e, tb);
+    tb = __builtin_fmaf(SQ ? e : z, e, tb);
   };
   auto add_vec = [&](const vec_t& v) {
     float z[N];
@@ -980,7 +981,7 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
     if (vm > tm) {  // one rescale per vector
       const float sc = fast_exp2((tm - vm) * kLog2e);
       ta *= sc;
-      tb *= sc;
+      tb *= SQ ? sc * sc : sc;
       tm = vm;
     }
     const float ntm2 = -tm * kLog2e;
@@ -988,8 +989,16 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
     for (int e = 0; e < N; ++e) {
       const float ex = fast_exp2(__builtin_fmaf(z[e], kLog2e, ntm2));
       ta += ex;
-      tb = __builtin_fmaf(z[e], ex, tb);
+      tb = __builtin_fmaf(SQ ? ex : z[e], ex, tb);
     }
+  };
+  auto merge = [&](float& m1, float& a1, float& b1, float m2, float a2, float b2) {
+    if (!SQ) return merge_stats(m1, a1, b1, m2, a2, b2, kLog2e);
+    const float mn = fmaxf(m1, m2);
+    const float s1 = fast_exp2((m1 - mn) * kLog2e), s2 = fast_exp2((m2 - mn) * kLog2e);
+    a1 = a1 * s1 + a2 * s2;
+    b1 = b1 * s1 * s1 + b2 * s2 * s2;
+    m1 = mn;
   };
   const RS rs(row, V);
   for (int64_t v = threadIdx.x; v < rs.head; v += NT) add_one(load_as_float(row, v));
@@ -1005,7 +1014,7 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
   // wave reduce
   for (int off = 32; off > 0; off >>= 1) {
     const float m2 = __shfl_xor(tm, off), a2 = __shfl_xor(ta, off), b2 = __shfl_xor(tb, off);
-    merge_stats(tm, ta, tb, m2, a2, b2, kLog2e);
+    merge(tm, ta, tb, m2, a2, b2);
   }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) {
@@ -1017,7 +1026,7 @@ LCE_DEV void row_stats(const TIN* row, int64_t V, float& m, float& a, float& b, 
   tm = sh[0];
   ta = sh[1];
   tb = sh[2];
-  for (int w = 1; w < NT / 64; ++w) merge_stats(tm, ta, tb, sh[w * 3], sh[w * 3 + 1], sh[w * 3 + 2], kLog2e);
+  for (int w = 1; w < NT / 64; ++w) merge(tm, ta, tb, sh[w * 3], sh[w * 3 + 1], sh[w * 3 + 2]);
   m = tm;
   a = ta;
   b = tb;
@@ -1046,6 +1055,16 @@ __global__ __launch_bounds__(NT) void logits_fwd_kernel(const TIN* logits, int64
       stats[2 * r + 1] = b / a;
     }
   }
+}
+
+// sum over the vocabulary of softmax(row)^2 = sum exp(z - m)^2 / (sum exp(z - m))^2, one pass
+template <typename TIN, int NT>
+__global__ __launch_bounds__(NT) void logits_pi2_kernel(const TIN* logits, int64_t ldl, int64_t V, float* out) {
+  __shared__ float sh[3 * NT / 64];
+  const int64_t r = blockIdx.x;
+  float m, a, q;
+  row_stats<TIN, NT, true>(logits + r * ldl, V, m, a, q, sh);
+  if (threadIdx.x == 0) out[r] = q / (a * a);
 }
 
 template <typename TIN, int NT>

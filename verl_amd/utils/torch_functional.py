@@ -3,7 +3,7 @@
 Same signatures and result dtypes/shapes as the reference's ``verl/utils/torch_functional.py``
 (``gather_from_labels`` :50-70, ``logprobs_from_logits`` :73-107, ``logprobs_from_logits_naive`` :155-170,
 ``logprobs_from_logits_v2`` :173-207, ``entropy_from_logits`` :231-245, ``entropy_from_logits_with_chunking``
-:248-270, ``masked_sum`` :273-291, ``masked_mean`` :294-308).  The row reductions run as single-pass
+:248-270, ``masked_sum`` :273-291, ``masked_mean`` :294-308, ``calculate_sum_pi_squared_from_logits`` :687-703).  The row reductions run as single-pass
 HIP kernels (one read of the logits; fp32 arithmetic whatever the storage dtype) with an autograd
 backward that is one more fused pass; there is no eager fallback on this path.
 """
@@ -117,6 +117,26 @@ def entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
 def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048) -> torch.Tensor:
     """Same value, always fp32 like the reference's chunked variant; the kernel needs no chunking."""
     return _EntropyFromLogits.apply(logits, torch.float32)
+
+
+def calculate_sum_pi_squared_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """sum over the vocabulary of softmax(logits)**2 = exp(logsumexp(2*logits) - 2*logsumexp(logits));
+    shape ``logits.shape[:-1]``, dtype of ``logits``.  One pass over the logits.  The reference calls it on
+    the actor's logits while collecting log-probs (no graph); differentiating through it is not wired and
+    raises instead of returning a detached value."""
+    assert logits.is_cuda, "verl_amd.utils.torch_functional runs on the GPU only"
+    if torch.is_grad_enabled() and logits.requires_grad:
+        raise NotImplementedError("calculate_sum_pi_squared_from_logits has no backward; call it under torch.no_grad()")
+    rows, V = _as_rows(logits)
+    R = rows.shape[0]
+    out = torch.empty((R,), device=logits.device, dtype=torch.float32)
+    if R > 0:
+        with torch.cuda.device(logits.device):
+            rc = _abi.load().lce_logits_sum_pi_squared(
+                rows.data_ptr(), rows.stride(0), R, V, _abi.dtype_code(logits.dtype), out.data_ptr(), _abi.current_stream(logits.device)
+            )
+            _abi.check(rc, "lce_logits_sum_pi_squared")
+    return out.reshape(logits.shape[:-1]).to(logits.dtype)
 
 
 def masked_sum(values, mask, axis=None):
