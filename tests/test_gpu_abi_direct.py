@@ -65,6 +65,44 @@ def test_padded_row_strides_side_stream_and_shifted_workspace(dtype):
         torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_hidden_spanning_more_than_4_gib_runs_without_the_token_list(dtype):
+    """The backward lists the tokens with gradient and gathers their rows of `hidden` with 32-bit byte offsets;
+    when T * ldh * esize reaches 4 GiB it runs on all tokens in place instead.  A [T, H] view with an 8 MiB row
+    stride takes that branch at small T; tokens without gradient must still come out as exact zeros."""
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V, tau = 520, 256, 1500, 1.3
+    ld = (8 << 20) // torch.empty((), dtype=dtype).element_size() + 64
+    assert T * ld * torch.empty((), dtype=dtype).element_size() >= 1 << 32
+    g = torch.Generator().manual_seed(7)
+    hbuf = torch.empty(T, ld, device=DEV, dtype=dtype)
+    hbuf[:, :H] = (torch.rand(T, H, generator=g) - 0.5).to(dtype).to(DEV)
+    h = hbuf[:, :H]
+    w = (torch.rand(V, H, generator=g) - 0.5).to(dtype).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    keep = (torch.rand(T, generator=g) < 0.5).to(DEV)
+    g_lp = (torch.rand(T, generator=g) * 2 - 1).to(DEV) * keep
+    g_ent = (torch.rand(T, generator=g) - 0.5).to(DEV) * keep
+    st = _abi.current_stream(torch.device(DEV))
+    lp, ent, dh, dw = _call(lib, _abi, hbuf, ld, w, H, y, T, H, V, dtype, tau, g_lp, g_ent, st)
+    torch.cuda.synchronize()
+    cd = torch.float64 if dtype == torch.float32 else torch.float32
+    rlp, rent = O.lce_forward(h, w, y, tau, compute_dtype=cd)
+    rdh, rdw = O.lce_backward(g_lp.to(cd), g_ent.to(cd), h, w, y, tau, compute_dtype=cd)
+    if dtype == torch.float32:
+        for got, want in ((lp, rlp), (ent, rent), (dh, rdh), (dw, rdw)):
+            err = (got.double() - want).abs().max().item()
+            assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
+    else:
+        torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+        torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+        torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+        torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+    assert torch.count_nonzero(dh[~keep]) == 0
+
+
 def test_error_codes_leave_the_device_untouched():
     from verl_amd import _abi
 
@@ -82,6 +120,7 @@ def test_error_codes_leave_the_device_untouched():
     assert lib.lce_forward(*args(ldh=H - 8)) == -1           # row stride shorter than a row
     assert lib.lce_forward(*args(ldw=H + 3)) == -1           # row stride not a multiple of 16 bytes
     assert lib.lce_forward(*args(h=h.data_ptr() + 2)) == -1  # misaligned pointer
+    assert lib.lce_forward(*args(ldh=1 << 23)) == -1         # 256 rows would span 4 GiB
     assert lib.lce_forward(*args(tau=0.0)) == -1
     assert lib.lce_forward(*args(red=9)) == -1
     assert lib.lce_forward(*args(nws=16)) == -2              # workspace too small

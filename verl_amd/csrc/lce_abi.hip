@@ -474,6 +474,10 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
   if (V >= (1LL << 31) || T >= (1LL << 31)) return fail(LCE_E_ARG, "T and V must be below 2^31");
   if (H % kmul != 0) return fail(LCE_E_ARG, "hidden size %lld must be a multiple of %lld", (long long)H, (long long)kmul);
   if (ldh < H || ldw < H || ldh % ldmul != 0 || ldw % ldmul != 0) return fail(LCE_E_ARG, "bad row strides ldh=%lld ldw=%lld", (long long)ldh, (long long)ldw);
+  // the loads address a 256-row tile with 32-bit byte offsets from its first row
+  const int64_t esz = dtype == LCE_DTYPE_BF16 ? 2 : 4;
+  if (ldh * esz * 256 >= (1LL << 32) || ldw * esz * 256 >= (1LL << 32))
+    return fail(LCE_E_ARG, "row strides ldh=%lld ldw=%lld too large: 256 rows must span less than 4 GiB", (long long)ldh, (long long)ldw);
   if (T > 0 && (!hidden || !weight || !labels)) return fail(LCE_E_ARG, "null input pointer");
   if (!aligned16(hidden) || !aligned16(weight)) return fail(LCE_E_ARG, "hidden and weight must be 16-byte aligned");
   if (!(temperature > 0.f)) return fail(LCE_E_ARG, "temperature must be positive");
