@@ -176,6 +176,7 @@ def main():
     ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
     ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
     ap.add_argument("--no-transposed-reads", action="store_true", help="diagnostic: d_weight GEMM from a vocab-major copy of the d_logits")
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE", help="diagnostic: lce_set_option(KEY, VALUE)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -200,6 +201,9 @@ def main():
         _abi.check(lib.lce_set_option(3, 0), "lce_set_option")
     if args.dlogits_tokens_first:
         _abi.check(lib.lce_set_option(2, 1), "lce_set_option")
+    for kv in args.option:
+        k, v = kv.split("=")
+        _abi.check(lib.lce_set_option(int(k), int(v)), "lce_set_option")
     if args.vchunk >= 0:
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
