@@ -21,12 +21,14 @@ if ROOT not in sys.path:
 PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
 # HBM-side bytes per launch (fetch + write) of the MFMA kernels on the default workload, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run
-# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt); counters cannot be read from inside this process.
+# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt, profiles/lce_fwd_kernel_qwen2.5-7b-head-T64-fwd.txt); counters
+# cannot be read from inside this process.
 MEASURED_TRAFFIC = {
     "qwen2.5-7b-head-T16384": {
         "lce_bwd_chunk_kernel": 8471482 * 1024 * 2.0 + 1383069 * 1024 * 1.0,
         "lce_fwd_kernel": 13773737 * 1024 * 2.0 + 8184 * 1024 * 1.0,
-    }
+    },
+    "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 536539 * 1024 * 2.0 + 1024 * 1024 * 1.0},
 }
 WORKLOADS = {
     # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step[, forward only])
@@ -301,7 +303,8 @@ def main():
             "data": "synthetic",
             "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
             "roofline": {"bound": "hbm", "kernel": "lce_fwd_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
-                         "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM, "traffic": None,
+                         "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
+                         "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("lce_fwd_kernel"),
                          "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes},
             "kernels": kernels,
             "cpu_baseline": None,
