@@ -108,7 +108,7 @@ def test_product_code_never_imports_the_oracle():
 def test_fused_linear_for_ppo_constructor():
     from verl_amd.utils.experimental.torch_functional import FusedLinearForPPO
 
-    with pytest.raises(ValueError):  # tests/utils/test_experimental_torch_functional_on_cpu.py:127-129
+    with pytest.raises(ValueError, match="Unsupported FusedLinearForPPO backend"):  # tests/utils/test_experimental_torch_functional_on_cpu.py:127-129
         FusedLinearForPPO(impl_backend="nope")
     m = FusedLinearForPPO(chunk_size=3)
     with pytest.raises(ValueError):

@@ -1,7 +1,8 @@
 """Unfused twins on logits that already exist: ``logprobs_from_logits`` and ``entropy_from_logits``.
 
 Same signatures and result dtypes/shapes as the reference's ``verl/utils/torch_functional.py``
-(``gather_from_labels`` :50-70, ``logprobs_from_logits`` :73-107, ``logprobs_from_logits_naive`` :155-170,
+(``gather_from_labels`` :50-70, ``logprobs_from_logits`` :73-107, ``logprobs_from_logits_flash_attn`` :110-133,
+``logprobs_from_logits_naive`` :155-170,
 ``logprobs_from_logits_v2`` :173-207, ``entropy_from_logits`` :231-245, ``entropy_from_logits_with_chunking``
 :248-270, ``masked_sum`` :273-291, ``masked_mean`` :294-308, ``calculate_sum_pi_squared_from_logits`` :687-703).  The row reductions run as single-pass
 HIP kernels (one read of the logits; fp32 arithmetic whatever the storage dtype) with an autograd
@@ -98,6 +99,12 @@ class _EntropyFromLogits(torch.autograd.Function):
 def logprobs_from_logits(logits, labels, inplace_backward=True):
     """log_softmax(logits)[label]; shape ``logits.shape[:-1]``, dtype of ``logits``.
     ``inplace_backward`` is accepted for signature compatibility; the logits are never overwritten."""
+    return _LogprobsFromLogits.apply(logits, labels)
+
+
+def logprobs_from_logits_flash_attn(logits, labels, inplace_backward=True):
+    """The reference routes here when flash-attn's cross-entropy is importable; same value, same kernel
+    (the ``torch_npu`` twin of the reference, :136-152, has no counterpart on this hardware)."""
     return _LogprobsFromLogits.apply(logits, labels)
 
 
