@@ -114,6 +114,25 @@ def test_fp32_inputs_relative_1e5(shape, tau):
         assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
 
 
+def test_config1_fp32_forward_and_backward_full_size():
+    """The reference's CPU-runnable case (Qwen2.5-0.5B-shaped head, T=1024, H=896, V=151936, fp32, weight
+    ~ N(0, 0.02)) at full size: forward to 1e-5 relative against the fp64 oracle, and the backward as well."""
+    T, H, V, tau = 1024, 896, 151936, 1.0
+    g = torch.Generator().manual_seed(1235)
+    h = torch.randn(T, H, generator=g).to(DEV)
+    w = (torch.randn(V, H, generator=g) * 0.02).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = torch.randn(T, generator=g).to(DEV)
+    g_ent = torch.randn(T, generator=g).to(DEV)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau, compute_dtype=torch.float64)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+    for got, want in ((lp, rlp), (ent, rent), (dh, rdh), (dw, rdw)):
+        assert got.dtype == torch.float32
+        err = (got.double() - want).abs().max().item()
+        assert err <= 1e-5 * want.abs().max().item(), (err, want.abs().max().item())
+
+
 @pytest.mark.parametrize("reduction", ["sum", "mean"])
 def test_reductions(reduction):
     T, H, V, tau = 700, 256, 3001, 1.3

@@ -137,3 +137,25 @@ def test_sum_pi_squared_closed_forms_strides_and_errors():
         F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))
     with torch.no_grad():
         F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))
+
+
+@pytest.mark.parametrize("shape", [(8, 17), (3, 5, 32), (1, 1024)])
+def test_sum_pi_squared_at_the_reference_tests_cases(shape):
+    """The reference's own checks (tests/utils/test_torch_functional.py:126-150), in the dtypes the kernels take:
+    the value equals the naive softmax-then-square, lies in (0, 1], and stays finite at logits of +-1000."""
+    from verl_amd.utils import torch_functional as F
+
+    g = torch.Generator().manual_seed(0)
+    logits = (torch.randn(*shape, generator=g) * 5.0).to(DEV)
+    actual = F.calculate_sum_pi_squared_from_logits(logits)
+    expected = torch.softmax(logits.double(), dim=-1).pow(2).sum(dim=-1)
+    assert actual.shape == expected.shape
+    torch.testing.assert_close(actual.double(), expected, atol=1e-5, rtol=1e-5)
+    assert torch.all(actual > 0) and torch.all(actual <= 1.0 + 1e-5)
+    big = torch.tensor([[1000.0, 1001.0, 999.0], [-1000.0, -999.0, -998.0]], device=DEV)
+    got = F.calculate_sum_pi_squared_from_logits(big)
+    want = torch.softmax(big.double(), dim=-1).pow(2).sum(dim=-1)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.double(), want, atol=1e-5, rtol=1e-5)
+    with pytest.raises(NotImplementedError):  # fp64 logits: the kernels take bf16 and fp32
+        F.calculate_sum_pi_squared_from_logits(big.double())
