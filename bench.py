@@ -28,7 +28,7 @@ MEASURED_TRAFFIC = {
         "lce_bwd_chunk_kernel": 8471482 * 1024 * 2.0 + 1383069 * 1024 * 1.0,
         "lce_fwd_kernel": 13773737 * 1024 * 2.0 + 8184 * 1024 * 1.0,
     },
-    "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 536539 * 1024 * 2.0 + 1024 * 1024 * 1.0},
+    "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 537764 * 1024 * 2.0 + 1024 * 1024 * 1.0},
 }
 WORKLOADS = {
     # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step[, forward only])

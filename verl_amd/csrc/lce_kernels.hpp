@@ -43,8 +43,13 @@ struct FwdArgs {
   float c;           // log2(e) / temperature
   f32x4_t* parts;    // [S][T] of (m, a, b, unused)
   float* xlabel;     // [T] raw accumulator value at the label (pre-zeroed; written by the one lane that owns it)
-  int S;             // vocabulary splits; split s owns vocab tiles s, s+S, s+2S, ...
-  int nvt;           // vocabulary tiles
+  int S;             // vocabulary splits
+  // Split s owns the tiles that start at rows s * split_stride + i * tile_step (i = 0, 1, ...) below its end row
+  // min(V, s * split_stride + split_span).  Two layouts: tiles dealt round robin (split_stride = BM, tile_step =
+  // S * BM, split_span = V: concurrently running workgroups stay on neighbouring tiles), or one contiguous row
+  // range per split (split_stride = split_span = rows per split, tile_step = BM: every split reads the same
+  // number of rows of W whatever V is; its last tile is partial).
+  int64_t split_stride, tile_step, split_span;
   TileMap map;       // rows = token tiles, cols = splits
   int64_t label_offset;  // W holds vocabulary rows [label_offset, label_offset + V) of a larger vocabulary (0 = all of it)
 };
@@ -75,18 +80,20 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
   }
 
   f32x16_t acc[Cfg::FM][Cfg::FN];
-  g.init(p.W, p.ldw, (int64_t)s * Cfg::BM, p.V, p.h, p.ldh, n0, p.T);
+  const int64_t row0 = (int64_t)s * p.split_stride;
+  const int64_t vend64 = row0 + p.split_span < p.V ? row0 + p.split_span : p.V;
+  const int vend = (int)vend64;
+  g.init(p.W, p.ldw, row0, vend64, p.h, p.ldh, n0, p.T);
   g.prologue(lds, p.H);
-  for (int vt = s; vt < p.nvt; vt += p.S) {
-    const int64_t m0 = (int64_t)vt * Cfg::BM;
+  for (int64_t m0 = row0; m0 < vend64; m0 += p.tile_step) {
     g.main(lds, p.H, acc);
     const int vbase = (int)m0 + g.wave_m * Cfg::WM;  // vocabulary index of this wave's first row
-    const bool full = m0 + Cfg::BM <= p.V;
+    const bool full = m0 + Cfg::BM <= vend64;
     // start fetching the next tile's first slabs now: the loads fly while this tile's statistics are
     // folded in (the epilogue touches neither LDS nor vector memory on its common path)
     __syncthreads();  // every wave is past its last LDS read and has drained its own loads
-    if (vt + p.S < p.nvt) {
-      g.init(p.W, p.ldw, (int64_t)(vt + p.S) * Cfg::BM, p.V, p.h, p.ldh, n0, p.T);
+    if (m0 + p.tile_step < vend64) {
+      g.init(p.W, p.ldw, m0 + p.tile_step, vend64, p.h, p.ldh, n0, p.T);
       g.prologue(lds, p.H);
     }
     if (!full) {
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
         for (int j = 0; j < Cfg::FN; ++j)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            if (vbase + acc_row(i, r, hh) >= p.V) acc[i][j][r] = -INFINITY;
+            if (vbase + acc_row(i, r, hh) >= vend) acc[i][j][r] = -INFINITY;
     }
 #pragma unroll
     for (int j = 0; j < Cfg::FN; ++j) {
@@ -138,7 +145,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       b[j] = bj;
       // label logit: rare (a token's label falls in this wave tile with probability WM / V)
       const int rel = lab[j] - vbase;
-      const bool mine = lab[j] >= 0 && rel >= 0 && rel < Cfg::WM && (((rel >> 2) & 1) == hh);
+      const bool mine = lab[j] >= 0 && lab[j] < vend && rel >= 0 && rel < Cfg::WM && (((rel >> 2) & 1) == hh);
       if (__builtin_amdgcn_ballot_w64(mine) != 0) {
         float pick = 0.f;
 #pragma unroll
