@@ -43,7 +43,7 @@ const char* lce_last_error(void);
  *   maximum [T], accumulate [T], entropy_b [T]: per-token max logit, sum exp(logit - max) and
  *   sum softmax * logit, kept for the backward.
  * H must be a multiple of 64 (bf16) / 32 (fp32); pointers 16-byte aligned; ldh, ldw multiples of
- * 8 (bf16) / 4 (fp32) elements. */
+ * 8 (bf16) / 4 (fp32) elements and below 16 MiB per row (256 rows are addressed with 32-bit offsets). */
 size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype);
 int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
                 int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
