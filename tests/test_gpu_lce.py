@@ -395,6 +395,28 @@ def test_tokens_without_upstream_gradient(pattern, dtype):
         assert torch.count_nonzero(dw) == 0
 
 
+@pytest.mark.parametrize("T,H,V", [(1, 3584, 152064), (64, 3584, 152064), (100, 1024, 128256), (128, 512, 100003), (7, 256, 70)])
+def test_few_token_forward_splits_take_contiguous_row_ranges(T, H, V):
+    """Up to 128 tokens every vocabulary split of the forward owns one contiguous range of rows whose last tile is
+    partial.  Labels are put on the first and last rows of such ranges (multiples of 64 rows and their
+    neighbours) and on the last row of the vocabulary, where a wrong range end would drop or double a row."""
+    from verl_amd import linear_cross_entropy
+
+    tau = 0.8
+    g = torch.Generator().manual_seed(V + T)
+    h = torch.randn(T, H, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(V, H, generator=g) * 0.03).bfloat16().to(DEV)
+    edges = [0, V - 1] + [r + d for r in range(64, V, 64 * max(1, V // 64 // 97)) for d in (-1, 0)]
+    y = torch.tensor([edges[i % len(edges)] for i in range(T)], dtype=torch.int64)
+    y[T // 2:] = torch.randint(0, V, (T - T // 2,), generator=g)
+    y = y.clamp_(0, V - 1).to(DEV)
+    with torch.no_grad():
+        lp, ent = linear_cross_entropy(h, w, y, tau, "none")
+    rlp, rent = O.lce_forward(h, w, y, tau)
+    torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+    torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+
+
 @pytest.mark.parametrize("T", [8192, 8193, 9001])
 def test_d_hidden_operand_mode_switches_with_token_count(T):
     """Up to 8192 tokens the bf16 d_hidden GEMM reads W as it lies in memory; beyond that it reads a
