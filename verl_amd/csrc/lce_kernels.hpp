@@ -834,7 +834,7 @@ __global__ __launch_bounds__(NT) void active_rows_kernel(const float* g_lp, int6
   __syncthreads();
   // inclusive scan (Hillis-Steele)
   for (int off = 1; off < NT; off <<= 1) {
-    const int v = threadIdx.x >= off ? counts[threadIdx.x - off] : 0;
+    const int v = (int)threadIdx.x >= off ? counts[threadIdx.x - off] : 0;
     __syncthreads();
     counts[threadIdx.x] += v;
     __syncthreads();
