@@ -284,18 +284,20 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   return L;
 }
 
-// vchunk <= 0 picks the default chunk width: as wide as possible (fewer, longer launches) while the
-// whole workspace stays below a quarter of one [T, V] tile plus one fp32 [V, H],
+// vchunk <= 0 picks the default chunk width: as wide as possible (fewer, longer launches; the whole vocabulary
+// in one chunk where that fits, which it does up to about 8192 tokens) while the whole workspace stays below a
+// quarter of one [T, V] tile plus one fp32 [V, H],
 //   (2 or 4)*T*vc*esz + esz*vc*H + (esz + 4*ksplit)*T*H (+ padding)  <=  0.25*T*V*esz + 4*V*H,
-// and no wider than 65536 columns or, with few tokens, than what gives the d_logits pass 512 tiles.
+// then evened out over the number of chunks that width needs.
 // gt, gv: K-permutation groups that tokens / vocabulary are rounded up to (at most one workgroup
 // tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
 BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
     const double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
-    const int64_t ntt = (T + 255) / 256;
-    vchunk = ntt >= 8 ? 65536 : 512 * 256 / ntt;
+    vchunk = round_up(V, 256);
     while (vchunk > 2048 && (double)bwd_layout_for(T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
+    const int64_t n = (V + vchunk - 1) / vchunk;
+    vchunk = round_up((V + n - 1) / n, 256);
   }
   return bwd_layout_for(T, H, V, esz, vchunk, gt, gv);
 }
