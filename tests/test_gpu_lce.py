@@ -304,12 +304,12 @@ def test_config4_weight_grad_accumulates_over_many_tokens():
 
 
 def _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw, chunk=2048):
-    """Bound on |d_weight - exact| that follows from the data format the reference uses and this build keeps: the
-    gradient of the logits is stored in the input dtype before the two GEMMs (verl/utils/kernel/kernels.py:1666-1724:
-    `_d_logits` in hidden.dtype), so every dz carries a relative error of up to 2^-9, and d_weight is rounded to bf16
-    once more: |err| <= 2^-9 * (|dz|^T |h|) + 2^-8 * |d_weight|, plus the north-star 2e-2.  Where two tokens with the
-    same label pull a weight in opposite directions, |dz|^T |h| is much larger than |d_weight| and a bar relative to
-    |d_weight| alone cannot hold for any implementation with that format."""
+    """Bound on |d_weight - exact| that follows from the reference's data format: the gradient of the logits is
+    stored in the input dtype before the two GEMMs (verl/utils/kernel/kernels.py:1666-1724: `_d_logits` in
+    hidden.dtype), so every dz carries a relative error of up to 2^-9, and d_weight is rounded to bf16 once more:
+    |err| <= 2^-9 * (|dz|^T |h|) + 2^-8 * |d_weight|, plus the north-star 2e-2.  Where two tokens with the same
+    label pull a weight in opposite directions, |dz|^T |h| is much larger than |d_weight| and a bar relative to
+    |d_weight| alone cannot hold with that format."""
     T = h.shape[0]
     _, _, mx, acc, eb = O.lce_forward(h, w, y, tau, return_stats=True, chunk=chunk)
     wf = w.float()
@@ -324,12 +324,16 @@ def _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw, chunk=2048):
     return 2e-2 + 2.0**-9 * absdw + 2.0**-8 * rdw.abs()
 
 
-def test_config3_full_size_against_the_whole_oracle():
+@pytest.mark.parametrize("label_term_outside", [1, 0])
+def test_config3_full_size_against_the_whole_oracle(label_term_outside):
     """Llama-3-8B-shaped head at full size: T = 8 x 4096, H=4096, V=128256, tau=0.6, a response mask that zeroes a
     random suffix of each row (valid length U{512..4096}).  Every output is compared with the oracle.  At this
     size some labels occur several times with upstream gradients of opposite sign (d_weight entries of 1.7 that
-    are sums of +14 and -12): d_weight is held to the rounding bound of the bf16 d_logits format, and all but a
-    few hundred of its 525 M entries to the plain bar as well."""
+    are sums of +14 and -12).  By default the one-hot part of d_logits is added in fp32 outside the bf16 tiles and
+    the plain bar holds for every entry; with the reference's format (the one-hot part rounded to bf16 inside the
+    tile) a few hundred of the 525 M entries exceed it and d_weight is held to that format's rounding bound."""
+    from verl_amd import _abi
+
     H, V, tau = 4096, 128256, 0.6
     rows, L = 8, 4096
     T = rows * L
@@ -337,7 +341,12 @@ def test_config3_full_size_against_the_whole_oracle():
     valid = torch.randint(512, L + 1, (rows,), generator=torch.Generator().manual_seed(3))
     mask = (torch.arange(L)[None, :] < valid[:, None]).reshape(-1).to(DEV)
     g_lp, g_ent = g_lp * mask, g_ent * mask
-    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    lib = _abi.load()
+    try:
+        assert lib.lce_set_option(4, label_term_outside) == 0
+        lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    finally:
+        lib.lce_set_option(4, 1)
     rlp, rent = O.lce_forward(h, w, y, tau, chunk=2048)
     rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, chunk=2048)
     assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2
@@ -345,9 +354,13 @@ def test_config3_full_size_against_the_whole_oracle():
     torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
     assert_bf16_bar(dh, rdh)
     assert (dh[~mask] == 0).all()
-    err = (dw.float() - rdw).abs()
-    assert (err <= _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw)).all()
-    assert int((err > 2e-2 + 2.0**-7 * rdw.abs()).sum()) <= 1000
+    if label_term_outside:
+        assert_bf16_bar(dw, rdw)
+        torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)  # the reference's own tolerance
+    else:
+        err = (dw.float() - rdw).abs()
+        assert (err <= _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw)).all()
+        assert int((err > 2e-2 + 2.0**-7 * rdw.abs()).sum()) <= 1000
 
 
 def test_config4_full_size_against_the_whole_oracle():
@@ -363,10 +376,8 @@ def test_config4_full_size_against_the_whole_oracle():
     del rlp, rent
     rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, chunk=2048)
     assert_bf16_bar(dh, rdh)
-    del rdh
-    err = (dw.float() - rdw).abs()
-    assert (err <= _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw)).all()
-    assert int((err > 2e-2 + 2.0**-7 * rdw.abs()).sum()) <= 1000
+    assert_bf16_bar(dw, rdw)
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
 
 
 @pytest.mark.parametrize("vchunk", [256, 1024, 8192])

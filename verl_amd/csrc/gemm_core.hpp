@@ -594,16 +594,16 @@ struct TileMap {
   int total;                   // launched workgroups (multiple of 8)
 
   // shape of the 32-tile blocks that one XCD works on: up to 8 tiles along the row side
-  __host__ __device__ static int block_rows(int nrow_tiles) {
+  __host__ __device__ __forceinline__ static int block_rows(int nrow_tiles) {
     int br = 1;
     while (br < 8 && br < nrow_tiles) br <<= 1;
     return br;
   }
   // the same map over fewer row tiles (a count that only the device knows): its workgroups are the
   // first `total` ids of the grid that was sized for the full map, the others have nothing to do
-  __device__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, rows >= br ? br : block_rows(rows), rows_fastest); }
+  __device__ __forceinline__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, rows >= br ? br : block_rows(rows), rows_fastest); }
 
-  __host__ __device__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
+  __host__ __device__ __forceinline__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
     TileMap t;
     t.nrow_tiles = nrow_tiles;
     t.ncol_tiles = ncol_tiles;
@@ -616,7 +616,7 @@ struct TileMap {
     return t;
   }
   // returns false when the slot is padding (no tile)
-  __device__ bool decode(int bid, int& rt, int& ct) const {
+  __device__ __forceinline__ bool decode(int bid, int& rt, int& ct) const {
     if (bid >= total) return false;
     const int per_xcd = total >> 3;
     const int vid = (bid & 7) * per_xcd + (bid >> 3);

@@ -1,0 +1,204 @@
+// The one-hot part of the gradient of the logits, carried outside the 16-bit d_logits tiles.
+//
+// d_logits[t][v] = G_t * 1[v == label_t] + (terms proportional to softmax_t[v]),  G_t = g_logprob_t / temperature.
+// The softmax terms are small everywhere; G_t is O(1..10) and sits in one column per token.  Rounded to bf16
+// with the rest of the tile it carries an error of up to 2^-9 * |G_t| into d_hidden[t] and into the label's row
+// of d_weight, where several tokens with the same label and gradients of opposite sign leave a small difference
+// of large terms.  So the tiles hold the softmax terms only, and the one-hot part is added in fp32:
+//   d_hidden[t][:]        += G_t * W[label_t][:]        (when the fp32 partials are summed and rounded)
+//   d_weight[label][:]    += sum over tokens t with that label, in ascending t, of G_t * hidden[t][:]
+//                            (written first; the GEMM epilogue adds the softmax terms to these rows)
+// The second sum needs the tokens grouped by label in a fixed order: a stable LSD radix sort of
+// (label row, position in the token list) pairs, 8 bits per pass, written here (no float atomics anywhere, and
+// no library call that a captured graph could not replay).
+#pragma once
+
+#include "lce_kernels.hpp"
+
+namespace lce {
+
+constexpr int kSortBlock = 1024;      // items per workgroup of a sort pass: 4 rounds of 256 threads
+constexpr uint32_t kNoRow = 0xFFFFFFFFu;  // key of a token that contributes no one-hot term; sorts last
+
+// label row of `tok` inside this call's weight, or kNoRow when the label is elsewhere or G is zero
+LCE_DEV uint32_t label_row(const LabelTerm& lt, int64_t tok, float& G) {
+  G = lt.g_lp[tok * lt.g_stride] * lt.scale;
+  const int64_t y = lt.labels[tok] - lt.v0;
+  return (G != 0.f && y >= 0 && y < lt.V) ? (uint32_t)y : kNoRow;
+}
+
+// keys[k] = label row of the k-th listed token (rows[k], or k itself without a list), vals[k] = that token;
+// positions from the list's length up to n_items are filled with kNoRow.
+__global__ __launch_bounds__(256) void label_keys_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int n_items,
+                                                         uint32_t* keys, int* vals) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  if (k >= n_items) return;
+  const int64_t n = n_rows ? (int64_t)*n_rows : T;
+  uint32_t key = kNoRow;
+  int tok = -1;
+  if (k < n) {
+    tok = rows ? rows[k] : k;
+    float G;
+    key = label_row(lt, tok, G);
+  }
+  keys[k] = key;
+  vals[k] = tok;
+}
+
+// ---- one radix pass over `nblocks` blocks of kSortBlock items: histogram, scan, stable scatter ----
+
+// gh[digit * nblocks + block] = number of items of `block` whose digit is `digit`
+LCE_DEV void sort_hist_block(const uint32_t* keys, int shift, int block, int nblocks, int* gh, int* h /* LDS [256] */) {
+  const int tid = threadIdx.x;
+  h[tid] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < kSortBlock / 256; ++q) atomicAdd(&h[(keys[block * kSortBlock + q * 256 + tid] >> shift) & 255], 1);
+  __syncthreads();
+  gh[tid * nblocks + block] = h[tid];
+}
+
+// Items keep their order inside a digit: the item at position q * 256 + tid of a block ranks behind all items of
+// earlier rounds q, earlier waves and lower lanes with the same digit.
+LCE_DEV void sort_scatter_block(const uint32_t* kin, const int* vin, uint32_t* kout, int* vout, int shift, int block,
+                                int nblocks, const int* gh, int* base /* LDS [256] */) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  base[tid] = gh[tid * nblocks + block];
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < kSortBlock / 256; ++q) {
+    const int i = block * kSortBlock + q * 256 + tid;
+    const uint32_t key = kin[i];
+    const int val = vin[i];
+    const int d = (int)((key >> shift) & 255);
+    uint64_t peers = ~0ull;  // lanes of this wave with the same digit
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const uint64_t bal = __builtin_amdgcn_ballot_w64((d >> b) & 1);
+      peers &= ((d >> b) & 1) ? bal : ~bal;
+    }
+    const int rank = __builtin_popcountll(peers & ((1ull << lane) - 1ull));
+    const int cnt = __builtin_popcountll(peers);
+    int off = 0;
+    for (int w = 0; w < 4; ++w) {
+      if (wave == w) {
+        off = base[d];                     // every lane of the group reads the running offset ...
+        __builtin_amdgcn_wave_barrier();
+        if (rank == 0) base[d] = off + cnt;  // ... before its first lane moves it on
+      }
+      __syncthreads();
+    }
+    kout[off + rank] = key;
+    vout[off + rank] = val;
+  }
+}
+
+__global__ __launch_bounds__(256) void sort_hist_kernel(const uint32_t* keys, int shift, int nblocks, int* gh) {
+  __shared__ int h[256];
+  sort_hist_block(keys, shift, blockIdx.x, nblocks, gh, h);
+}
+
+// exclusive scan of gh[0 .. n) in place, one workgroup of 1024 threads
+__global__ __launch_bounds__(1024) void sort_scan_kernel(int* gh, int n) {
+  __shared__ int part[1024];
+  const int tid = threadIdx.x;
+  const int per = (n + 1023) / 1024;
+  const int i0 = tid * per, i1 = i0 + per < n ? i0 + per : n;
+  int s = 0;
+  for (int i = i0; i < i1; ++i) s += gh[i];
+  part[tid] = s;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = tid >= off ? part[tid - off] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - s;
+  for (int i = i0; i < i1; ++i) {
+    const int v = gh[i];
+    gh[i] = run;
+    run += v;
+  }
+}
+
+__global__ __launch_bounds__(256) void sort_scatter_kernel(const uint32_t* kin, const int* vin, uint32_t* kout, int* vout, int shift,
+                                                           int nblocks, const int* gh) {
+  __shared__ int base[256];
+  sort_scatter_block(kin, vin, kout, vout, shift, blockIdx.x, nblocks, gh, base);
+}
+
+// Up to kSortBlock tokens: keys and all passes in one workgroup (buffers 0 / 1 alternate; `passes` is even or
+// odd, the caller reads the result from buffer passes % 2).
+__global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int passes,
+                                                                uint32_t* keys0, int* vals0, uint32_t* keys1, int* vals1) {
+  __shared__ int tab[256];
+  __shared__ int gh[256];
+  const int tid = threadIdx.x;
+  const int64_t n = n_rows ? (int64_t)*n_rows : T;
+  for (int k = tid; k < kSortBlock; k += 256) {
+    uint32_t key = kNoRow;
+    int tok = -1;
+    if (k < n) {
+      tok = rows ? rows[k] : k;
+      float G;
+      key = label_row(lt, tok, G);
+    }
+    keys0[k] = key;
+    vals0[k] = tok;
+  }
+  __syncthreads();
+  for (int p = 0; p < passes; ++p) {
+    const uint32_t* kin = (p & 1) ? keys1 : keys0;
+    const int* vin = (p & 1) ? vals1 : vals0;
+    uint32_t* kout = (p & 1) ? keys0 : keys1;
+    int* vout = (p & 1) ? vals0 : vals1;
+    sort_hist_block(kin, 8 * p, 0, 1, gh, tab);
+    __syncthreads();
+    // exclusive scan of the 256 digit counts
+    const int own = gh[tid];
+    tab[tid] = own;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      const int v = tid >= off ? tab[tid - off] : 0;
+      __syncthreads();
+      tab[tid] += v;
+      __syncthreads();
+    }
+    gh[tid] = tab[tid] - own;
+    __syncthreads();
+    sort_scatter_block(kin, vin, kout, vout, 8 * p, 0, 1, gh, tab);
+    __syncthreads();
+  }
+}
+
+// d_weight[row][:] = (T)(sum of G_t * hidden[t][:] over the run of sorted positions with key == row, in order) and
+// flags[row] = 1.  One workgroup per sorted position; only the first position of a run works.  Runs before the
+// d_weight GEMMs, whose epilogues add their accumulators to the flagged rows and round once more (the first
+// rounding is that of a complete sum, 2^-9 of its own magnitude).
+template <typename T>
+__global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys, const int* toks, int n_items, LabelTerm lt, const T* h,
+                                                            int64_t ldh, int64_t H, T* dW, unsigned char* flags) {
+  constexpr int N = 16 / (int)sizeof(T);
+  typedef typename VecOf<T, N>::type vec_t;
+  const int i = blockIdx.x;
+  const uint32_t key = keys[i];
+  if (key == kNoRow || (i > 0 && keys[i - 1] == key)) return;
+  T* row = dW + (int64_t)key * H;
+  if (threadIdx.x == 0) flags[key] = 1;
+  for (int64_t c = (int64_t)threadIdx.x * N; c < H; c += 256 * N) {
+    float acc[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] = 0.f;
+    for (int j = i; j < n_items && keys[j] == key; ++j) {
+      const int64_t tok = toks[j];
+      const float G = lt.g_lp[tok * lt.g_stride] * lt.scale;
+      const vec_t hv = *reinterpret_cast<const vec_t*>(h + tok * ldh + c);
+#pragma unroll
+      for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(G, (float)hv[e], acc[e]);
+    }
+    store_run<T, N>(row + c, acc);
+  }
+}
+
+}  // namespace lce

@@ -10,6 +10,7 @@
 #include <utility>
 #include <vector>
 
+#include "label_rows.hpp"
 #include "lce_kernels.hpp"
 
 using namespace lce;
@@ -25,6 +26,7 @@ int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
 int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
 int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
+int g_label_outside = 1;  // 16-bit inputs: one-hot part of d_logits added in fp32 outside the d_logits tiles
 int g_dw_transposed_reads = 1;  // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
 
 int fail(int code, const char* fmt, ...) {
@@ -36,7 +38,7 @@ int fail(int code, const char* fmt, ...) {
 }
 
 // ---- optional per-kernel-class timing with HIP events (off by default; used by the benchmark) ----
-enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_BWD_CHUNK, PC_ACTIVE_ROWS, PC_DH_FINISH, PC_COUNT };
+enum { PC_FWD = 0, PC_FWD_MERGE, PC_BWD_DS, PC_GEMM_DH, PC_GEMM_DW, PC_TRANSPOSE, PC_LOGITS_FWD, PC_LOGITS_BWD, PC_BWD_CHUNK, PC_ACTIVE_ROWS, PC_DH_FINISH, PC_LABEL_ROWS, PC_COUNT };
 struct ProfRec { int cls; hipEvent_t a, b; };
 std::mutex g_prof_mu;
 bool g_prof_on = false;
@@ -215,7 +217,8 @@ int forward_splits_upper_bound(int64_t T) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_keys[2], off_vals[2], off_hist, off_flags, total;
+  int sort_items, sort_passes;  // label sort (0 items: the one-hot part stays inside the d_logits tiles)
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
   bool tn;     // the gradient GEMMs read dS, a compact copy of hidden and W as they lie in memory (transposing LDS
@@ -280,6 +283,17 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   L.off_rows = o;  o += align256((size_t)L.tpad * 4);
   L.off_inv = o;   o += align256((size_t)T * 4);
   L.off_nrows = o; o += 256;
+  // (label row, token) pairs, two buffers each, and the per-block digit counts of one radix pass
+  L.sort_items = (esz == 2 && g_label_outside) ? (int)round_up(T, kSortBlock) : 0;
+  int vbits = 1;
+  while (vbits < 32 && ((int64_t)1 << vbits) < V) ++vbits;
+  L.sort_passes = (vbits + 1 + 7) / 8;
+  for (int b = 0; b < 2; ++b) {
+    L.off_keys[b] = o; o += align256((size_t)L.sort_items * 4);
+    L.off_vals[b] = o; o += align256((size_t)L.sort_items * 4);
+  }
+  L.off_hist = o;  o += align256((size_t)(L.sort_items / kSortBlock) * 256 * 4);
+  L.off_flags = o; o += L.sort_items ? align256((size_t)V) : 0;  // one byte per weight row: holds a one-hot sum
   L.total = o;
   return L;
 }
@@ -331,6 +345,43 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                        (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), dentropy, T, rows, inv, n_rows);
     if ((rc = check_launch("active_rows_kernel"))) return rc;
   }
+  // tokens grouped by label for the one-hot part of d_weight (added after the GEMMs)
+  LabelTerm lt;
+  lt.labels = nullptr; lt.v0 = vocab_offset; lt.V = V; lt.g_lp = dlogprobs;
+  lt.g_stride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
+  lt.scale = (reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f) / temperature;
+  uint32_t* skeys[2] = {reinterpret_cast<uint32_t*>(ws + L.off_keys[0]), reinterpret_cast<uint32_t*>(ws + L.off_keys[1])};
+  int* svals[2] = {reinterpret_cast<int*>(ws + L.off_vals[0]), reinterpret_cast<int*>(ws + L.off_vals[1])};
+  unsigned char* row_flags = L.sort_items ? reinterpret_cast<unsigned char*>(ws + L.off_flags) : nullptr;
+  if (L.sort_items) {
+    lt.labels = labels;
+    ProfScope prof(PC_LABEL_ROWS, st);
+    const int nblocks = L.sort_items / kSortBlock;
+    if (nblocks == 1) {
+      hipLaunchKernelGGL(label_sort_single_kernel, dim3(1), dim3(256), 0, st, lt, rows, n_rows, T, L.sort_passes, skeys[0], svals[0],
+                         skeys[1], svals[1]);
+      if ((rc = check_launch("label_sort_single_kernel"))) return rc;
+    } else {
+      int* hist = reinterpret_cast<int*>(ws + L.off_hist);
+      hipLaunchKernelGGL(label_keys_kernel, dim3(L.sort_items / 256), dim3(256), 0, st, lt, rows, n_rows, T, L.sort_items, skeys[0], svals[0]);
+      if ((rc = check_launch("label_keys_kernel"))) return rc;
+      for (int ps = 0; ps < L.sort_passes; ++ps) {
+        const int in = ps & 1, out = in ^ 1;
+        hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(256), 0, st, skeys[in], 8 * ps, nblocks, hist);
+        hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(1024), 0, st, hist, 256 * nblocks);
+        hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(256), 0, st, skeys[in], svals[in], skeys[out], svals[out], 8 * ps,
+                           nblocks, hist);
+        if ((rc = check_launch("label sort pass"))) return rc;
+      }
+    }
+    // the label rows of d_weight get their one-hot sums now; the GEMM epilogues add the softmax terms to them
+    const int res = L.sort_passes & 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(V / 1024 + 1 < 1024 ? V / 1024 + 1 : 1024)), dim3(256), 0, st, reinterpret_cast<uint32_t*>(row_flags),
+                       (int64_t)(align256((size_t)V) / 4));
+    hipLaunchKernelGGL(dw_label_rows_kernel<TIN>, dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h, ldh, H,
+                       d_weight, row_flags);
+    if ((rc = check_launch("dw_label_rows_kernel"))) return rc;
+  }
   // second operand of the d_weight GEMM (W^T for d_hidden follows chunk by chunk): the listed rows of hidden,
   // as they are (K-major, for the transposing reads), or transposed to h^T [H][T]
   if (L.tn) {
@@ -352,6 +403,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   for (int c = 0; c <= L.nchunks; ++c) {
     BwdChunkArgs<TIN> p;
     p.n_gw = p.n_gh = p.n_ds = 0;
+    p.row_flags = nullptr;
     bool swapped = false;
     if (c < L.nchunks) {
       const int64_t v0 = (int64_t)c * L.vchunk;
@@ -365,6 +417,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_ent = dentropy;
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = L.tn ? nullptr : dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       d.rows = rows; d.n_rows = n_rows;
+      d.label_outside = lt.labels != nullptr;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
       // faster on the launch while `hidden` is small enough to stay in the memory-side cache next to the
@@ -378,6 +431,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int cc = c - 1;
       const int64_t v0 = (int64_t)cc * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
+      p.row_flags = row_flags ? row_flags + v0 : nullptr;
       // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . W[v0 : v0 + Kc][H]  (rows = listed tokens)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
       if (L.tn_dh) {
@@ -442,7 +496,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     int64_t blocks = (T * (H / 4) + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     hipLaunchKernelGGL(dh_finish_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
-                       (int64_t)(align256((size_t)T * H * 4) / 4), inv, T, H, d_hidden);
+                       (int64_t)(align256((size_t)T * H * 4) / 4), inv, T, H, d_hidden, lt, W, ldw);
     if ((rc = check_launch("dh_finish_kernel"))) return rc;
   }
   return LCE_OK;
@@ -530,6 +584,7 @@ int lce_set_option(int key, int64_t value) {
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
     case LCE_OPT_DW_TRANSPOSED_READS: g_dw_transposed_reads = value != 0; return LCE_OK;
+    case LCE_OPT_LABEL_TERM_OUTSIDE: g_label_outside = value != 0; return LCE_OK;
     case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
@@ -544,7 +599,7 @@ int lce_profile_num_classes(void) { return PC_COUNT; }
 const char* lce_profile_class_name(int cls) {
   static const char* names[PC_COUNT] = {"lce_fwd_kernel", "lce_fwd_merge_kernel", "lce_bwd_ds_kernel", "gemm_nt_kernel(d_hidden)",
                                         "gemm_nt_kernel(d_weight)", "transpose_pad_kernel", "logits_fwd_kernel", "logits_bwd_kernel",
-                                        "lce_bwd_chunk_kernel", "active_rows_kernel", "dh_finish_kernel"};
+                                        "lce_bwd_chunk_kernel", "active_rows_kernel", "dh_finish_kernel", "label_rows_kernels"};
   return (cls >= 0 && cls < PC_COUNT) ? names[cls] : "";
 }
 int lce_profile_read(double* total_ms, int64_t* launches, int reset) {
