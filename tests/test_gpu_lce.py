@@ -510,6 +510,29 @@ def test_d_hidden_operand_mode_switches_with_token_count(T):
     assert torch.count_nonzero(dh[~keep]) == 0
 
 
+@pytest.mark.parametrize("T,V,labels", [(3000, 300, "random"), (700, 5000, "one"), (2500, 1024, "two"), (5000, 70000, "random")])
+def test_many_tokens_share_a_label(T, V, labels):
+    """The one-hot part of d_weight is summed per label over a label-sorted token list (one workgroup up to 1024
+    tokens, several radix passes beyond): labels that repeat tens of times, all tokens on one label, two labels
+    with cancelling gradients, and a third of the tokens without gradient; bit-identical on a second run."""
+    H, tau = 256, 0.7
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=T + V)
+    g_lp, g_ent = g_lp.float() * 4, g_ent.float()
+    if labels == "one":
+        y = torch.full_like(y, 1234)
+    elif labels == "two":
+        y = torch.where(torch.arange(T, device=DEV) % 2 == 0, 7, V - 1)
+        g_lp = torch.where(torch.arange(T, device=DEV) % 4 < 2, g_lp.abs(), -g_lp.abs())
+    keep = (torch.arange(T, device=DEV) % 3) != 1
+    g_lp, g_ent = g_lp * keep, g_ent * keep
+    _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    assert_bf16_bar(dh, rdh)
+    assert_bf16_bar(dw, rdw)
+    _, _, dh2, dw2 = _run(h, w, y, tau, g_lp, g_ent)
+    assert torch.equal(dh, dh2) and torch.equal(dw, dw2)
+
+
 def test_every_tile_variant_agrees():
     from verl_amd import _abi
 
