@@ -7,7 +7,7 @@
 // of large terms.  So the tiles hold the softmax terms only, and the one-hot part is added in fp32:
 //   d_hidden[t][:]        += G_t * W[label_t][:]        (when the fp32 partials are summed and rounded)
 //   d_weight[label][:]    += sum over tokens t with that label, in ascending t, of G_t * hidden[t][:]
-//                            (written first; the GEMM epilogue adds the softmax terms to these rows)
+//                            (after the GEMMs have written the softmax terms)
 // The second sum needs the tokens grouped by label in a fixed order: a stable LSD radix sort of
 // (label row, position in the token list) pairs, 8 bits per pass, written here (no float atomics anywhere, and
 // no library call that a captured graph could not replay).
@@ -172,21 +172,21 @@ __global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm lt, co
   }
 }
 
-// d_weight[row][:] = (T)(sum of G_t * hidden[t][:] over the run of sorted positions with key == row, in order) and
-// flags[row] = 1.  One workgroup per sorted position; only the first position of a run works.  Runs before the
-// d_weight GEMMs, whose epilogues add their accumulators to the flagged rows and round once more (the first
-// rounding is that of a complete sum, 2^-9 of its own magnitude).
+// d_weight[row][:] += sum of G_t * hidden[t][:] over the run of sorted positions with key == row, in order.
+// One workgroup per sorted position; only the first position of a run works.  Runs after the d_weight GEMMs:
+// the rows are read back in the output dtype (rounded once by the GEMM that wrote the softmax terms, which are
+// small next to the one-hot sums on all but a few rows) and rounded once more with the sum added in fp32.
 template <typename T>
 __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys, const int* toks, int n_items, LabelTerm lt, const T* h,
-                                                            int64_t ldh, int64_t H, T* dW, unsigned char* flags) {
+                                                            int64_t ldh, int64_t H, T* dW) {
   constexpr int N = 16 / (int)sizeof(T);
   typedef typename VecOf<T, N>::type vec_t;
   const int i = blockIdx.x;
   const uint32_t key = keys[i];
   if (key == kNoRow || (i > 0 && keys[i - 1] == key)) return;
   T* row = dW + (int64_t)key * H;
-  if (threadIdx.x == 0) flags[key] = 1;
   for (int64_t c = (int64_t)threadIdx.x * N; c < H; c += 256 * N) {
+    const vec_t cur = *reinterpret_cast<const vec_t*>(row + c);
     float acc[N];
 #pragma unroll
     for (int e = 0; e < N; ++e) acc[e] = 0.f;
@@ -197,6 +197,8 @@ __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys
 #pragma unroll
       for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(G, (float)hv[e], acc[e]);
     }
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] += (float)cur[e];
     store_run<T, N>(row + c, acc);
   }
 }

@@ -217,7 +217,7 @@ int forward_splits_upper_bound(int64_t T) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_keys[2], off_vals[2], off_hist, off_flags, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_keys[2], off_vals[2], off_hist, total;
   int sort_items, sort_passes;  // label sort (0 items: the one-hot part stays inside the d_logits tiles)
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
@@ -293,7 +293,6 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
     L.off_vals[b] = o; o += align256((size_t)L.sort_items * 4);
   }
   L.off_hist = o;  o += align256((size_t)(L.sort_items / kSortBlock) * 256 * 4);
-  L.off_flags = o; o += L.sort_items ? align256((size_t)V) : 0;  // one byte per weight row: holds a one-hot sum
   L.total = o;
   return L;
 }
@@ -352,7 +351,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   lt.scale = (reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f) / temperature;
   uint32_t* skeys[2] = {reinterpret_cast<uint32_t*>(ws + L.off_keys[0]), reinterpret_cast<uint32_t*>(ws + L.off_keys[1])};
   int* svals[2] = {reinterpret_cast<int*>(ws + L.off_vals[0]), reinterpret_cast<int*>(ws + L.off_vals[1])};
-  unsigned char* row_flags = L.sort_items ? reinterpret_cast<unsigned char*>(ws + L.off_flags) : nullptr;
   if (L.sort_items) {
     lt.labels = labels;
     ProfScope prof(PC_LABEL_ROWS, st);
@@ -374,13 +372,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         if ((rc = check_launch("label sort pass"))) return rc;
       }
     }
-    // the label rows of d_weight get their one-hot sums now; the GEMM epilogues add the softmax terms to them
-    const int res = L.sort_passes & 1;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(V / 1024 + 1 < 1024 ? V / 1024 + 1 : 1024)), dim3(256), 0, st, reinterpret_cast<uint32_t*>(row_flags),
-                       (int64_t)(align256((size_t)V) / 4));
-    hipLaunchKernelGGL(dw_label_rows_kernel<TIN>, dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h, ldh, H,
-                       d_weight, row_flags);
-    if ((rc = check_launch("dw_label_rows_kernel"))) return rc;
   }
   // second operand of the d_weight GEMM (W^T for d_hidden follows chunk by chunk): the listed rows of hidden,
   // as they are (K-major, for the transposing reads), or transposed to h^T [H][T]
@@ -403,7 +394,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   for (int c = 0; c <= L.nchunks; ++c) {
     BwdChunkArgs<TIN> p;
     p.n_gw = p.n_gh = p.n_ds = 0;
-    p.row_flags = nullptr;
     bool swapped = false;
     if (c < L.nchunks) {
       const int64_t v0 = (int64_t)c * L.vchunk;
@@ -431,7 +421,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int cc = c - 1;
       const int64_t v0 = (int64_t)cc * L.vchunk;
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
-      p.row_flags = row_flags ? row_flags + v0 : nullptr;
       // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . W[v0 : v0 + Kc][H]  (rows = listed tokens)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
       if (L.tn_dh) {
@@ -498,6 +487,14 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     hipLaunchKernelGGL(dh_finish_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
                        (int64_t)(align256((size_t)T * H * 4) / 4), inv, T, H, d_hidden, lt, W, ldw);
     if ((rc = check_launch("dh_finish_kernel"))) return rc;
+  }
+  if (L.sort_items) {
+    // one-hot part of d_weight: every chunk's rows hold their softmax terms by now
+    ProfScope prof(PC_LABEL_ROWS, st);
+    const int res = L.sort_passes & 1;
+    hipLaunchKernelGGL(dw_label_rows_kernel<TIN>, dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h, ldh, H,
+                       d_weight);
+    if ((rc = check_launch("dw_label_rows_kernel"))) return rc;
   }
   return LCE_OK;
 }

@@ -330,22 +330,22 @@ template <typename Cfg>
 struct KPerm {
   static constexpr int GT = Cfg::WN, GV = Cfg::WM;
   // token t (lane ln = t % 32 of block column j = (t % GT) / 32)  ->  ln * FN + j
-  static __host__ __device__ int64_t token(int64_t t) {
+  static __host__ __device__ __forceinline__ int64_t token(int64_t t) {
     const int64_t l = t % GT;
     return t - l + (l % 32) * Cfg::FN + l / 32;
   }
   // vocabulary row v = i*32 + 8*(r/4) + 4*hh + r%4 of its group  ->  hh * 16*FM + i*16 + r
-  static __host__ __device__ int64_t vocab(int64_t v) {
+  static __host__ __device__ __forceinline__ int64_t vocab(int64_t v) {
     const int64_t l = v % GV;
     const int64_t i = l / 32, w = l % 32, hh = (w >> 2) & 1, r = (w >> 3) * 4 + (w & 3);
     return v - l + hh * 16 * Cfg::FM + i * 16 + r;
   }
   // inverses: which token / vocabulary row sits at position u
-  static __host__ __device__ int64_t token_at(int64_t u) {
+  static __host__ __device__ __forceinline__ int64_t token_at(int64_t u) {
     const int64_t l = u % GT;
     return u - l + (l % Cfg::FN) * 32 + l / Cfg::FN;
   }
-  static __host__ __device__ int64_t vocab_at(int64_t u) {
+  static __host__ __device__ __forceinline__ int64_t vocab_at(int64_t u) {
     const int64_t l = u % GV;
     const int64_t hh = l / (16 * Cfg::FM), rem = l % (16 * Cfg::FM), i = rem / 16, r = rem % 16;
     return u - l + i * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
@@ -546,24 +546,11 @@ struct GemmArgs {
   int64_t b_rows_valid;  // tn == 2: rows of B that exist (K may be rounded up beyond them; A is zero there)
 };
 
-// Out_mode 2 (d_weight) only: row_flags[m] != 0 marks rows of Ct that already hold a value (the one-hot part of
-// d_weight, label_rows.hpp); the accumulator is added to it before the one rounding, other rows are only written.
-// bit u of the mask: row (first + u) of a 64-row wave tile is such a row.
-LCE_DEV uint64_t row_flag_mask(const unsigned char* flags, int64_t first, int64_t M) {
-  if (!flags) return 0;
-  const int lane = threadIdx.x & 63;
-  const int64_t m = first + lane;
-  return __builtin_amdgcn_ballot_w64(m < M && flags[m] != 0);
-}
-
 template <typename Cfg, int MODE, bool EDGE>
 LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t m0,
-                           int64_t n0, int wave_m, int wave_n, int hh, int ln, uint64_t held0 = 0, uint64_t held1 = 0) {
+                           int64_t n0, int wave_m, int wave_n, int hh, int ln) {
   typedef typename Cfg::TIN TIN;
   const int64_t mw = m0 + wave_m * Cfg::WM + 4 * hh;  // row of register 0 of block row 0
-  static_assert(Cfg::WM % 64 == 0 && Cfg::WM <= 128, "row flag mask");
-  const uint64_t held[2] = {held0, held1};  // rows of the wave tile that hold a value to add to (out_mode 2)
-  const bool any_held = (held0 | held1) != 0;
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
     const int64_t n = n0 + wave_n * Cfg::WN + j * 32 + ln;
@@ -573,23 +560,12 @@ LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t 
       __builtin_amdgcn_sched_barrier(0);  // one 32x32 block at a time (register pressure)
       float* cf = (MODE != 2) ? p.Cf + (mw + i * 32) * p.ldcf + n : nullptr;
       TIN* ct = (MODE & 2) ? p.Ct + (mw + i * 32) * p.ldct + n : nullptr;
-      float add[16];  // what the flagged rows hold already: all loads of the block go out before the first store
-#pragma unroll
-      for (int r = 0; r < 16; ++r) add[r] = 0.f;
-      if (MODE == 2 && any_held) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if ((!EDGE || mw + i * 32 + 8 * q + u < p.M) && ((held[i / 2] >> (4 * hh + (i % 2) * 32 + 8 * q + u)) & 1))
-              add[q * 4 + u] = (float)ct[(8 * q + u) * p.ldct];
-      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           if (EDGE && mw + i * 32 + 8 * q + u >= p.M) continue;
-          float v = acc[i][j][q * 4 + u] + add[q * 4 + u];
+          float v = acc[i][j][q * 4 + u];
           if (MODE & 1) v += cf[(8 * q + u) * p.ldcf];
           if (MODE & 2) ct[(8 * q + u) * p.ldct] = (TIN)v;
           else cf[(8 * q + u) * p.ldcf] = v;
@@ -600,7 +576,7 @@ LCE_DEV void gemm_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t 
 }
 
 template <typename Cfg>
-LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds, const unsigned char* row_flags = nullptr) {
+LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
   GemmArgs<typename Cfg::TIN> p = pin;
   if (p.m_dev) {
     const int64_t m = *p.m_dev;
@@ -625,9 +601,6 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
   g.init(p.A + k0, p.lda, m0, p.M, p.B + k0, p.ldb, n0, p.N);
-  // (read ahead of the K loop: the flags are needed by the epilogue only)
-  const uint64_t held0 = p.out_mode == 2 ? row_flag_mask(row_flags, m0 + g.wave_m * Cfg::WM, p.M) : 0;
-  const uint64_t held1 = p.out_mode == 2 && Cfg::WM > 64 ? row_flag_mask(row_flags, m0 + g.wave_m * Cfg::WM + 64, p.M) : 0;
   f32x16_t acc[Cfg::FM][Cfg::FN];
   if (k0 < k1) {
     g.run(lds, k1 - k0, acc);
@@ -642,8 +615,8 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
   }
   const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
 #define LCE_EPI(MODE)                                                                           \
-  if (edge) gemm_epilogue<Cfg, MODE, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held0, held1);  \
-  else gemm_epilogue<Cfg, MODE, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held0, held1)
+  if (edge) gemm_epilogue<Cfg, MODE, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);         \
+  else gemm_epilogue<Cfg, MODE, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln)
   switch (p.out_mode) {
     case 0: LCE_EPI(0); break;
     case 1: LCE_EPI(1); break;
@@ -658,9 +631,8 @@ LCE_DEV void gemm_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* ld
 // out_mode 2: Ct[KPerm::vocab_at(m)][n] = (TIN)acc (see GemmArgs::tn).
 template <typename Cfg, typename PermCfg, int MODE, bool EDGE>
 LCE_DEV void gemm_tn_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16_t (&acc)[Cfg::FM][Cfg::FN], int64_t m0, int64_t n0,
-                              int wave_m, int wave_n, int hh, int ln, uint64_t held) {
+                              int wave_m, int wave_n, int hh, int ln) {
   typedef typename Cfg::TIN TIN;
-  static_assert(Cfg::WM == 64, "row flag mask");  // held: rows of the wave tile that hold a value to add to (out_mode 2)
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
     const int64_t n = n0 + wave_n * Cfg::WN + j * 32 + ln;
@@ -668,24 +640,13 @@ LCE_DEV void gemm_tn_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16
 #pragma unroll
     for (int i = 0; i < Cfg::FM; ++i) {
       __builtin_amdgcn_sched_barrier(0);  // one 32x32 block at a time (register pressure)
-      float add[16];  // what the flagged rows hold already: all loads of the block go out before the first store
-#pragma unroll
-      for (int r = 0; r < 16; ++r) add[r] = 0.f;
-      if (MODE == 2 && held != 0) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int um = (int)KPerm<PermCfg>::vocab_at(acc_row(i, r, hh));
-          const int64_t m = m0 + wave_m * Cfg::WM + um;
-          if ((!EDGE || m < p.M) && ((held >> um) & 1)) add[r] = (float)p.Ct[m * p.ldct + n];
-        }
-      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int u = acc_row(i, r, hh);  // row inside the wave tile
         const int um = MODE == 2 ? (int)KPerm<PermCfg>::vocab_at(u) : u;
         const int64_t m = m0 + wave_m * Cfg::WM + um;
         if (EDGE && m >= p.M) continue;
-        if (MODE == 2) p.Ct[m * p.ldct + n] = (TIN)(acc[i][j][r] + add[r]);
+        if (MODE == 2) p.Ct[m * p.ldct + n] = (TIN)acc[i][j][r];
         else p.Cf[m * p.ldcf + n] = acc[i][j][r];
       }
     }
@@ -693,7 +654,7 @@ LCE_DEV void gemm_tn_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16
 }
 
 template <typename Cfg, typename PermCfg>
-LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds, const unsigned char* row_flags = nullptr) {
+LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
   GemmArgs<typename Cfg::TIN> p = pin;
   if (p.k_dev) {
     const int64_t k = ((int64_t)*p.k_dev + p.k_gran - 1) / p.k_gran * p.k_gran;
@@ -705,7 +666,6 @@ LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char*
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
   g.init_tn(p.A, p.lda, m0, p.B, p.ldb, n0);
-  const uint64_t held = p.out_mode == 2 ? row_flag_mask(row_flags, m0 + g.wave_m * Cfg::WM, p.M) : 0;  // ahead of the K loop
   f32x16_t acc[Cfg::FM][Cfg::FN];
   if (p.K > 0) {
     g.run(lds, p.K, acc);
@@ -719,11 +679,11 @@ LCE_DEV void gemm_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char*
   }
   const bool edge = m0 + Cfg::BM > p.M || n0 + Cfg::BN > p.N;
   if (p.out_mode == 2) {
-    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 2, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held);
-    else gemm_tn_epilogue<Cfg, PermCfg, 2, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held);
+    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 2, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_tn_epilogue<Cfg, PermCfg, 2, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
   } else {
-    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held);
-    else gemm_tn_epilogue<Cfg, PermCfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln, held);
+    if (edge) gemm_tn_epilogue<Cfg, PermCfg, 0, true>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
+    else gemm_tn_epilogue<Cfg, PermCfg, 0, false>(p, acc, m0, n0, g.wave_m, g.wave_n, hh, ln);
   }
 }
 
@@ -757,9 +717,6 @@ struct BwdChunkArgs {
   GemmArgs<TIN> gh;
   DsArgs<TIN> ds;    // d_logits of chunk c                     (K = H, heavy epilogue)
   int n_gw, n_gh, n_ds;
-  // rows of the d_weight chunk that hold their one-hot sums already (see row_flag_mask), or null; only the
-  // GEMM with out_mode 2 looks at it
-  const unsigned char* row_flags;
 };
 
 // C[m][n] (+)= sum_k A[m][k] * B[k][n]: A row-major, B K-major as it lies in memory (Cfg::TRANS == 2).  Column k of A
@@ -819,10 +776,10 @@ struct TransOf {
 };
 
 template <typename Cfg>
-LCE_DEV void any_gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds, const unsigned char* row_flags) {
+LCE_DEV void any_gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   if constexpr (sizeof(typename Cfg::TIN) == 2 && Cfg::BM == 256 && Cfg::BN == 256 && Cfg::WAVES_M == 4 && Cfg::WAVES_N == 2) {
     if (p.tn == 1) {
-      gemm_tn_tile<typename TransOf<Cfg>::type, Cfg>(p, bid, lds, row_flags);
+      gemm_tn_tile<typename TransOf<Cfg>::type, Cfg>(p, bid, lds);
       return;
     }
     if (p.tn == 2) {
@@ -830,15 +787,15 @@ LCE_DEV void any_gemm_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* 
       return;
     }
   }
-  gemm_tile<Cfg>(p, bid, lds, row_flags);
+  gemm_tile<Cfg>(p, bid, lds);
 }
 
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NTHREADS) void lce_bwd_chunk_kernel(BwdChunkArgs<typename Cfg::TIN> p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int bid = blockIdx.x;
-  if (bid < p.n_gw) any_gemm_tile<Cfg>(p.gw, bid, lds, p.row_flags);
-  else if (bid < p.n_gw + p.n_gh) any_gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds, p.row_flags);
+  if (bid < p.n_gw) any_gemm_tile<Cfg>(p.gw, bid, lds);
+  else if (bid < p.n_gw + p.n_gh) any_gemm_tile<Cfg>(p.gh, bid - p.n_gw, lds);
   else ds_tile<Cfg>(p.ds, bid - p.n_gw - p.n_gh, lds);
 }
 
