@@ -284,7 +284,7 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   L.off_inv = o;   o += align256((size_t)T * 4);
   L.off_nrows = o; o += 256;
   // (label row, token) pairs, two buffers each, and the per-block digit counts of one radix pass
-  L.sort_items = (esz == 2 && g_label_outside) ? (int)round_up(T, kSortBlock) : 0;
+  L.sort_items = (esz == 2 && g_label_outside && T <= ((int64_t)1 << 30)) ? (int)round_up(T, kSortBlock) : 0;
   int vbits = 1;
   while (vbits < 32 && ((int64_t)1 << vbits) < V) ++vbits;
   L.sort_passes = (vbits + 1 + 7) / 8;
