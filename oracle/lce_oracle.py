@@ -284,14 +284,18 @@ def ppo_actor_loss(
     entropy_coeff: float = 0.0,
     loss_agg_mode: str = "token-mean",
     clip_ratio_c: float = 3.0,
+    rollout_is_weights=None,
+    **global_batch_info,
 ):
-    """policy loss - entropy_coeff * agg(entropy): the scalar the actor back-propagates."""
+    """policy loss - entropy_coeff * agg(entropy): the scalar the actor back-propagates
+    (verl/workers/utils/losses.py:109-140; both terms aggregated with the same mode and global batch info)."""
     pg, metrics = policy_loss_vanilla(
-        old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, clip_ratio, clip_ratio_c=clip_ratio_c
-    )
+        old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, clip_ratio, clip_ratio_c=clip_ratio_c,
+        rollout_is_weights=rollout_is_weights, **global_batch_info,
+    )  # fmt: skip
     loss = pg
     if entropy is not None:
-        ent = agg_loss(entropy, response_mask, loss_agg_mode)
+        ent = agg_loss(entropy, response_mask, loss_agg_mode, **global_batch_info)
         loss = loss - entropy_coeff * ent
         metrics["actor/entropy_loss"] = ent.detach().item()
     metrics["actor/pg_loss"] = pg.detach().item()

@@ -56,14 +56,74 @@ def test_global_batch_scaling_and_errors():
     torch.testing.assert_close(loss, want, atol=1e-6, rtol=1e-5)
     with pytest.raises(ValueError):
         fused_ppo_loss(lp, ent, old, adv, mask, dp_size=2)
-    with pytest.raises(NotImplementedError):
-        fused_ppo_loss(lp, ent, old, adv, mask, loss_agg_mode="seq-mean-token-sum")
+    with pytest.raises(ValueError, match="global_batch_size is required"):
+        fused_ppo_loss(lp, ent, old, adv, mask, dp_size=2, loss_agg_mode="seq-mean-token-sum")
+    with pytest.raises(ValueError, match="Invalid loss_agg_mode"):  # core_algos.py:1203-1204
+        fused_ppo_loss(lp, ent, old, adv, mask, loss_agg_mode="nope")
     # NaNs outside the mask do not leak (masked_sum semantics, verl/utils/torch_functional.py:273-291)
     lp_nan = lp.clone()
     lp_nan[mask == 0] = float("nan")
     loss_nan, _ = fused_ppo_loss(lp_nan, ent, old, adv, mask, entropy_coeff=0.01)
     loss_ok, _ = fused_ppo_loss(lp, ent, old, adv, mask, entropy_coeff=0.01)
     torch.testing.assert_close(loss_nan, loss_ok)
+
+
+AGG_CASES = [
+    ("token-mean", {}),
+    ("token-mean", dict(dp_size=4, batch_num_tokens=5000)),
+    ("token-sum", {}),
+    ("token-sum", dict(dp_size=2)),
+    ("seq-mean-token-sum", {}),
+    ("seq-mean-token-sum", dict(dp_size=2, global_batch_size=64)),
+    ("seq-mean-token-sum-norm", {}),
+    ("seq-mean-token-sum-norm", dict(loss_scale_factor=1000)),
+    ("seq-mean-token-sum-norm", dict(dp_size=8, global_batch_size=128, loss_scale_factor=512)),
+    ("seq-mean-token-mean", {}),
+    ("seq-mean-token-mean", dict(dp_size=2, global_batch_size=40)),
+]
+
+
+@pytest.mark.parametrize("mode,info", AGG_CASES)
+@pytest.mark.parametrize("B,L", [(16, 257), (3, 5000), (5000, 3), (1, 1)])
+def test_every_aggregation_mode(mode, info, B, L):
+    """agg_loss's five modes (verl/trainer/ppo/core_algos.py:1172-1204) with and without the global batch
+    information, rows without any valid token included, rollout correction weights on the policy term."""
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask = _case(B, L, seed=B + L, spread=0.6)
+    if B > 2:
+        mask[1] = 0  # a fully masked sequence: left out of every sequence mean
+    isw = torch.rand(B, L, device=DEV) * 2
+    lp1, ent1 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    loss, met = fused_ppo_loss(lp1, ent1, old, adv, mask.bool(), entropy_coeff=1e-2, loss_agg_mode=mode,
+                               rollout_is_weights=isw, **info)  # fmt: skip
+    loss.backward()
+    lp2, ent2 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    rloss, rmet = O.ppo_actor_loss(lp2, ent2, old, adv, mask, entropy_coeff=1e-2, loss_agg_mode=mode,
+                                   rollout_is_weights=isw, **info)  # fmt: skip
+    rloss.backward()
+    torch.testing.assert_close(loss, rloss, atol=1e-6, rtol=2e-5)
+    for k, v in met.items():
+        assert v.item() == pytest.approx(rmet[k], rel=2e-5, abs=1e-6), k
+    scale = max(lp2.grad.abs().max().item(), 1e-30)
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-6 * scale, rtol=1e-5)
+    torch.testing.assert_close(ent1.grad, ent2.grad, atol=1e-6 * max(ent2.grad.abs().max().item(), 1e-30), rtol=1e-5)
+    assert (lp1.grad[mask == 0] == 0).all() and (ent1.grad[mask == 0] == 0).all()
+    # bit-identical on a second call (fixed reduction order)
+    loss_b, _ = fused_ppo_loss(lp, ent, old, adv, mask, entropy_coeff=1e-2, loss_agg_mode=mode,
+                               rollout_is_weights=isw, **info)  # fmt: skip
+    assert loss_b.item() == loss.item()
+
+
+def test_flat_token_list_equals_rows_in_token_modes():
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask = _case(7, 300, seed=11)
+    for mode in ("token-mean", "token-sum"):
+        a, _ = fused_ppo_loss(lp, ent, old, adv, mask, entropy_coeff=1e-3, loss_agg_mode=mode)
+        b, _ = fused_ppo_loss(lp.reshape(-1), ent.reshape(-1), old.reshape(-1), adv.reshape(-1), mask.reshape(-1),
+                              entropy_coeff=1e-3, loss_agg_mode=mode)  # fmt: skip
+        torch.testing.assert_close(a, b, atol=1e-6, rtol=1e-5)
 
 
 def test_actor_step_fused_end_to_end():

@@ -826,33 +826,67 @@ int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_
   return check_launch("logits_pi2_kernel");
 }
 
-size_t lce_ppo_loss_workspace_bytes(int64_t N) {
-  (void)N;
-  return 1024 * 8 * sizeof(float);
+// geometry of the PPO loss launches: workgroups per row and elements per workgroup
+static void ppo_geometry(int64_t rows, int64_t row_len, int* segs, int64_t* seg_len) {
+  int64_t want = (row_len + 1023) / 1024;        // about 4 elements per thread
+  int64_t cap = rows >= 4096 ? 1 : 4096 / rows;  // bounds what the single finishing workgroup walks
+  int64_t s = want < cap ? want : cap;
+  if (s < 1) s = 1;
+  *seg_len = (row_len + s - 1) / s;
+  *segs = (int)((row_len + *seg_len - 1) / *seg_len);
+}
+
+static size_t ppo_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t lce_ppo_loss_workspace_bytes(int64_t rows, int64_t row_len) {
+  if (rows <= 0 || row_len <= 0) return 0;
+  int segs;
+  int64_t seg_len;
+  ppo_geometry(rows, row_len, &segs, &seg_len);
+  return ppo_align((size_t)rows * segs * 8 * sizeof(float)) + ppo_align((size_t)rows * 3 * sizeof(double)) +
+         ppo_align((size_t)rows * sizeof(float));
 }
 
 int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
-                 const float* mask, int64_t N, float clip_low, float clip_high, float clip_c, float entropy_coeff,
-                 float token_scale, float* out, float* g_log_prob, float* g_entropy, void* workspace,
-                 size_t workspace_bytes, void* stream) {
-  if (N <= 0) return fail(LCE_E_ARG, "ppo loss: N must be positive");
+                 const float* mask, const float* is_weights, int64_t rows, int64_t row_len, int agg_mode,
+                 float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
+                 float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
+                 float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream) {
+  if (rows <= 0 || row_len <= 0) return fail(LCE_E_ARG, "ppo loss: rows and row_len must be positive");
+  if (rows > ((int64_t)1 << 30) || row_len > ((int64_t)1 << 40) / rows) return fail(LCE_E_ARG, "ppo loss: too many elements");
   if (!log_prob || !old_log_prob || !advantages || !mask || !out || !g_log_prob) return fail(LCE_E_ARG, "null pointer");
   if ((entropy == nullptr) != (g_entropy == nullptr)) return fail(LCE_E_ARG, "entropy and g_entropy go together");
   if (!(clip_c > 1.f)) return fail(LCE_E_ARG, "clip_ratio_c must be greater than 1");
-  if (!workspace || workspace_bytes < lce_ppo_loss_workspace_bytes(N)) return fail(LCE_E_WORKSPACE, "ppo workspace too small");
+  if (agg_mode < PPO_TOKEN_MEAN || agg_mode > PPO_SEQ_MEAN_TOKEN_MEAN) return fail(LCE_E_ARG, "Invalid loss_agg_mode: %d", agg_mode);
+  if (!(dp_size > 0.f)) return fail(LCE_E_ARG, "ppo loss: dp_size must be positive");
+  if (!workspace || workspace_bytes < lce_ppo_loss_workspace_bytes(rows, row_len))
+    return fail(LCE_E_WORKSPACE, "ppo workspace too small");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  int blocks = (int)((N + 255) / 256);
-  if (blocks > 1024) blocks = 1024;
   PpoArgs p;
+  ppo_geometry(rows, row_len, &p.segs, &p.seg_len);
+  const int64_t blocks = rows * p.segs;
+  if (blocks > 0x7fffffff) return fail(LCE_E_ARG, "ppo loss: too many rows");
+  char* ws = static_cast<char*>(workspace);
+  p.partials = reinterpret_cast<float*>(ws);
+  ws += ppo_align((size_t)blocks * 8 * sizeof(float));
+  double* row_tot = reinterpret_cast<double*>(ws);
+  ws += ppo_align((size_t)rows * 3 * sizeof(double));
+  float* row_weight = reinterpret_cast<float*>(ws);
   p.log_prob = log_prob; p.entropy = entropy; p.old_log_prob = old_log_prob; p.advantages = advantages; p.mask = mask;
-  p.N = N; p.clip_low = clip_low; p.clip_high = clip_high; p.clip_c = clip_c; p.entropy_coeff = entropy_coeff;
-  p.g_log_prob = g_log_prob; p.g_entropy = g_entropy; p.partials = static_cast<float*>(workspace);
-  hipLaunchKernelGGL(ppo_terms_kernel, dim3(blocks), dim3(256), 0, st, p);
+  p.is_weights = is_weights; p.rows = rows; p.row_len = row_len;
+  p.clip_low = clip_low; p.clip_high = clip_high; p.clip_c = clip_c; p.entropy_coeff = entropy_coeff;
+  p.g_log_prob = g_log_prob; p.g_entropy = g_entropy;
+  PpoAgg g;
+  g.mode = agg_mode; g.dp_size = dp_size; g.batch_num_tokens = batch_num_tokens; g.global_batch_size = global_batch_size;
+  g.loss_scale_factor = loss_scale_factor; g.entropy_coeff = entropy_coeff;
+  hipLaunchKernelGGL(ppo_terms_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
   int rc = check_launch("ppo_terms_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL(ppo_finish_kernel, dim3(1), dim3(64), 0, st, p.partials, blocks, token_scale, entropy_coeff, out);
+  hipLaunchKernelGGL(ppo_finish_kernel, dim3(1), dim3(256), 0, st, p.partials, rows, p.segs, row_len, g, row_tot,
+                     row_weight, out);
   if ((rc = check_launch("ppo_finish_kernel"))) return rc;
-  hipLaunchKernelGGL(ppo_scale_kernel, dim3(blocks), dim3(256), 0, st, g_log_prob, g_entropy, N, out);
+  hipLaunchKernelGGL(ppo_scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g_log_prob, g_entropy, rows, row_len,
+                     p.segs, p.seg_len, row_weight);
   return check_launch("ppo_scale_kernel");
 }
 

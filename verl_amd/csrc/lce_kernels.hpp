@@ -1164,26 +1164,37 @@ __global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64
 }
 
 // ------------------------------------------------------------------------------------------------
-// consumer of the path's outputs: clipped PPO policy loss + entropy bonus, token-mean aggregation
+// consumer of the path's outputs: clipped PPO policy loss + entropy bonus, every aggregation mode of agg_loss
 // ------------------------------------------------------------------------------------------------
+enum { PPO_TOKEN_MEAN = 0, PPO_TOKEN_SUM = 1, PPO_SEQ_MEAN_TOKEN_SUM = 2, PPO_SEQ_MEAN_TOKEN_SUM_NORM = 3,
+       PPO_SEQ_MEAN_TOKEN_MEAN = 4 };
+
 struct PpoArgs {
   const float* log_prob;
   const float* entropy;  // may be null
   const float* old_log_prob;
   const float* advantages;
   const float* mask;
-  int64_t N;
+  const float* is_weights;  // may be null: per-token factor on the policy loss (rollout correction), a constant
+  int64_t rows, row_len;    // [rows][row_len], row-major, contiguous
+  int segs;                 // workgroups per row
+  int64_t seg_len;          // elements per workgroup (the last one of a row may be short)
   float clip_low, clip_high, clip_c, entropy_coeff;
   float* g_log_prob;  // unscaled d(sum of masked losses)/d log_prob
   float* g_entropy;   // may be null
-  float* partials;    // [blocks][8]
+  float* partials;    // [rows * segs][8]
 };
 
-// one element; returns the masked per-token terms and the unscaled gradients
+// Per-token terms and unscaled gradients; workgroup (row, seg) reduces its segment of one row to
+// partials[row * segs + seg][0..5] = sums of (loss, entropy, clipped, -log ratio, dual-clipped, 1) x mask.
 __global__ void ppo_terms_kernel(PpoArgs p) {
   __shared__ float sh[8][256];
   float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < p.N; t += (int64_t)gridDim.x * blockDim.x) {
+  const int64_t row = (int64_t)blockIdx.x / p.segs;
+  const int64_t c0 = ((int64_t)blockIdx.x % p.segs) * p.seg_len;
+  const int64_t c1 = c0 + p.seg_len < p.row_len ? c0 + p.seg_len : p.row_len;
+  for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
+    const int64_t t = row * p.row_len + c;
     const float m = p.mask[t];
     const float lp = p.log_prob[t], A = p.advantages[t];
     const float d = lp - p.old_log_prob[t];
@@ -1196,8 +1207,9 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
     const float lc1 = fmaxf(l1, l2);
     const float dlc1 = l1 > l2 ? -A * dr : (l2 > l1 ? -A * drc : -A * 0.5f * (dr + drc));
     const bool dual = A < 0.f;
-    const float loss = dual ? fminf(l3, lc1) : lc1;
-    const float dloss = (dual && l3 < lc1) ? 0.f : dlc1;
+    const float isw = p.is_weights ? p.is_weights[t] : 1.f;
+    const float loss = (dual ? fminf(l3, lc1) : lc1) * isw;
+    const float dloss = ((dual && l3 < lc1) ? 0.f : dlc1) * isw;
     const bool on = m != 0.f;  // values outside the mask never reach a sum (NaNs there are harmless)
     p.g_log_prob[t] = on ? dloss * m : 0.f;
     float ent = 0.f;
@@ -1223,37 +1235,102 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
       for (int k = 0; k < 8; ++k) sh[k][threadIdx.x] += sh[k][threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x < 8) p.partials[blockIdx.x * 8 + threadIdx.x] = sh[threadIdx.x][0];
+  if (threadIdx.x < 8) p.partials[(int64_t)blockIdx.x * 8 + threadIdx.x] = sh[threadIdx.x][0];
 }
 
-// out: [0] loss, [1] pg_loss, [2] entropy_loss, [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower,
-//      [6] number of masked tokens, [7] scale applied to the per-token sums
-__global__ void ppo_finish_kernel(const float* partials, int blocks, float token_scale, float entropy_coeff, float* out) {
-  __shared__ double tot[8];
-  if (threadIdx.x < 8) {
-    double a = 0.0;
-    for (int b = 0; b < blocks; ++b) a += (double)partials[b * 8 + threadIdx.x];
-    tot[threadIdx.x] = a;
-  }
+struct PpoAgg {
+  int mode;
+  float dp_size;            // factor on every mode
+  float batch_num_tokens;   // token-mean denominator, <= 0: sum(mask)
+  float global_batch_size;  // seq-mean denominator, <= 0: number of rows with sum(mask) > 0
+  float loss_scale_factor;  // seq-mean-token-sum-norm divisor, <= 0: row_len
+  float entropy_coeff;
+};
+
+// fixed-order sum of NV doubles per thread over the workgroup (256 threads); result valid in every thread
+template <int NV>
+__device__ inline void ppo_block_sum(double (&v)[NV], double (*sh)[256]) {
   __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NV; ++k) sh[k][threadIdx.x] = v[k];
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w)
+#pragma unroll
+      for (int k = 0; k < NV; ++k) sh[k][threadIdx.x] += sh[k][threadIdx.x + w];
+    __syncthreads();
+  }
+#pragma unroll
+  for (int k = 0; k < NV; ++k) v[k] = sh[k][0];
+}
+
+// One workgroup of 256 threads.  Row totals from the segment partials (ascending segment), the weight each
+// row's token sums carry under the aggregation mode, the loss and the metrics.
+// row_tot [rows][3] double (loss, entropy, mask), row_weight [rows] float.
+// out: [0] loss, [1] pg_loss, [2] entropy_loss, [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower,
+//      [6] sum(mask), [7] dp_size / denominator of the mode (1 / tokens or 1 / sequences included)
+__global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs, int64_t row_len, PpoAgg g,
+                                  double* row_tot, float* row_weight, float* out) {
+  __shared__ double sh[5][256];
+  double a[5] = {0.0, 0.0, 0.0, 0.0, 0.0};  // clipped, -log ratio, dual-clipped, sum(mask), rows with tokens
+  for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
+    double t[6] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    for (int sgm = 0; sgm < segs; ++sgm)
+#pragma unroll
+      for (int k = 0; k < 6; ++k) t[k] += (double)partials[(r * segs + sgm) * 8 + k];
+    row_tot[r * 3 + 0] = t[0];
+    row_tot[r * 3 + 1] = t[1];
+    row_tot[r * 3 + 2] = t[5];
+    a[0] += t[2];
+    a[1] += t[3];
+    a[2] += t[4];
+    a[3] += t[5];
+    a[4] += t[5] > 0.0 ? 1.0 : 0.0;
+  }
+  ppo_block_sum(a, sh);
+  const double n_tok = a[3];
+  const double tok_den = g.batch_num_tokens > 0.f ? (double)g.batch_num_tokens : n_tok;
+  const double seq_den = g.global_batch_size > 0.f ? (double)g.global_batch_size : a[4];
+  const double norm = g.loss_scale_factor > 0.f ? (double)g.loss_scale_factor : (double)row_len;
+  double base;
+  switch (g.mode) {
+    case PPO_TOKEN_MEAN: base = (double)g.dp_size / tok_den; break;
+    case PPO_TOKEN_SUM: base = (double)g.dp_size; break;
+    case PPO_SEQ_MEAN_TOKEN_SUM_NORM: base = (double)g.dp_size / seq_den / norm; break;
+    default: base = (double)g.dp_size / seq_den; break;
+  }
+  const bool per_seq = g.mode >= PPO_SEQ_MEAN_TOKEN_SUM;
+  double b[2] = {0.0, 0.0};
+  for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
+    const double cnt = row_tot[r * 3 + 2];
+    double w = base;
+    if (per_seq && !(cnt > 0.0)) w = 0.0;  // rows without tokens are excluded from a sequence mean
+    if (g.mode == PPO_SEQ_MEAN_TOKEN_MEAN) w /= cnt + 1e-8;
+    row_weight[r] = (float)w;
+    b[0] += w * row_tot[r * 3 + 0];
+    b[1] += w * row_tot[r * 3 + 1];
+  }
+  ppo_block_sum(b, sh);
   if (threadIdx.x == 0) {
-    const double n = tot[5];
-    const double scale = token_scale > 0.f ? (double)token_scale : 1.0 / n;  // token-mean: dp_size / batch_num_tokens
-    const double pg = tot[0] * scale, el = tot[1] * scale;
-    out[0] = (float)(pg - (double)entropy_coeff * el);
-    out[1] = (float)pg;
-    out[2] = (float)el;
-    out[3] = (float)(tot[2] / (n + 1e-8));
-    out[4] = (float)(tot[3] / (n + 1e-8));
-    out[5] = (float)(tot[4] / (n + 1e-8));
-    out[6] = (float)n;
-    out[7] = (float)scale;
+    out[0] = (float)(b[0] - (double)g.entropy_coeff * b[1]);
+    out[1] = (float)b[0];
+    out[2] = (float)b[1];
+    out[3] = (float)(a[0] / (n_tok + 1e-8));
+    out[4] = (float)(a[1] / (n_tok + 1e-8));
+    out[5] = (float)(a[2] / (n_tok + 1e-8));
+    out[6] = (float)n_tok;
+    out[7] = (float)base;
   }
 }
 
-__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t N, const float* out) {
-  const float scale = out[7];
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < N; t += (int64_t)gridDim.x * blockDim.x) {
+__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t rows, int64_t row_len, int segs, int64_t seg_len,
+                                 const float* row_weight) {
+  const int64_t row = (int64_t)blockIdx.x / segs;
+  const int64_t c0 = ((int64_t)blockIdx.x % segs) * seg_len;
+  const int64_t c1 = c0 + seg_len < row_len ? c0 + seg_len : row_len;
+  const float scale = row_weight[row];
+  for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
+    const int64_t t = row * row_len + c;
     g_lp[t] *= scale;
     if (g_ent) g_ent[t] *= scale;
   }

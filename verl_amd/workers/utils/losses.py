@@ -2,8 +2,8 @@
 
 One HIP pass computes what the reference assembles from ``compute_policy_loss_vanilla`` + ``agg_loss`` and
 the entropy bonus in ``ppo_loss`` (``verl/trainer/ppo/core_algos.py:1140-1206,1286-1376``,
-``verl/workers/utils/losses.py:57-140``) for the vanilla loss with ``token-mean`` aggregation, together with the
-gradients w.r.t. ``log_prob`` and ``entropy``, so the backward of ``linear_cross_entropy`` starts from two
+``verl/workers/utils/losses.py:57-140``) for the vanilla loss under any of ``agg_loss``'s aggregation modes, together
+with the gradients w.r.t. ``log_prob`` and ``entropy``, so the backward of ``linear_cross_entropy`` starts from two
 ready vectors instead of an elementwise autograd graph.  Metric names are the reference's.
 """
 
@@ -16,10 +16,19 @@ import torch
 from ... import _abi
 
 
+AGG_MODES = {
+    "token-mean": 0,
+    "token-sum": 1,
+    "seq-mean-token-sum": 2,
+    "seq-mean-token-sum-norm": 3,
+    "seq-mean-token-mean": 4,
+}
+
+
 class _FusedPPOLoss(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, clip_low, clip_high, clip_c,
-                entropy_coeff, token_scale):
+    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, agg, clip_low, clip_high,
+                clip_c, entropy_coeff):
         assert log_prob.is_cuda, "fused_ppo_loss runs on the GPU only"
         dev = log_prob.device
         shape = log_prob.shape
@@ -29,18 +38,25 @@ class _FusedPPOLoss(torch.autograd.Function):
 
         lp, old, adv, mask = f32(log_prob), f32(old_log_prob), f32(advantages), f32(response_mask)
         ent = None if entropy is None else f32(entropy)
+        isw = None if is_weights is None else f32(is_weights)
         n = lp.numel()
         assert old.numel() == n and adv.numel() == n and mask.numel() == n and (ent is None or ent.numel() == n)
+        assert isw is None or isw.numel() == n
+        # rows are the sequences the seq-mean modes average over: the last dimension is the response
+        row_len = shape[-1] if len(shape) >= 1 else 1
+        rows = n // row_len if row_len else 0
+        mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor = agg
         out = torch.empty(8, device=dev, dtype=torch.float32)
         g_lp = torch.empty(n, device=dev, dtype=torch.float32)
         g_ent = None if ent is None else torch.empty(n, device=dev, dtype=torch.float32)
         lib = _abi.load()
         with torch.cuda.device(dev):
-            ws_bytes = lib.lce_ppo_loss_workspace_bytes(n)
+            ws_bytes = lib.lce_ppo_loss_workspace_bytes(rows, row_len)
             ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
             rc = lib.lce_ppo_loss(
-                lp.data_ptr(), _abi.ptr(ent), old.data_ptr(), adv.data_ptr(), mask.data_ptr(), n, clip_low, clip_high,
-                clip_c, entropy_coeff, token_scale, out.data_ptr(), g_lp.data_ptr(), _abi.ptr(g_ent), ws.data_ptr(),
+                lp.data_ptr(), _abi.ptr(ent), old.data_ptr(), adv.data_ptr(), mask.data_ptr(), _abi.ptr(isw), rows,
+                row_len, mode, clip_low, clip_high, clip_c, entropy_coeff, dp_size, batch_num_tokens,
+                global_batch_size, loss_scale_factor, out.data_ptr(), g_lp.data_ptr(), _abi.ptr(g_ent), ws.data_ptr(),
                 ws_bytes, _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_ppo_loss")
@@ -56,7 +72,7 @@ class _FusedPPOLoss(torch.autograd.Function):
         g_lp, g_ent = ctx.saved_tensors
         d_lp = (g_lp * g_loss).reshape(ctx.shape).to(ctx.dtypes[0])
         d_ent = (g_ent * g_loss).reshape(ctx.shape).to(ctx.dtypes[1]) if ctx.has_entropy else None
-        return d_lp, d_ent, None, None, None, None, None, None, None, None
+        return d_lp, d_ent, None, None, None, None, None, None, None, None, None
 
 
 def fused_ppo_loss(
@@ -73,23 +89,35 @@ def fused_ppo_loss(
     loss_agg_mode: str = "token-mean",
     dp_size: int = 1,
     batch_num_tokens: Optional[int] = None,
+    global_batch_size: Optional[int] = None,
+    loss_scale_factor: Optional[int] = None,
+    rollout_is_weights: Optional[torch.Tensor] = None,
 ):
     """Returns ``(policy_loss, metrics)``: ``policy_loss = pg_loss - entropy_coeff * entropy_loss`` (a 0-dim tensor
-    with autograd), ``metrics`` a dict of 0-dim tensors under the reference's keys (no host sync is forced)."""
-    if loss_agg_mode != "token-mean":
-        raise NotImplementedError(f"fused_ppo_loss implements token-mean aggregation, got {loss_agg_mode}")
+    with autograd), ``metrics`` a dict of 0-dim tensors under the reference's keys (no host sync is forced).
+    ``dp_size``, ``batch_num_tokens``, ``global_batch_size`` and ``loss_scale_factor`` are ``agg_loss``'s
+    (``core_algos.py:1140-1206``); the sequences of the ``seq-mean-*`` modes are the rows of the last dimension.
+    ``rollout_is_weights`` multiplies the per-token policy loss (``core_algos.py:1362-1363``) and takes no gradient."""
+    if loss_agg_mode not in AGG_MODES:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
     assert clip_ratio_c > 1.0, f"clip_ratio_c must be greater than 1.0, got {clip_ratio_c}"
     lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
     hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
-    if batch_num_tokens is None:
-        if dp_size > 1:
+    if dp_size > 1:
+        if loss_agg_mode == "token-mean" and batch_num_tokens is None:
             raise ValueError("(global) batch_num_tokens is required when dp_size > 1")
-        token_scale = -1.0
-    else:
-        token_scale = float(dp_size) / float(batch_num_tokens)
+        if loss_agg_mode.startswith("seq-mean") and global_batch_size is None:
+            raise ValueError("global_batch_size is required when dp_size > 1")
+    agg = (
+        AGG_MODES[loss_agg_mode],
+        float(dp_size),
+        -1.0 if batch_num_tokens is None else float(batch_num_tokens),
+        -1.0 if global_batch_size is None else float(global_batch_size),
+        -1.0 if loss_scale_factor is None else float(loss_scale_factor),
+    )
     loss, out = _FusedPPOLoss.apply(
-        log_prob, entropy, old_log_prob, advantages, response_mask, float(lo), float(hi), float(clip_ratio_c),
-        float(entropy_coeff), token_scale,
+        log_prob, entropy, old_log_prob, advantages, response_mask, rollout_is_weights, agg, float(lo), float(hi),
+        float(clip_ratio_c), float(entropy_coeff),
     )  # fmt: skip
     metrics = {
         "actor/pg_loss": out[1],
