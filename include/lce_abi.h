@@ -112,26 +112,35 @@ int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, 
 int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream);
 
 /* Consumer of the path's outputs: the clipped PPO policy loss with dual clip, any of agg_loss's aggregation
- * modes and the entropy bonus.  Replaces, for the vanilla loss, compute_policy_loss_vanilla + agg_loss
- * (verl/trainer/ppo/core_algos.py:1140-1206, :1286-1376) and the entropy term of ppo_loss
- * (verl/workers/utils/losses.py:134-140), and yields the upstream gradients lce_backward consumes, so no
- * elementwise autograd graph sits between the two kernels.
+ * modes, the entropy bonus and the KL penalty against a reference policy.  Replaces, for the vanilla loss,
+ * compute_policy_loss_vanilla + agg_loss (verl/trainer/ppo/core_algos.py:1140-1206, :1286-1376), kl_penalty
+ * (:2188-2251) and the entropy and KL terms of ppo_loss (verl/workers/utils/losses.py:134-153), and yields the
+ * upstream gradients lce_backward consumes, so no elementwise autograd graph sits between the two kernels.
  *   all inputs fp32 [rows, row_len] contiguous (batch x response; rows = 1 for a flat token list, which the
  *   token modes treat alike); entropy / g_entropy may both be NULL; is_weights (rollout correction factor on
  *   the policy loss, core_algos.py:1362-1363, a constant w.r.t. the gradients) may be NULL
+ *   kl_type LCE_PPO_KL_* (K1 "kl", ABS "abs", K2 "mse", K3 "low_var_kl"), optionally | LCE_PPO_KL_STRAIGHT_THROUGH
+ *   (the reference's "+" suffix: the estimator's value with k2's gradient); needs ref_log_prob; adds
+ *   kl_coef * agg(kl) to the loss
+ *   log_prob == NULL (then old_log_prob, advantages are ignored, g_log_prob is NULL, no KL): the call is agg_loss
+ *   applied to `entropy`; with entropy_coeff = -1, out[0] = agg(entropy) and g_entropy is its gradient
  *   agg_mode LCE_PPO_*: per row r with n_r = sum(mask_r), a token of row r weighs
  *     TOKEN_MEAN dp_size / batch_num_tokens; TOKEN_SUM dp_size; SEQ_MEAN_TOKEN_SUM dp_size / global_batch_size;
  *     SEQ_MEAN_TOKEN_SUM_NORM that / loss_scale_factor; SEQ_MEAN_TOKEN_MEAN dp_size / global_batch_size / (n_r + 1e-8);
  *     the SEQ modes skip rows with n_r = 0
  *   batch_num_tokens <= 0: sum(mask); global_batch_size <= 0: number of rows with n_r > 0;
  *   loss_scale_factor <= 0: row_len
- *   out [8]: loss, pg_loss, entropy_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower, sum(mask), the mode's common factor
+ *   out [16]: loss, pg_loss, entropy_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower, sum(mask), the mode's common
+ *   factor, kl_loss; the rest is reserved
  *   g_log_prob, g_entropy [rows, row_len]: d loss / d log_prob, d loss / d entropy (zero outside the mask) */
 enum { LCE_PPO_TOKEN_MEAN = 0, LCE_PPO_TOKEN_SUM = 1, LCE_PPO_SEQ_MEAN_TOKEN_SUM = 2,
        LCE_PPO_SEQ_MEAN_TOKEN_SUM_NORM = 3, LCE_PPO_SEQ_MEAN_TOKEN_MEAN = 4 };
+enum { LCE_PPO_KL_NONE = 0, LCE_PPO_KL_K1 = 1, LCE_PPO_KL_ABS = 2, LCE_PPO_KL_K2 = 3, LCE_PPO_KL_K3 = 4,
+       LCE_PPO_KL_STRAIGHT_THROUGH = 16 };
 size_t lce_ppo_loss_workspace_bytes(int64_t rows, int64_t row_len);
 int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
-                 const float* mask, const float* is_weights, int64_t rows, int64_t row_len, int agg_mode,
+                 const float* mask, const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef,
+                 int64_t rows, int64_t row_len, int agg_mode,
                  float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
                  float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
                  float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream);

@@ -20,7 +20,8 @@ What each function follows in the reference tree (paths relative to the referenc
 * ``masked_sum/masked_mean`` verl/utils/torch_functional.py:273-308
 * ``agg_loss``               verl/trainer/ppo/core_algos.py:1140-1206
 * ``policy_loss_vanilla``    verl/trainer/ppo/core_algos.py:1286-1376
-* ``ppo_actor_loss``         verl/workers/utils/losses.py:57-140 (policy loss minus entropy bonus)
+* ``kl_penalty``             verl/trainer/ppo/core_algos.py:2188-2251
+* ``ppo_actor_loss``         verl/workers/utils/losses.py:57-153 (policy loss minus entropy bonus plus KL penalty)
 
 How each is pinned (see tests/test_oracle_*.py): the reference's own known-answer vector for the
 padded-vocab regression (tests/utils/test_linear_cross_entropy.py:352-395, closed form
@@ -30,7 +31,9 @@ for the gradients, the invariant ``sum_v dz = 0``, for ``sum_pi_squared_from_log
 ``1/V`` (uniform), ``(1 + (V-1) r^2) / (1 + (V-1) r)^2`` (one logit raised by ``log(1/r)``) and a pure-Python
 ``sum(softmax**2)``, the independent C restatement in
 ``lce_oracle.c``, and the reference's known answers for ``agg_loss`` / ``masked_mean``
-(tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-65, tests/utils/test_torch_functional.py:61-72).
+(tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-65, tests/utils/test_torch_functional.py:61-72);
+``kl_penalty`` by its definitions evaluated with ``math.exp`` on scalars, ``k3 >= 0``, ``k3 = d^2/2 + O(d^3)``,
+``E_pi[k1] = E_pi[k3] = KL`` on a small categorical distribution and autograd for the straight-through variants.
 No function here is "parity unpinned".
 """
 
@@ -274,6 +277,27 @@ def policy_loss_vanilla(
     return loss, metrics
 
 
+def kl_penalty(logprob, ref_logprob, kl_penalty_type: str):
+    """verl/trainer/ppo/core_algos.py:2188-2251: the k1 / abs / k2 / k3 estimators of KL(pi || pi_ref) per token; a
+    trailing "+" keeps the estimator's value and gives it the gradient of k2 (straight through), k2 itself unchanged."""
+    base = kl_penalty_type[:-1] if kl_penalty_type.endswith("+") else kl_penalty_type
+    if base in ("kl", "k1"):
+        fwd = logprob - ref_logprob
+    elif base == "abs":
+        fwd = (logprob - ref_logprob).abs()
+    elif base in ("mse", "k2"):
+        fwd = 0.5 * (logprob - ref_logprob).square()
+    elif base in ("low_var_kl", "k3"):
+        kl = torch.clamp(ref_logprob - logprob, min=-20, max=20)
+        fwd = torch.clamp(torch.exp(kl) - kl - 1, min=-10, max=10)
+    else:
+        raise NotImplementedError
+    if not kl_penalty_type.endswith("+") or kl_penalty_type in ("mse", "k2"):
+        return fwd
+    bwd = 0.5 * (logprob - ref_logprob).square()
+    return bwd - bwd.detach() + fwd.detach()
+
+
 def ppo_actor_loss(
     log_prob,
     entropy,
@@ -285,10 +309,14 @@ def ppo_actor_loss(
     loss_agg_mode: str = "token-mean",
     clip_ratio_c: float = 3.0,
     rollout_is_weights=None,
+    ref_log_prob=None,
+    kl_loss_type: str = "low_var_kl",
+    kl_loss_coef: float = 0.001,
     **global_batch_info,
 ):
-    """policy loss - entropy_coeff * agg(entropy): the scalar the actor back-propagates
-    (verl/workers/utils/losses.py:109-140; both terms aggregated with the same mode and global batch info)."""
+    """policy loss - entropy_coeff * agg(entropy) [+ kl_loss_coef * agg(kl_penalty)]: the scalar the actor
+    back-propagates (verl/workers/utils/losses.py:109-153; every term aggregated with the same mode and global
+    batch info; the KL term is the reference's use_kl_loss branch, taken here when ref_log_prob is given)."""
     pg, metrics = policy_loss_vanilla(
         old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, clip_ratio, clip_ratio_c=clip_ratio_c,
         rollout_is_weights=rollout_is_weights, **global_batch_info,
@@ -298,6 +326,12 @@ def ppo_actor_loss(
         ent = agg_loss(entropy, response_mask, loss_agg_mode, **global_batch_info)
         loss = loss - entropy_coeff * ent
         metrics["actor/entropy_loss"] = ent.detach().item()
+    if ref_log_prob is not None:
+        kld = kl_penalty(log_prob, ref_log_prob, kl_loss_type)
+        kl = agg_loss(kld, response_mask, loss_agg_mode, **global_batch_info)
+        loss = loss + kl * kl_loss_coef
+        metrics["kl_loss"] = kl.detach().item()
+        metrics["kl_coef"] = kl_loss_coef
     metrics["actor/pg_loss"] = pg.detach().item()
     return loss, metrics
 

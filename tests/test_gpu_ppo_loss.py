@@ -126,6 +126,86 @@ def test_flat_token_list_equals_rows_in_token_modes():
         torch.testing.assert_close(a, b, atol=1e-6, rtol=1e-5)
 
 
+@pytest.mark.parametrize("kl_type", ["kl", "abs", "mse", "low_var_kl", "k1+", "abs+", "k2+", "k3+", "low_var_kl+"])
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-mean"])
+def test_kl_penalty_term(kl_type, mode):
+    """ppo_loss's use_kl_loss branch (verl/workers/utils/losses.py:142-153) with every estimator of kl_penalty
+    (verl/trainer/ppo/core_algos.py:2188-2251), the oracle evaluated in fp64."""
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask = _case(16, 257, seed=21, spread=0.3)
+    g = torch.Generator().manual_seed(22)
+    ref = lp + (torch.randn(16, 257, generator=g) * 0.2).to(DEV)
+    ref[0, :4] = lp[0, :4] + torch.tensor([25.0, -25.0, 3.0, 0.0], device=DEV)  # both clamps of k3, and equality
+    lp1, ent1 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    loss, met = fused_ppo_loss(lp1, ent1, old, adv, mask, entropy_coeff=1e-2, loss_agg_mode=mode, ref_log_prob=ref,
+                               kl_loss_type=kl_type, kl_loss_coef=0.05)  # fmt: skip
+    loss.backward()
+    d = [t.double() for t in (lp, ent, old, adv, mask, ref)]
+    lp2, ent2 = d[0].clone().requires_grad_(True), d[1].clone().requires_grad_(True)
+    rloss, rmet = O.ppo_actor_loss(lp2, ent2, d[2], d[3], d[4], entropy_coeff=1e-2, loss_agg_mode=mode,
+                                   ref_log_prob=d[5], kl_loss_type=kl_type, kl_loss_coef=0.05)  # fmt: skip
+    rloss.backward()
+    torch.testing.assert_close(loss.double(), rloss, atol=1e-6, rtol=2e-5)
+    assert met["kl_coef"] == 0.05
+    assert met["kl_loss"].item() == pytest.approx(rmet["kl_loss"], rel=2e-5, abs=1e-7)
+    scale = lp2.grad.abs().max().item()
+    torch.testing.assert_close(lp1.grad.double(), lp2.grad, atol=2e-6 * scale, rtol=2e-5)
+    torch.testing.assert_close(ent1.grad.double(), ent2.grad, atol=1e-9, rtol=1e-5)
+    with pytest.raises(NotImplementedError):
+        fused_ppo_loss(lp, ent, old, adv, mask, ref_log_prob=ref, kl_loss_type="full")
+
+
+@pytest.mark.parametrize("mode,info", AGG_CASES)
+def test_agg_loss_and_policy_loss_under_the_reference_names(mode, info):
+    """verl_amd.trainer.ppo.core_algos.agg_loss / compute_policy_loss_vanilla: the reference's signatures
+    (verl/trainer/ppo/core_algos.py:1140-1206, :1286-1376), values and gradients against the oracle."""
+    from types import SimpleNamespace
+
+    from verl_amd.trainer.ppo.core_algos import agg_loss, compute_policy_loss_vanilla
+
+    lp, ent, old, adv, mask = _case(9, 700, seed=31, spread=0.6)
+    mask[4] = 0
+    x1 = ent.clone().requires_grad_(True)
+    got = agg_loss(x1, mask, mode, **info)
+    (got * 3.0).backward()
+    x2 = ent.clone().requires_grad_(True)
+    want = O.agg_loss(x2, mask, mode, **info)
+    (want * 3.0).backward()
+    torch.testing.assert_close(got, want, atol=1e-6, rtol=2e-5)
+    torch.testing.assert_close(x1.grad, x2.grad, atol=1e-6 * x2.grad.abs().max().item(), rtol=1e-5)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.1, clip_ratio_high=0.3, global_batch_info=info,
+                          get=lambda k, dflt=None: {"clip_ratio_c": 2.5}.get(k, dflt))  # fmt: skip
+    lp1 = lp.clone().requires_grad_(True)
+    pg, pm = compute_policy_loss_vanilla(old, lp1, adv, mask, mode, cfg)
+    pg.backward()
+    lp2 = lp.clone().requires_grad_(True)
+    rpg, rpm = O.policy_loss_vanilla(old, lp2, adv, mask, mode, 0.2, 0.1, 0.3, 2.5, **info)
+    rpg.backward()
+    torch.testing.assert_close(pg, rpg, atol=1e-6, rtol=2e-5)
+    assert set(pm) == set(rpm) and all(isinstance(v, float) for v in pm.values())
+    for k in pm:
+        assert pm[k] == pytest.approx(rpm[k], rel=2e-5, abs=1e-6), k
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-6 * lp2.grad.abs().max().item(), rtol=1e-5)
+
+
+def test_agg_loss_errors_like_the_reference():
+    from verl_amd.trainer.ppo.core_algos import agg_loss
+
+    lp, ent, old, adv, mask = _case(2, 8, seed=1)
+    with pytest.raises(ValueError, match="Invalid loss_agg_mode"):
+        agg_loss(ent, mask, "nope")
+    with pytest.raises(ValueError, match="batch_num_tokens is required"):
+        agg_loss(ent, mask, "token-mean", dp_size=2)
+    with pytest.raises(ValueError, match="global_batch_size is required"):
+        agg_loss(ent, mask, "seq-mean-token-mean", dp_size=2)
+    # the reference's own known answers (tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-30)
+    loss_mat = torch.tensor([[1.0, 2.0, 30.0], [4.0, 50.0, 6.0]], device=DEV)
+    loss_mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 0.0, 1.0]], device=DEV)
+    assert agg_loss(loss_mat, loss_mask, "token-sum", dp_size=4).item() == pytest.approx((1 + 2 + 4 + 6) * 4)
+    assert agg_loss(loss_mat, loss_mask, "seq-mean-token-mean").item() == pytest.approx((1.5 + 5) / 2)
+
+
 def test_actor_step_fused_end_to_end():
     """fused head -> fused loss -> fused backward, against the all-oracle pipeline (config-5 family, reduced)."""
     from verl_amd import linear_cross_entropy

@@ -84,3 +84,57 @@ def test_ppo_actor_loss_entropy_bonus():
     loss.backward()
     torch.testing.assert_close(ent.grad, torch.tensor([[-5e-4, -5e-4, 0.0]]))
     assert met["actor/entropy_loss"] == pytest.approx(3.0)
+
+
+def test_kl_penalty_estimators_against_scalar_arithmetic():
+    """verl/trainer/ppo/core_algos.py:2188-2251, pinned by the definitions evaluated with math.exp on scalars, the
+    textbook facts about the estimators (k3 >= 0 with equality at equal log-probs, k3 ~ k2 for small differences,
+    E_pi[k1] = E_pi[k3] = KL on a small categorical distribution) and autograd for the straight-through variants."""
+    import math
+
+    lp = torch.tensor([-1.0, -0.5, -2.0, -0.7, -30.0, 5.0], dtype=torch.float64)
+    ref = torch.tensor([-1.5, -0.5, -1.0, -0.71, 0.0, -30.0], dtype=torch.float64)
+    for i in range(6):
+        d = lp[i].item() - ref[i].item()
+        q = min(max(-d, -20.0), 20.0)
+        want = {"kl": d, "abs": abs(d), "mse": 0.5 * d * d, "low_var_kl": min(max(math.exp(q) - q - 1, -10.0), 10.0)}
+        for name, alias in (("kl", "k1"), ("abs", "abs"), ("mse", "k2"), ("low_var_kl", "k3")):
+            assert O.kl_penalty(lp, ref, name)[i].item() == pytest.approx(want[name], rel=1e-12, abs=1e-15)
+            assert O.kl_penalty(lp, ref, alias)[i].item() == pytest.approx(want[name], rel=1e-12, abs=1e-15)
+    k3 = O.kl_penalty(lp, ref, "k3")
+    assert (k3 >= 0).all() and k3[1].item() == 0.0
+    assert k3[3].item() == pytest.approx(0.5 * 0.01**2, rel=1e-2)  # k3 = d^2/2 + O(d^3)
+    assert k3[4].item() == 10.0  # exp(20) - 20 - 1 clamped to 10
+    assert k3[5].item() == 10.0  # exp(-20) + 20 - 1 = 19.0 clamped to 10
+    # expectations over a categorical pi: sum_x pi(x) k1(x) = KL(pi || ref) = sum_x pi(x) k3(x)
+    pi = torch.tensor([0.5, 0.3, 0.2], dtype=torch.float64)
+    rf = torch.tensor([0.2, 0.5, 0.3], dtype=torch.float64)
+    kl_true = (pi * (pi / rf).log()).sum().item()
+    assert (pi * O.kl_penalty(pi.log(), rf.log(), "k1")).sum().item() == pytest.approx(kl_true, rel=1e-12)
+    assert (pi * O.kl_penalty(pi.log(), rf.log(), "k3")).sum().item() == pytest.approx(kl_true, rel=1e-12)
+    # straight-through: the value of the estimator, the gradient of k2 (= log_prob - ref_log_prob)
+    for name in ("kl+", "abs+", "low_var_kl+", "k3+", "k2+", "mse+"):
+        x = lp.clone().requires_grad_(True)
+        v = O.kl_penalty(x, ref, name)
+        torch.testing.assert_close(v.detach(), O.kl_penalty(lp, ref, name[:-1]))
+        v.sum().backward()
+        torch.testing.assert_close(x.grad, lp - ref)
+    with pytest.raises(NotImplementedError):
+        O.kl_penalty(lp, ref, "full")
+
+
+def test_actor_loss_with_kl_term_is_the_sum_of_its_parts():
+    g = torch.Generator().manual_seed(5)
+    lp = -torch.rand(3, 7, generator=g)
+    old = lp + 0.1 * torch.randn(3, 7, generator=g)
+    ref = lp + 0.2 * torch.randn(3, 7, generator=g)
+    adv = torch.randn(3, 7, generator=g)
+    ent = torch.rand(3, 7, generator=g)
+    mask = (torch.rand(3, 7, generator=g) < 0.7).float()
+    for mode in ("token-mean", "seq-mean-token-mean"):
+        loss, met = O.ppo_actor_loss(lp, ent, old, adv, mask, entropy_coeff=0.1, loss_agg_mode=mode, ref_log_prob=ref,
+                                     kl_loss_type="low_var_kl", kl_loss_coef=0.3)  # fmt: skip
+        pg, _ = O.policy_loss_vanilla(old, lp, adv, mask, mode)
+        want = pg - 0.1 * O.agg_loss(ent, mask, mode) + 0.3 * O.agg_loss(O.kl_penalty(lp, ref, "k3"), mask, mode)
+        torch.testing.assert_close(loss, want)
+        assert met["kl_coef"] == 0.3 and met["kl_loss"] == pytest.approx(O.agg_loss(O.kl_penalty(lp, ref, "k3"), mask, mode).item())

@@ -843,20 +843,30 @@ size_t lce_ppo_loss_workspace_bytes(int64_t rows, int64_t row_len) {
   int segs;
   int64_t seg_len;
   ppo_geometry(rows, row_len, &segs, &seg_len);
-  return ppo_align((size_t)rows * segs * 8 * sizeof(float)) + ppo_align((size_t)rows * 3 * sizeof(double)) +
+  return ppo_align((size_t)rows * segs * 8 * sizeof(float)) + ppo_align((size_t)rows * 4 * sizeof(double)) +
          ppo_align((size_t)rows * sizeof(float));
 }
 
 int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
-                 const float* mask, const float* is_weights, int64_t rows, int64_t row_len, int agg_mode,
+                 const float* mask, const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef,
+                 int64_t rows, int64_t row_len, int agg_mode,
                  float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
                  float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
                  float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream) {
   if (rows <= 0 || row_len <= 0) return fail(LCE_E_ARG, "ppo loss: rows and row_len must be positive");
   if (rows > ((int64_t)1 << 30) || row_len > ((int64_t)1 << 40) / rows) return fail(LCE_E_ARG, "ppo loss: too many elements");
-  if (!log_prob || !old_log_prob || !advantages || !mask || !out || !g_log_prob) return fail(LCE_E_ARG, "null pointer");
+  if (!mask || !out) return fail(LCE_E_ARG, "null pointer");
+  if (log_prob) {
+    if (!old_log_prob || !advantages || !g_log_prob) return fail(LCE_E_ARG, "null pointer");
+    if (!(clip_c > 1.f)) return fail(LCE_E_ARG, "clip_ratio_c must be greater than 1");
+  } else if (!entropy || g_log_prob || kl_type != LCE_PPO_KL_NONE) {
+    return fail(LCE_E_ARG, "without log_prob the call aggregates `entropy` alone");
+  }
   if ((entropy == nullptr) != (g_entropy == nullptr)) return fail(LCE_E_ARG, "entropy and g_entropy go together");
-  if (!(clip_c > 1.f)) return fail(LCE_E_ARG, "clip_ratio_c must be greater than 1");
+  const int kl_base = kl_type & ~LCE_PPO_KL_STRAIGHT_THROUGH;
+  if (kl_base < LCE_PPO_KL_NONE || kl_base > LCE_PPO_KL_K3 || (kl_base == LCE_PPO_KL_NONE && kl_type != LCE_PPO_KL_NONE))
+    return fail(LCE_E_ARG, "ppo loss: unknown kl_type %d", kl_type);
+  if (kl_base != LCE_PPO_KL_NONE && !ref_log_prob) return fail(LCE_E_ARG, "the KL penalty needs ref_log_prob");
   if (agg_mode < PPO_TOKEN_MEAN || agg_mode > PPO_SEQ_MEAN_TOKEN_MEAN) return fail(LCE_E_ARG, "Invalid loss_agg_mode: %d", agg_mode);
   if (!(dp_size > 0.f)) return fail(LCE_E_ARG, "ppo loss: dp_size must be positive");
   if (!workspace || workspace_bytes < lce_ppo_loss_workspace_bytes(rows, row_len))
@@ -870,15 +880,19 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
   p.partials = reinterpret_cast<float*>(ws);
   ws += ppo_align((size_t)blocks * 8 * sizeof(float));
   double* row_tot = reinterpret_cast<double*>(ws);
-  ws += ppo_align((size_t)rows * 3 * sizeof(double));
+  ws += ppo_align((size_t)rows * 4 * sizeof(double));
   float* row_weight = reinterpret_cast<float*>(ws);
   p.log_prob = log_prob; p.entropy = entropy; p.old_log_prob = old_log_prob; p.advantages = advantages; p.mask = mask;
   p.is_weights = is_weights; p.rows = rows; p.row_len = row_len;
+  p.ref_log_prob = ref_log_prob; p.kl_type = kl_base; p.kl_coef = kl_coef;
+  // (k2's own gradient is already the straight-through one, verl/trainer/ppo/core_algos.py:2203-2204)
+  p.kl_straight_through = (kl_type & LCE_PPO_KL_STRAIGHT_THROUGH) != 0 && kl_base != LCE_PPO_KL_K2;
   p.clip_low = clip_low; p.clip_high = clip_high; p.clip_c = clip_c; p.entropy_coeff = entropy_coeff;
   p.g_log_prob = g_log_prob; p.g_entropy = g_entropy;
   PpoAgg g;
   g.mode = agg_mode; g.dp_size = dp_size; g.batch_num_tokens = batch_num_tokens; g.global_batch_size = global_batch_size;
   g.loss_scale_factor = loss_scale_factor; g.entropy_coeff = entropy_coeff;
+  g.kl_coef = kl_base != LCE_PPO_KL_NONE ? kl_coef : 0.f;
   hipLaunchKernelGGL(ppo_terms_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
   int rc = check_launch("ppo_terms_kernel");
   if (rc) return rc;

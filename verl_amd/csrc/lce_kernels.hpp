@@ -1164,18 +1164,24 @@ __global__ __launch_bounds__(NT) void logits_bwd_kernel(const TIN* logits, int64
 }
 
 // ------------------------------------------------------------------------------------------------
-// consumer of the path's outputs: clipped PPO policy loss + entropy bonus, every aggregation mode of agg_loss
+// consumer of the path's outputs: clipped PPO policy loss + entropy bonus + KL penalty against a reference
+// policy, every aggregation mode of agg_loss
 // ------------------------------------------------------------------------------------------------
+enum { PPO_KL_NONE = 0, PPO_KL_K1 = 1, PPO_KL_ABS = 2, PPO_KL_K2 = 3, PPO_KL_K3 = 4 };
 enum { PPO_TOKEN_MEAN = 0, PPO_TOKEN_SUM = 1, PPO_SEQ_MEAN_TOKEN_SUM = 2, PPO_SEQ_MEAN_TOKEN_SUM_NORM = 3,
        PPO_SEQ_MEAN_TOKEN_MEAN = 4 };
 
 struct PpoArgs {
-  const float* log_prob;
-  const float* entropy;  // may be null
+  const float* log_prob;  // null: no policy term (plain aggregation of `entropy`)
+  const float* entropy;   // may be null
   const float* old_log_prob;
   const float* advantages;
   const float* mask;
   const float* is_weights;  // may be null: per-token factor on the policy loss (rollout correction), a constant
+  const float* ref_log_prob;  // with kl_type != PPO_KL_NONE
+  int kl_type;
+  int kl_straight_through;  // the estimator's value with the gradient of 0.5 * (log_prob - ref_log_prob)^2
+  float kl_coef;
   int64_t rows, row_len;    // [rows][row_len], row-major, contiguous
   int segs;                 // workgroups per row
   int64_t seg_len;          // elements per workgroup (the last one of a row may be short)
@@ -1186,7 +1192,7 @@ struct PpoArgs {
 };
 
 // Per-token terms and unscaled gradients; workgroup (row, seg) reduces its segment of one row to
-// partials[row * segs + seg][0..5] = sums of (loss, entropy, clipped, -log ratio, dual-clipped, 1) x mask.
+// partials[row * segs + seg][0..6] = sums of (loss, entropy, clipped, -log ratio, dual-clipped, 1, kl) x mask.
 __global__ void ppo_terms_kernel(PpoArgs p) {
   __shared__ float sh[8][256];
   float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -1196,22 +1202,51 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
   for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
     const int64_t t = row * p.row_len + c;
     const float m = p.mask[t];
-    const float lp = p.log_prob[t], A = p.advantages[t];
-    const float d = lp - p.old_log_prob[t];
-    const float nkl = fminf(fmaxf(d, -20.f), 20.f);
-    const float r = __expf(nkl);
-    const float dr = (d > -20.f && d < 20.f) ? r : 0.f;          // d ratio / d log_prob
-    const float rc = fminf(fmaxf(r, 1.f - p.clip_low), 1.f + p.clip_high);
-    const float drc = (r > 1.f - p.clip_low && r < 1.f + p.clip_high) ? dr : 0.f;
-    const float l1 = -A * r, l2 = -A * rc, l3 = -A * p.clip_c;
-    const float lc1 = fmaxf(l1, l2);
-    const float dlc1 = l1 > l2 ? -A * dr : (l2 > l1 ? -A * drc : -A * 0.5f * (dr + drc));
-    const bool dual = A < 0.f;
-    const float isw = p.is_weights ? p.is_weights[t] : 1.f;
-    const float loss = (dual ? fminf(l3, lc1) : lc1) * isw;
-    const float dloss = ((dual && l3 < lc1) ? 0.f : dlc1) * isw;
     const bool on = m != 0.f;  // values outside the mask never reach a sum (NaNs there are harmless)
-    p.g_log_prob[t] = on ? dloss * m : 0.f;
+    float loss = 0.f, dloss = 0.f, nkl = 0.f, clipped = 0.f, dual_clipped = 0.f;
+    if (p.log_prob) {
+      const float lp = p.log_prob[t], A = p.advantages[t];
+      const float d = lp - p.old_log_prob[t];
+      nkl = fminf(fmaxf(d, -20.f), 20.f);
+      const float r = __expf(nkl);
+      const float dr = (d > -20.f && d < 20.f) ? r : 0.f;          // d ratio / d log_prob
+      const float rc = fminf(fmaxf(r, 1.f - p.clip_low), 1.f + p.clip_high);
+      const float drc = (r > 1.f - p.clip_low && r < 1.f + p.clip_high) ? dr : 0.f;
+      const float l1 = -A * r, l2 = -A * rc, l3 = -A * p.clip_c;
+      const float lc1 = fmaxf(l1, l2);
+      const float dlc1 = l1 > l2 ? -A * dr : (l2 > l1 ? -A * drc : -A * 0.5f * (dr + drc));
+      const bool dual = A < 0.f;
+      const float isw = p.is_weights ? p.is_weights[t] : 1.f;
+      loss = (dual ? fminf(l3, lc1) : lc1) * isw;
+      dloss = ((dual && l3 < lc1) ? 0.f : dlc1) * isw;
+      clipped = l2 > l1 ? 1.f : 0.f;
+      dual_clipped = (lc1 > l3 && dual) ? 1.f : 0.f;
+      float kl = 0.f;
+      if (p.kl_type != PPO_KL_NONE) {
+        const float e = lp - p.ref_log_prob[t];
+        float dkl;
+        if (p.kl_type == PPO_KL_K1) {
+          kl = e;
+          dkl = 1.f;
+        } else if (p.kl_type == PPO_KL_ABS) {
+          kl = fabsf(e);
+          dkl = e > 0.f ? 1.f : (e < 0.f ? -1.f : 0.f);
+        } else if (p.kl_type == PPO_KL_K2) {
+          kl = 0.5f * e * e;
+          dkl = e;
+        } else {  // k3 = exp(q) - q - 1, q = clamp(ref - log_prob, +-20), clamped to +-10
+          const float q = fminf(fmaxf(-e, -20.f), 20.f);
+          const float em1 = expm1f(q);  // (exp(q) - 1 - q without cancellation near q = 0, where it is q^2 / 2)
+          const float k = em1 - q;
+          kl = fminf(fmaxf(k, -10.f), 10.f);
+          dkl = (-e >= -20.f && -e <= 20.f && k >= -10.f && k <= 10.f) ? -em1 : 0.f;
+        }
+        if (p.kl_straight_through) dkl = e;
+        dloss += p.kl_coef * dkl;
+      }
+      p.g_log_prob[t] = on ? dloss * m : 0.f;
+      if (on) s[6] += kl * m;
+    }
     float ent = 0.f;
     if (p.entropy) {
       ent = p.entropy[t];
@@ -1220,9 +1255,9 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
     if (on) {
       s[0] += loss * m;
       s[1] += ent * m;
-      s[2] += (l2 > l1 ? 1.f : 0.f) * m;
+      s[2] += clipped * m;
       s[3] += -nkl * m;
-      s[4] += ((lc1 > l3 && dual) ? 1.f : 0.f) * m;
+      s[4] += dual_clipped * m;
     }
     s[5] += m;
   }
@@ -1244,7 +1279,7 @@ struct PpoAgg {
   float batch_num_tokens;   // token-mean denominator, <= 0: sum(mask)
   float global_batch_size;  // seq-mean denominator, <= 0: number of rows with sum(mask) > 0
   float loss_scale_factor;  // seq-mean-token-sum-norm divisor, <= 0: row_len
-  float entropy_coeff;
+  float entropy_coeff, kl_coef;
 };
 
 // fixed-order sum of NV doubles per thread over the workgroup (256 threads); result valid in every thread
@@ -1266,21 +1301,23 @@ __device__ inline void ppo_block_sum(double (&v)[NV], double (*sh)[256]) {
 
 // One workgroup of 256 threads.  Row totals from the segment partials (ascending segment), the weight each
 // row's token sums carry under the aggregation mode, the loss and the metrics.
-// row_tot [rows][3] double (loss, entropy, mask), row_weight [rows] float.
-// out: [0] loss, [1] pg_loss, [2] entropy_loss, [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower,
-//      [6] sum(mask), [7] dp_size / denominator of the mode (1 / tokens or 1 / sequences included)
+// row_tot [rows][4] double (loss, entropy, mask, kl), row_weight [rows] float.
+// out: [0] loss = pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss, [1] pg_loss, [2] entropy_loss,
+//      [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower, [6] sum(mask),
+//      [7] dp_size / denominator of the mode (1 / tokens or 1 / sequences included), [8] kl_loss
 __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs, int64_t row_len, PpoAgg g,
                                   double* row_tot, float* row_weight, float* out) {
   __shared__ double sh[5][256];
   double a[5] = {0.0, 0.0, 0.0, 0.0, 0.0};  // clipped, -log ratio, dual-clipped, sum(mask), rows with tokens
   for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
-    double t[6] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    double t[7] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
     for (int sgm = 0; sgm < segs; ++sgm)
 #pragma unroll
-      for (int k = 0; k < 6; ++k) t[k] += (double)partials[(r * segs + sgm) * 8 + k];
-    row_tot[r * 3 + 0] = t[0];
-    row_tot[r * 3 + 1] = t[1];
-    row_tot[r * 3 + 2] = t[5];
+      for (int k = 0; k < 7; ++k) t[k] += (double)partials[(r * segs + sgm) * 8 + k];
+    row_tot[r * 4 + 0] = t[0];
+    row_tot[r * 4 + 1] = t[1];
+    row_tot[r * 4 + 2] = t[5];
+    row_tot[r * 4 + 3] = t[6];
     a[0] += t[2];
     a[1] += t[3];
     a[2] += t[4];
@@ -1300,19 +1337,20 @@ __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs,
     default: base = (double)g.dp_size / seq_den; break;
   }
   const bool per_seq = g.mode >= PPO_SEQ_MEAN_TOKEN_SUM;
-  double b[2] = {0.0, 0.0};
+  double b[3] = {0.0, 0.0, 0.0};
   for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
-    const double cnt = row_tot[r * 3 + 2];
+    const double cnt = row_tot[r * 4 + 2];
     double w = base;
     if (per_seq && !(cnt > 0.0)) w = 0.0;  // rows without tokens are excluded from a sequence mean
     if (g.mode == PPO_SEQ_MEAN_TOKEN_MEAN) w /= cnt + 1e-8;
     row_weight[r] = (float)w;
-    b[0] += w * row_tot[r * 3 + 0];
-    b[1] += w * row_tot[r * 3 + 1];
+    b[0] += w * row_tot[r * 4 + 0];
+    b[1] += w * row_tot[r * 4 + 1];
+    b[2] += w * row_tot[r * 4 + 3];
   }
   ppo_block_sum(b, sh);
   if (threadIdx.x == 0) {
-    out[0] = (float)(b[0] - (double)g.entropy_coeff * b[1]);
+    out[0] = (float)(b[0] - (double)g.entropy_coeff * b[1] + (double)g.kl_coef * b[2]);
     out[1] = (float)b[0];
     out[2] = (float)b[1];
     out[3] = (float)(a[0] / (n_tok + 1e-8));
@@ -1320,6 +1358,7 @@ __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs,
     out[5] = (float)(a[2] / (n_tok + 1e-8));
     out[6] = (float)n_tok;
     out[7] = (float)base;
+    out[8] = (float)b[2];
   }
 }
 
@@ -1331,7 +1370,7 @@ __global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t rows, int64_
   const float scale = row_weight[row];
   for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
     const int64_t t = row * row_len + c;
-    g_lp[t] *= scale;
+    if (g_lp) g_lp[t] *= scale;
     if (g_ent) g_ent[t] *= scale;
   }
 }

@@ -1,8 +1,8 @@
 """Fused PPO actor loss on the fused head's outputs.
 
-One HIP pass computes what the reference assembles from ``compute_policy_loss_vanilla`` + ``agg_loss`` and
-the entropy bonus in ``ppo_loss`` (``verl/trainer/ppo/core_algos.py:1140-1206,1286-1376``,
-``verl/workers/utils/losses.py:57-140``) for the vanilla loss under any of ``agg_loss``'s aggregation modes, together
+One HIP pass computes what the reference assembles from ``compute_policy_loss_vanilla`` + ``agg_loss``, ``kl_penalty``
+and the entropy and KL terms of ``ppo_loss`` (``verl/trainer/ppo/core_algos.py:1140-1206,1286-1376,2188-2251``,
+``verl/workers/utils/losses.py:57-155``) for the vanilla loss under any of ``agg_loss``'s aggregation modes, together
 with the gradients w.r.t. ``log_prob`` and ``entropy``, so the backward of ``linear_cross_entropy`` starts from two
 ready vectors instead of an elementwise autograd graph.  Metric names are the reference's.
 """
@@ -24,55 +24,88 @@ AGG_MODES = {
     "seq-mean-token-mean": 4,
 }
 
+# kl_penalty's estimators (core_algos.py:2228-2245); a trailing "+" selects the straight-through variant (:2201-2213)
+KL_TYPES = {"kl": 1, "k1": 1, "abs": 2, "mse": 3, "k2": 3, "low_var_kl": 4, "k3": 4}
+KL_STRAIGHT_THROUGH = 16
+
+
+def kl_type_number(kl_penalty: str) -> int:
+    base = kl_penalty[:-1] if kl_penalty.endswith("+") else kl_penalty
+    if base not in KL_TYPES:
+        raise NotImplementedError(f"kl_penalty {kl_penalty!r}")  # core_algos.py:2247-2251 ("full" included)
+    return KL_TYPES[base] | (KL_STRAIGHT_THROUGH if kl_penalty.endswith("+") else 0)
+
+
+def agg_numbers(loss_agg_mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor):
+    """agg_loss's arguments as the C ABI takes them; raises what the reference raises (core_algos.py:1172-1204)."""
+    if loss_agg_mode not in AGG_MODES:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    if dp_size > 1:
+        if loss_agg_mode == "token-mean" and batch_num_tokens is None:
+            raise ValueError("(global) batch_num_tokens is required when dp_size > 1")
+        if loss_agg_mode.startswith("seq-mean") and global_batch_size is None:
+            raise ValueError("global_batch_size is required when dp_size > 1")
+    return (
+        AGG_MODES[loss_agg_mode],
+        float(dp_size),
+        -1.0 if batch_num_tokens is None else float(batch_num_tokens),
+        -1.0 if global_batch_size is None else float(global_batch_size),
+        -1.0 if loss_scale_factor is None else float(loss_scale_factor),
+    )
+
 
 class _FusedPPOLoss(torch.autograd.Function):
+    """``log_prob`` may be None: then the call is ``agg_loss`` of ``entropy`` (the C ABI's aggregation-only form)."""
+
     @staticmethod
-    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, agg, clip_low, clip_high,
-                clip_c, entropy_coeff):
-        assert log_prob.is_cuda, "fused_ppo_loss runs on the GPU only"
-        dev = log_prob.device
-        shape = log_prob.shape
+    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, agg, kl,
+                clip_low, clip_high, clip_c, entropy_coeff):
+        lead = log_prob if log_prob is not None else entropy
+        assert lead.is_cuda, "fused_ppo_loss runs on the GPU only"
+        dev = lead.device
+        shape = lead.shape
 
         def f32(t):
-            return t.detach().reshape(-1).to(torch.float32).contiguous()
+            return None if t is None else t.detach().reshape(-1).to(torch.float32).contiguous()
 
-        lp, old, adv, mask = f32(log_prob), f32(old_log_prob), f32(advantages), f32(response_mask)
-        ent = None if entropy is None else f32(entropy)
-        isw = None if is_weights is None else f32(is_weights)
-        n = lp.numel()
-        assert old.numel() == n and adv.numel() == n and mask.numel() == n and (ent is None or ent.numel() == n)
-        assert isw is None or isw.numel() == n
+        lp, ent, old, adv, mask = f32(log_prob), f32(entropy), f32(old_log_prob), f32(advantages), f32(response_mask)
+        isw, ref = f32(is_weights), f32(ref_log_prob)
+        n = lead.numel()
+        for t in (lp, ent, old, adv, mask, isw, ref):
+            assert t is None or t.numel() == n, "all inputs have the shape of log_prob"
         # rows are the sequences the seq-mean modes average over: the last dimension is the response
         row_len = shape[-1] if len(shape) >= 1 else 1
         rows = n // row_len if row_len else 0
         mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor = agg
-        out = torch.empty(8, device=dev, dtype=torch.float32)
-        g_lp = torch.empty(n, device=dev, dtype=torch.float32)
+        kl_type, kl_coef = kl
+        out = torch.empty(16, device=dev, dtype=torch.float32)
+        g_lp = None if lp is None else torch.empty(n, device=dev, dtype=torch.float32)
         g_ent = None if ent is None else torch.empty(n, device=dev, dtype=torch.float32)
         lib = _abi.load()
         with torch.cuda.device(dev):
             ws_bytes = lib.lce_ppo_loss_workspace_bytes(rows, row_len)
             ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
             rc = lib.lce_ppo_loss(
-                lp.data_ptr(), _abi.ptr(ent), old.data_ptr(), adv.data_ptr(), mask.data_ptr(), _abi.ptr(isw), rows,
-                row_len, mode, clip_low, clip_high, clip_c, entropy_coeff, dp_size, batch_num_tokens,
-                global_batch_size, loss_scale_factor, out.data_ptr(), g_lp.data_ptr(), _abi.ptr(g_ent), ws.data_ptr(),
-                ws_bytes, _abi.current_stream(dev),
+                _abi.ptr(lp), _abi.ptr(ent), _abi.ptr(old), _abi.ptr(adv), mask.data_ptr(), _abi.ptr(isw),
+                _abi.ptr(ref), kl_type, kl_coef, rows, row_len, mode, clip_low, clip_high, clip_c, entropy_coeff,
+                dp_size, batch_num_tokens, global_batch_size, loss_scale_factor, out.data_ptr(), _abi.ptr(g_lp),
+                _abi.ptr(g_ent), ws.data_ptr(), ws_bytes, _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_ppo_loss")
-        ctx.save_for_backward(g_lp, g_ent if g_ent is not None else g_lp.new_empty(0))
-        ctx.has_entropy = ent is not None
+        empty = out.new_empty(0)
+        ctx.save_for_backward(g_lp if g_lp is not None else empty, g_ent if g_ent is not None else empty)
+        ctx.has = (lp is not None, ent is not None)
         ctx.shape = shape
-        ctx.dtypes = (log_prob.dtype, None if entropy is None else entropy.dtype)
+        ctx.dtypes = (None if log_prob is None else log_prob.dtype, None if entropy is None else entropy.dtype)
         ctx.mark_non_differentiable(out)
         return out[0], out
 
     @staticmethod
     def backward(ctx, g_loss, _g_out):
         g_lp, g_ent = ctx.saved_tensors
-        d_lp = (g_lp * g_loss).reshape(ctx.shape).to(ctx.dtypes[0])
-        d_ent = (g_ent * g_loss).reshape(ctx.shape).to(ctx.dtypes[1]) if ctx.has_entropy else None
-        return d_lp, d_ent, None, None, None, None, None, None, None, None, None
+        d_lp = (g_lp * g_loss).reshape(ctx.shape).to(ctx.dtypes[0]) if ctx.has[0] else None
+        d_ent = (g_ent * g_loss).reshape(ctx.shape).to(ctx.dtypes[1]) if ctx.has[1] else None
+        return (d_lp, d_ent) + (None,) * 11
 
 
 def fused_ppo_loss(
@@ -92,32 +125,26 @@ def fused_ppo_loss(
     global_batch_size: Optional[int] = None,
     loss_scale_factor: Optional[int] = None,
     rollout_is_weights: Optional[torch.Tensor] = None,
+    ref_log_prob: Optional[torch.Tensor] = None,
+    kl_loss_coef: float = 0.001,
+    kl_loss_type: str = "low_var_kl",
 ):
-    """Returns ``(policy_loss, metrics)``: ``policy_loss = pg_loss - entropy_coeff * entropy_loss`` (a 0-dim tensor
-    with autograd), ``metrics`` a dict of 0-dim tensors under the reference's keys (no host sync is forced).
+    """Returns ``(policy_loss, metrics)``: ``policy_loss = pg_loss - entropy_coeff * entropy_loss
+    [+ kl_loss_coef * kl_loss]`` (a 0-dim tensor with autograd), ``metrics`` a dict of 0-dim tensors under the
+    reference's keys (no host sync is forced).
     ``dp_size``, ``batch_num_tokens``, ``global_batch_size`` and ``loss_scale_factor`` are ``agg_loss``'s
     (``core_algos.py:1140-1206``); the sequences of the ``seq-mean-*`` modes are the rows of the last dimension.
-    ``rollout_is_weights`` multiplies the per-token policy loss (``core_algos.py:1362-1363``) and takes no gradient."""
-    if loss_agg_mode not in AGG_MODES:
-        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    ``rollout_is_weights`` multiplies the per-token policy loss (``core_algos.py:1362-1363``) and takes no gradient.
+    With ``ref_log_prob`` the KL penalty of ``ppo_loss`` (``use_kl_loss``, ``losses.py:142-153``) is added:
+    ``kl_loss_type`` is ``kl_penalty``'s estimator name, ``kl_loss_coef`` its weight."""
+    agg = agg_numbers(loss_agg_mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor)
     assert clip_ratio_c > 1.0, f"clip_ratio_c must be greater than 1.0, got {clip_ratio_c}"
     lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
     hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
-    if dp_size > 1:
-        if loss_agg_mode == "token-mean" and batch_num_tokens is None:
-            raise ValueError("(global) batch_num_tokens is required when dp_size > 1")
-        if loss_agg_mode.startswith("seq-mean") and global_batch_size is None:
-            raise ValueError("global_batch_size is required when dp_size > 1")
-    agg = (
-        AGG_MODES[loss_agg_mode],
-        float(dp_size),
-        -1.0 if batch_num_tokens is None else float(batch_num_tokens),
-        -1.0 if global_batch_size is None else float(global_batch_size),
-        -1.0 if loss_scale_factor is None else float(loss_scale_factor),
-    )
+    kl = (0, 0.0) if ref_log_prob is None else (kl_type_number(kl_loss_type), float(kl_loss_coef))
     loss, out = _FusedPPOLoss.apply(
-        log_prob, entropy, old_log_prob, advantages, response_mask, rollout_is_weights, agg, float(lo), float(hi),
-        float(clip_ratio_c), float(entropy_coeff),
+        log_prob, entropy, old_log_prob, advantages, response_mask, rollout_is_weights, ref_log_prob, agg, kl,
+        float(lo), float(hi), float(clip_ratio_c), float(entropy_coeff),
     )  # fmt: skip
     metrics = {
         "actor/pg_loss": out[1],
@@ -127,4 +154,7 @@ def fused_ppo_loss(
     }
     if entropy is not None:
         metrics["actor/entropy_loss"] = out[2]
+    if ref_log_prob is not None:
+        metrics["kl_loss"] = out[8]
+        metrics["kl_coef"] = kl_loss_coef
     return loss, metrics
