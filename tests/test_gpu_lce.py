@@ -186,7 +186,9 @@ def test_api_contract_on_device():
     with pytest.raises(NotImplementedError):
         linear_cross_entropy(h, w, y, 1.5, "none", object())
     with pytest.raises(NotImplementedError):
-        linear_cross_entropy(h.half(), w.half(), y, 1.5, "none")
+        linear_cross_entropy(h.double(), w.double(), y, 1.5, "none")
+    with pytest.raises(NotImplementedError):
+        linear_cross_entropy(h.half(), w, y, 1.5, "none")  # mixed dtypes
     with pytest.raises(AssertionError):
         linear_cross_entropy(h[:, :100].contiguous(), w[:, :100].contiguous(), y, 1.5, "none")  # H % 128
     with pytest.raises(AssertionError):

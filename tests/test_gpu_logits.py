@@ -157,5 +157,5 @@ def test_sum_pi_squared_at_the_reference_tests_cases(shape):
     want = torch.softmax(big.double(), dim=-1).pow(2).sum(dim=-1)
     assert torch.isfinite(got).all()
     torch.testing.assert_close(got.double(), want, atol=1e-5, rtol=1e-5)
-    with pytest.raises(NotImplementedError):  # fp64 logits: the kernels take bf16 and fp32
+    with pytest.raises(NotImplementedError):  # fp64 logits: the kernels take bf16, fp16 and fp32
         F.calculate_sum_pi_squared_from_logits(big.double())

@@ -29,10 +29,20 @@ def _case(seed):
 
 @pytest.mark.parametrize("seed", range(96))
 def test_random_shape(seed):
+    _check(seed, None)
+
+
+@pytest.mark.parametrize("seed", range(96, 128))
+def test_random_shape_fp16(seed):
+    _check(seed, torch.float16)
+
+
+def _check(seed, force_dtype):
     from verl_amd import linear_cross_entropy
     from verl_amd.utils.kernel import kernels
 
     dtype, T, H, V, tau, reduction, mask, vchunk = _case(seed)
+    dtype = force_dtype or dtype
     g = torch.Generator().manual_seed(1000 + seed)
     h = (torch.rand(T, H, generator=g) - 0.5).to(dtype).to(DEV)
     w = ((torch.rand(V, H, generator=g) - 0.5) * (4.0 / H ** 0.5)).to(dtype).to(DEV)

@@ -9,7 +9,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LCE_LIBRARY_PATH") or os.path.join(_HERE, "lib", "liblce_gfx950.so")
 
-DTYPE_BF16, DTYPE_F32 = 0, 1
+DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
 ABI_VERSION = 5
 
 # every symbol include/lce_abi.h declares: name -> (restype, argtypes)
@@ -94,7 +94,9 @@ def dtype_code(dtype) -> int:
         return DTYPE_BF16
     if dtype == torch.float32:
         return DTYPE_F32
-    raise NotImplementedError(f"verl_amd supports bfloat16 and float32 inputs, got {dtype}")
+    if dtype == torch.float16:
+        return DTYPE_F16
+    raise NotImplementedError(f"verl_amd supports bfloat16, float16 and float32 inputs, got {dtype}")
 
 
 def ptr(t) -> int | None:

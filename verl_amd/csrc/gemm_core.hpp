@@ -25,6 +25,8 @@ __device__ unsigned long long lce_dbg_times[16];
 
 typedef __bf16 bf16_t;
 typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16_t;
+typedef f16_t f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -69,6 +71,19 @@ struct Mma<bf16_t> {
 #endif
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
                                                   acc, 0, 0, 0);
+  }
+};
+
+// the same with IEEE half-precision operands
+template <>
+struct Mma<f16_t> {
+  static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
+#ifdef LCE_DBG_NO_MFMA
+    asm volatile("" ::"v"(a), "v"(b));
+    return;
+#endif
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
+                                                 acc, 0, 0, 0);
   }
 };
 

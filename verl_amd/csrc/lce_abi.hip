@@ -17,6 +17,9 @@ using namespace lce;
 
 namespace {
 
+bool known_dtype(int dtype) { return dtype == LCE_DTYPE_BF16 || dtype == LCE_DTYPE_F32 || dtype == LCE_DTYPE_F16; }
+size_t esize(int dtype) { return dtype == LCE_DTYPE_F32 ? 4 : 2; }
+
 thread_local char g_err[512] = "";
 // Defaults: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it only up
 // to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed
@@ -507,6 +510,9 @@ int dispatch_dtype_forward(int dtype, const void* h, int64_t ldh, const void* W,
   if (dtype == LCE_DTYPE_BF16)
     return forward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
                                                   reduction, lp, ent, mx, ac, eb, ws, st, label_offset, shard_out);
+  if (dtype == LCE_DTYPE_F16)
+    return forward_impl<typename Vt<f16_t>::Cfg>((const f16_t*)h, ldh, (const f16_t*)W, ldw, labels, T, H, V, temperature,
+                                                 reduction, lp, ent, mx, ac, eb, ws, st, label_offset, shard_out);
   return forward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
                                                reduction, lp, ent, mx, ac, eb, ws, st, label_offset, shard_out);
 }
@@ -520,6 +526,10 @@ int dispatch_dtype_backward(int dtype, const void* h, int64_t ldh, const void* W
     return backward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
                                                    reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st,
                                                    vocab_offset);
+  if (dtype == LCE_DTYPE_F16)
+    return backward_impl<typename Vt<f16_t>::Cfg>((const f16_t*)h, ldh, (const f16_t*)W, ldw, labels, T, H, V, temperature,
+                                                  reduction, mx, ac, eb, glp, gent, (f16_t*)dh, (f16_t*)dw, ws, vchunk, st,
+                                                  vocab_offset);
   return backward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
                                                 reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st, vocab_offset);
 }
@@ -529,19 +539,21 @@ int dispatch_dtype_gemm(int dtype, const void* A, int64_t lda, const void* B, in
                         int64_t N, int64_t K, hipStream_t st) {
   if (dtype == LCE_DTYPE_BF16)
     return launch_gemm<typename Vt<bf16_t>::Cfg>((const bf16_t*)A, lda, (const bf16_t*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0, st);
+  if (dtype == LCE_DTYPE_F16)
+    return launch_gemm<typename Vt<f16_t>::Cfg>((const f16_t*)A, lda, (const f16_t*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0, st);
   return launch_gemm<typename Vt<float>::Cfg>((const float*)A, lda, (const float*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0, st);
 }
 
 int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
                  int64_t H, int64_t V, int dtype, float temperature, int reduction) {
-  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
-  const int64_t kmul = dtype == LCE_DTYPE_BF16 ? 64 : 32, ldmul = dtype == LCE_DTYPE_BF16 ? 8 : 4;
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  const int64_t kmul = esize(dtype) == 2 ? 64 : 32, ldmul = esize(dtype) == 2 ? 8 : 4;
   if (T < 0 || H <= 0 || V <= 0) return fail(LCE_E_ARG, "bad shape T=%lld H=%lld V=%lld", (long long)T, (long long)H, (long long)V);
   if (V >= (1LL << 31) || T >= (1LL << 31)) return fail(LCE_E_ARG, "T and V must be below 2^31");
   if (H % kmul != 0) return fail(LCE_E_ARG, "hidden size %lld must be a multiple of %lld", (long long)H, (long long)kmul);
   if (ldh < H || ldw < H || ldh % ldmul != 0 || ldw % ldmul != 0) return fail(LCE_E_ARG, "bad row strides ldh=%lld ldw=%lld", (long long)ldh, (long long)ldw);
   // the loads address a 256-row tile with 32-bit byte offsets from its first row
-  const int64_t esz = dtype == LCE_DTYPE_BF16 ? 2 : 4;
+  const int64_t esz = esize(dtype);
   if (ldh * esz * 256 >= (1LL << 32) || ldw * esz * 256 >= (1LL << 32))
     return fail(LCE_E_ARG, "row strides ldh=%lld ldw=%lld too large: 256 rows must span less than 4 GiB", (long long)ldh, (long long)ldw);
   if (T > 0 && (!hidden || !weight || !labels)) return fail(LCE_E_ARG, "null input pointer");
@@ -647,7 +659,7 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
   if (!g_variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
   // the split ring: measured 4-7% faster than the 2-stage ring up to 8192 tokens, equal (+-1%) beyond, and
   // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
-  if (!g_variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * (dtype == LCE_DTYPE_BF16 ? 2 : 4) > (512ull << 20)))
+  if (!g_variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)))
     return LCE_FWD(Variant2);
   switch (g_variant_fwd) {
     case 1: return LCE_FWD(Variant1);
@@ -708,7 +720,7 @@ int lce_merge_shards(const float* partials, int R, int64_t T, int reduction, flo
 
 size_t lce_backward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype, int64_t vchunk) {
   if (T <= 0 || H <= 0 || V <= 0) return 256;
-  return bwd_layout(T, H, V, dtype == LCE_DTYPE_BF16 ? 2 : 4, vchunk).total + 256;
+  return bwd_layout(T, H, V, esize(dtype), vchunk).total + 256;
 }
 
 // shared body of lce_backward and lce_backward_shard
@@ -720,7 +732,7 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-  const size_t esz = dtype == LCE_DTYPE_BF16 ? 2 : 4;
+  const size_t esz = esize(dtype);
   if (!d_weight) return fail(LCE_E_ARG, "null d_weight");
   if (T == 0) {
     const int64_t words = (int64_t)((size_t)V * H * esz / 4);
@@ -766,7 +778,7 @@ int lce_backward_shard(const void* hidden, int64_t ldh, const void* weight_shard
 
 int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
                 int64_t K, int dtype, int variant, void* stream) {
-  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (!A || !B || !C || !aligned16(A) || !aligned16(B)) return fail(LCE_E_ARG, "bad pointer");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define LCE_GEMM(Vt) dispatch_dtype_gemm<Vt>(dtype, A, lda, B, ldb, C, ldc, M, N, K, st)
@@ -797,7 +809,7 @@ int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 
 int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                        float* logprobs, float* entropy, float* stats, void* stream) {
-  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
   if (R == 0) return LCE_OK;
   if (!logits || (logprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
@@ -806,13 +818,15 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   ProfScope prof(PC_LOGITS_FWD, st);
   if (dtype == LCE_DTYPE_BF16)
     hipLaunchKernelGGL((logits_fwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, logprobs, entropy, stats);
+  else if (dtype == LCE_DTYPE_F16)
+    hipLaunchKernelGGL((logits_fwd_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, labels, V, logprobs, entropy, stats);
   else
     hipLaunchKernelGGL((logits_fwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, logprobs, entropy, stats);
   return check_launch("logits_fwd_kernel");
 }
 
 int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream) {
-  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
   if (R == 0) return LCE_OK;
   if (!logits || !out) return fail(LCE_E_ARG, "null pointer");
@@ -821,6 +835,8 @@ int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_
   ProfScope prof(PC_LOGITS_FWD, st);
   if (dtype == LCE_DTYPE_BF16)
     hipLaunchKernelGGL((logits_pi2_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, V, out);
+  else if (dtype == LCE_DTYPE_F16)
+    hipLaunchKernelGGL((logits_pi2_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, V, out);
   else
     hipLaunchKernelGGL((logits_pi2_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, V, out);
   return check_launch("logits_pi2_kernel");
@@ -907,7 +923,7 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,
                         const float* stats, const float* dlogprobs, const float* dentropy, void* d_logits, int64_t ldd,
                         void* stream) {
-  if (dtype != LCE_DTYPE_BF16 && dtype != LCE_DTYPE_F32) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V || ldd < V) return fail(LCE_E_ARG, "bad shape");
   if (R == 0) return LCE_OK;
   if (!logits || !d_logits || (dlogprobs && !labels)) return fail(LCE_E_ARG, "null pointer");
@@ -916,6 +932,8 @@ int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, 
   ProfScope prof(PC_LOGITS_BWD, st);
   if (dtype == LCE_DTYPE_BF16)
     hipLaunchKernelGGL((logits_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, labels, V, stats, dlogprobs, dentropy, (bf16_t*)d_logits, ldd);
+  else if (dtype == LCE_DTYPE_F16)
+    hipLaunchKernelGGL((logits_bwd_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, labels, V, stats, dlogprobs, dentropy, (f16_t*)d_logits, ldd);
   else
     hipLaunchKernelGGL((logits_bwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, labels, V, stats, dlogprobs, dentropy, (float*)d_logits, ldd);
   return check_launch("logits_bwd_kernel");

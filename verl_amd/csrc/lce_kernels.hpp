@@ -358,6 +358,8 @@ template <int N>
 struct VecOf<float, N> { typedef float type __attribute__((ext_vector_type(N))); };
 template <int N>
 struct VecOf<bf16_t, N> { typedef bf16_t type __attribute__((ext_vector_type(N))); };
+template <int N>
+struct VecOf<f16_t, N> { typedef f16_t type __attribute__((ext_vector_type(N))); };
 
 // store N consecutive elements (N * sizeof(T) <= 16 bytes per store; wider runs are split);
 // STREAM: non-temporal stores, for data that this kernel does not read back
