@@ -124,3 +124,29 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr
+
+
+def test_process_group_of_one_rank_is_the_single_gpu_path():
+    """Megatron hands its tensor-parallel group over even at size 1 (verl/models/mcore/model_forward_fused.py:110-117)."""
+    import torch.distributed as dist
+
+    from verl_amd.utils.kernel.kernels import _require_single_rank
+
+    class Two:
+        def size(self):
+            return 2
+
+    _require_single_rank(None)
+    with pytest.raises(NotImplementedError):
+        _require_single_rank(Two())
+    with pytest.raises(NotImplementedError):
+        _require_single_rank(object())
+    created = not dist.is_initialized()
+    if created:
+        dist.init_process_group("gloo", init_method="tcp://127.0.0.1:29531", rank=0, world_size=1)
+    try:
+        _require_single_rank(dist.group.WORLD)
+        _require_single_rank(dist.new_group([0]))
+    finally:
+        if created:
+            dist.destroy_process_group()

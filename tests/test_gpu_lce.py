@@ -185,6 +185,14 @@ def test_api_contract_on_device():
     # unsupported pieces fail loudly
     with pytest.raises(NotImplementedError):
         linear_cross_entropy(h, w, y, 1.5, "none", object())
+
+    class OneRank:  # stands for a process group of one rank (Megatron at tensor-parallel size 1)
+        def size(self):
+            return 1
+
+    g_lp, g_ent = linear_cross_entropy(h, w, y, 1.5, "none", OneRank())
+    p_lp, p_ent = linear_cross_entropy(h, w, y, 1.5, "none")
+    assert torch.equal(g_lp, p_lp) and torch.equal(g_ent, p_ent)
     with pytest.raises(NotImplementedError):
         linear_cross_entropy(h.double(), w.double(), y, 1.5, "none")
     with pytest.raises(NotImplementedError):

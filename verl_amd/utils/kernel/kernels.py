@@ -11,7 +11,9 @@ Differences that are deliberate (all inside the reference's own tolerances):
 * ``BackwardEnum`` values are accepted by ``set_backward_method`` but select nothing: there is one
   backward schedule (recompute a vocab-chunk of d_logits, then two MFMA GEMMs);
 * labels outside ``[0, V)`` give ``logprob = -logsumexp`` instead of reading uninitialised memory;
-* ``dist_process_group`` (vocab-parallel) raises ``NotImplementedError``.
+* ``dist_process_group`` with more than one rank (vocab-parallel) raises ``NotImplementedError``; a group of one
+  rank (what Megatron passes at tensor-parallel size 1, ``verl/models/mcore/model_forward_fused.py:110-117``) is the
+  single-GPU path.
 """
 
 from __future__ import annotations
@@ -77,6 +79,24 @@ def set_vocab_chunk(columns: int):
     _config._vocab_chunk = int(columns)
 
 
+def _require_single_rank(dist_process_group) -> None:
+    """The vocabulary is not sharded here: only ``None`` or a process group of exactly one rank is accepted."""
+    if dist_process_group is None:
+        return
+    try:
+        size = getattr(dist_process_group, "size", None)
+        if callable(size):
+            world = int(size())
+        else:
+            import torch.distributed as dist
+
+            world = dist.get_world_size(dist_process_group)
+    except Exception:
+        world = -1  # not a process group
+    if world != 1:
+        raise NotImplementedError("vocab-parallel (dist_process_group) is not built: one GPU, no collectives")
+
+
 def _check_inputs(hidden, weight, labels):
     assert hidden.is_cuda and weight.is_cuda and labels.is_cuda
     assert weight.device == hidden.device and labels.device == hidden.device
@@ -100,8 +120,7 @@ def efficient_entropy_forward(
     dist_process_group=None,
 ) -> list[torch.Tensor]:
     """Returns (logprobs, entropy, maximum, accumulate, entropy_b), all fp32."""
-    if dist_process_group is not None:
-        raise NotImplementedError("vocab-parallel (dist_process_group) is not built: one GPU, no collectives")
+    _require_single_rank(dist_process_group)
     code = _check_inputs(hidden, weight, labels)
     reduction = get_entropy_reduction_enum(reduction)
     assert temperature > 0, "temperature must be positive"
@@ -146,8 +165,7 @@ def efficient_entropy_backward(
     dist_process_group=None,
 ) -> list[torch.Tensor]:
     """Returns (d_hidden, d_weight) in ``hidden.dtype`` (fp32 when ``should_return_fp32_grad``)."""
-    if dist_process_group is not None:
-        raise NotImplementedError("vocab-parallel (dist_process_group) is not built: one GPU, no collectives")
+    _require_single_rank(dist_process_group)
     if _config._backward == BackwardEnum._Split_Dlogits_M:
         raise NotImplementedError("BackwardEnum._Split_Dlogits_M is not implemented yet")
     code = _check_inputs(hidden, weight, labels)
