@@ -258,13 +258,42 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()  # (torch's current stream is the stream the library launches on)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = T / (elapsed / args.steps)
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    step_ms = {"median": per_step[len(per_step) // 2], "min": per_step[0], "max": per_step[-1]}
+
+    # Peak device memory of one forward and one backward beyond what is live before each (outputs, saved
+    # statistics, returned gradients and the workspace included), next to the bound the workspace is sized
+    # under and to what ONE materialised [T, V] tensor in the input dtype would take.
+    memory = None
+    if not fwd_only and not ppo:
+        h.grad = None
+        w.grad = None
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated(dev)
+        torch.cuda.reset_peak_memory_stats(dev)
+        lp, ent = linear_cross_entropy(h, w, y, tau, "none")
+        torch.cuda.synchronize()
+        fwd_peak = torch.cuda.max_memory_allocated(dev) - base
+        base = torch.cuda.memory_allocated(dev)
+        torch.cuda.reset_peak_memory_stats(dev)
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        torch.cuda.synchronize()
+        bwd_peak = torch.cuda.max_memory_allocated(dev) - base
+        del lp, ent
+        memory = {"forward_peak_extra_bytes": fwd_peak, "backward_peak_extra_bytes": bwd_peak,
+                  "returned_gradients_bytes": (T * H + V * H) * 2,
+                  "workspace_bound_bytes": 0.25 * T * V * 2 + 4.0 * V * H,
+                  "one_materialised_TV_tensor_bytes": T * V * 2}
 
     # per-kernel durations with HIP events on the launch stream (second pass, same process)
     lib.lce_profile_enable(1)
@@ -331,6 +360,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "step_ms": step_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -338,6 +368,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau,
                    "pass": "fwd+ppo_loss+bwd" if ppo else "fwd+bwd", "tokens_with_gradient": t_active},
+        "memory": memory,
         "algorithmic_tflops": algorithmic / 1e12,  # 6*T*V*H per step, the reference's accounting per token
         "frac_of_bf16_peak": algorithmic / PEAK_BF16,
         # what the kernels execute: forward on T tokens, recompute + two GEMMs on the tokens with gradient
