@@ -263,6 +263,25 @@ def test_config2_full_size_properties_and_sampled_parity():
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2) and torch.equal(dh, dh2) and torch.equal(dw, dw2)
 
 
+def test_config2_full_size_against_the_whole_oracle():
+    """The benchmark's workload itself (Qwen2.5-7B-shaped head, T=16384, H=3584, V=152064, tau=1, dense N(0,1)
+    upstream gradients, same seed as bench.py's inputs are drawn from): every log-prob, entropy, d_hidden and
+    d_weight entry against the oracle."""
+    T, H, V, tau = 16384, 3584, 152064, 1.0
+    h, w, y, g_lp, g_ent = _config_case(T, H, V, 0.02, seed=1236)
+    lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rlp, rent = O.lce_forward(h, w, y, tau, chunk=2048)
+    assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2
+    torch.testing.assert_close(lp, rlp, atol=1e-3, rtol=2e-4)
+    torch.testing.assert_close(ent, rent, atol=5e-3, rtol=5e-4)
+    del rlp, rent
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, chunk=2048)
+    assert_bf16_bar(dh, rdh)
+    assert_bf16_bar(dw, rdw)
+    torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)  # the reference's own tolerance
+    torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
 def test_wide_hidden_and_256k_vocabulary():
     """H = 8192 and V = 262144 (the largest vocabularies in use): 4.3 GB of weights, row offsets beyond
     2^31 bytes inside W, 128 K-slabs per logit tile; a quarter of the tokens without gradient."""
