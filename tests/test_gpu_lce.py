@@ -606,3 +606,84 @@ def test_memory_gate_no_T_by_V_tensor():
     bwd_peak = torch.cuda.max_memory_allocated() - base
     grads = (T * H + V * H) * 2
     assert bwd_peak - grads < 0.25 * T * V * 2 + 4 * V * H, (bwd_peak, grads)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_extreme_logits_closed_forms(dtype):
+    """Closed forms at the ends of the numeric range.  (1) Every logit of a token equal (W = 0, or one shared
+    weight row so that all logits are -|large|): entropy = log V, logprob = -log V, and d_logits reduces to
+    g_lp (1[v=y] - 1/V) / tau, whatever the common value (shift invariance; the reference seeds its running max
+    with 0 and loses tokens whose logits are all far below it, verl/utils/kernel/kernels.py:387).
+    (2) One logit far above the rest (temperature 0.05): entropy -> 0, logprob of the top label -> 0, of any other
+    label = its logit gap; gradients finite and equal to the oracle's."""
+    from verl_amd import linear_cross_entropy
+
+    T, H, V = 300, 256, 5003
+    g = torch.Generator().manual_seed(4)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = torch.randn(T, generator=g).to(DEV)
+    g_ent = torch.randn(T, generator=g).to(DEV)
+    h = torch.ones(T, H, dtype=dtype, device=DEV)
+    for fill, tau in ((0.0, 1.0), (-2.0, 0.5)):  # logits 0, and -2 * 256 / 0.5 = -1024 for every vocabulary entry
+        w = torch.full((V, H), fill, dtype=dtype, device=DEV)
+        hh, ww = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        lp, ent = linear_cross_entropy(hh, ww, y, tau, "none")
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        torch.testing.assert_close(ent, torch.full((T,), math.log(V), device=DEV), atol=1e-4, rtol=1e-5)
+        torch.testing.assert_close(lp, torch.full((T,), -math.log(V), device=DEV), atol=1e-4, rtol=1e-5)
+        dz = -g_lp[:, None].expand(T, V) / V / tau
+        want_dw = (dz.double().t() @ h.double())
+        want_dw.index_add_(0, y, (g_lp / tau).double()[:, None] * h.double())
+        want_dh = fill * (dz.double().sum(1, keepdim=True) + (g_lp / tau).double()[:, None]).expand(T, H)
+        tol = dict(atol=2e-2, rtol=2e-2) if dtype == torch.bfloat16 else dict(atol=1e-5, rtol=1e-4)
+        torch.testing.assert_close(ww.grad.double(), want_dw, **tol)
+        # d_hidden is an exact cancellation here (sum_v dz = 0 times a constant weight row).  With 16-bit inputs the
+        # V equal softmax terms are rounded to the input format before the GEMM (as the reference's _d_logits is,
+        # kernels.py:1666-1724), all in the same direction: allow that format's 2^-8 of the cancelling magnitude.
+        # (fp32: 1e-5 relative, of the cancelling magnitude)
+        # the entropy term carries (z - b), an exact zero formed from two numbers of size |z| = |fill| H / tau
+        rel = 2.0**-8 if dtype == torch.bfloat16 else 1e-5
+        slack = rel * abs(fill) * (2 * g_lp.abs() + g_ent.abs() * abs(fill) * H / tau)[:, None] / tau
+        assert ((hh.grad.double() - want_dh).abs() <= tol["atol"] + slack).all()
+    # (2) a dominant logit: row v of W is e_v-like along one hidden unit per 'class' bucket
+    w = torch.zeros(V, H, dtype=dtype, device=DEV)
+    w[:, 0] = 0.5
+    top = torch.randint(0, V, (T,), generator=g).to(DEV)
+    hh = torch.zeros(T, H, dtype=dtype, device=DEV)
+    hh[:, 0] = 1.0
+    w[torch.arange(256, device=DEV), torch.arange(256, device=DEV) % (H - 1) + 1] = 2.0  # 256 special rows
+    sel = torch.arange(T, device=DEV) % 256
+    hh[torch.arange(T, device=DEV), sel % (H - 1) + 1] = 3.0  # token t: logit 6.5 on row sel (and its alias row), 0.5 elsewhere
+    tau = 0.05  # gaps of 6 / 0.05 = 120 nats
+    y2 = torch.where(torch.arange(T, device=DEV) % 2 == 0, sel, top)
+    h2, w2 = hh.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(h2, w2, y2, tau, "none")
+    torch.autograd.backward([lp, ent], [g_lp, g_ent])
+    rlp, rent = O.lce_forward(hh, w, y2, tau, compute_dtype=torch.float64)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, hh, w, y2, tau, compute_dtype=torch.float64)
+    assert torch.isfinite(lp).all() and torch.isfinite(ent).all() and torch.isfinite(h2.grad).all() and torch.isfinite(w2.grad).all()
+    torch.testing.assert_close(lp.double(), rlp, atol=1e-3, rtol=1e-5)
+    torch.testing.assert_close(ent.double(), rent, atol=1e-4, rtol=1e-4)
+    # With 16-bit inputs every softmax term of d_logits, -p (G + g_ent (z - b) / tau), G = g_lp / tau (here up to 60),
+    # passes through the 16-bit d_logits format once (up to 2^-8 relative each, as the reference's _d_logits does,
+    # kernels.py:1666-1724) while the one-hot part G stays in fp32.  A token that is certain of its label has
+    # d_logits[label] = G (1 - p) with p -> 1: that cancellation is then good to the format's rounding of |G p|
+    # times |W[label]| (d_hidden) and |h| (the label's row of d_weight).  At the magnitudes of a model
+    # (|G| <= 10, |W| <= 0.1) that is below 4e-3.  With fp32 inputs the same cancellation is good to the rounding
+    # of p = exp(z - logsumexp) at |z| = 130: a few ulps of |z|, relative.
+    z = hh.double() @ w.double().t() / tau
+    P = torch.softmax(z, -1)
+    bstat = (P * z).sum(-1, keepdim=True)
+    soft = P * ((g_lp.abs() / tau).double()[:, None] + (g_ent.abs() / tau).double()[:, None] * (z - bstat).abs())
+    rel = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-20 * z.abs().max().item()  # (fp32: ~8 ulps of the log2-domain exponent)
+    floor = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    # (z - b) of the entropy term is formed in fp32 from two numbers of size |z|: a few ulps of |z| per term
+    soft = soft + 2.0**-21 * P * (g_ent.abs() / tau).double()[:, None] * z.abs() * (1.0 / rel)
+    bound_dh = floor + rel * rdh.abs() + rel * (soft @ w.double().abs())
+    # (d_weight: the softmax terms are rounded to the output format once more before the fp32 one-hot sums are added)
+    bound_dw = floor + rel * rdw.abs() + 2 * rel * (soft.t() @ hh.double().abs())
+    for name, got, want, bound in (("d_hidden", h2.grad, rdh, bound_dh), ("d_weight", w2.grad, rdw, bound_dw)):
+        excess = (got.double() - want).abs() - bound
+        i = int(excess.argmax())
+        assert excess.max() <= 0, (name, i // H, i % H, got.reshape(-1)[i].item(), want.reshape(-1)[i].item(),
+                                   bound.reshape(-1)[i].item())
