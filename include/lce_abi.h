@@ -167,10 +167,12 @@ int lce_num_variants(void);
  * LCE_OPT_DW_TRANSPOSED_READS (default 1, bf16 only): the d_weight GEMM reads the token-major d_logits with
  * transposing LDS reads; 0 builds a second, vocab-major copy of the d_logits for it (changes the workspace size:
  * set it before querying lce_backward_workspace_bytes).
- * LCE_OPT_LABEL_TERM_OUTSIDE (default 1, bf16 only): the one-hot part g_logprob / temperature * 1[v == label] of the
- * gradient of the logits is added to d_hidden and to the label rows of d_weight in fp32 instead of being rounded
- * to bf16 with the rest of the d_logits tile; 0 keeps it inside the tile, which is the reference's data format
- * (verl/utils/kernel/kernels.py:1666-1724).  Changes the workspace size like the option above. */
+ * LCE_OPT_LABEL_TERM_OUTSIDE (default 2, 16-bit inputs only): 1 = the one-hot part g_logprob / temperature * 1[v == label]
+ * of the gradient of the logits is added to d_hidden and to the label rows of d_weight in fp32 instead of being rounded
+ * to 16 bits with the rest of the d_logits tile; 2 = the label's whole entry of d_logits (one-hot and softmax part,
+ * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32; 0 keeps everything inside
+ * the tile, which is the reference's data format (verl/utils/kernel/kernels.py:1666-1724).  Changes the workspace size
+ * like the option above. */
 enum {
   LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
   LCE_OPT_DLOGITS_TOKENS_FIRST = 2,

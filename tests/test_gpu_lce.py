@@ -353,7 +353,7 @@ def _d_weight_rounding_bound(h, w, y, tau, g_lp, g_ent, rdw, chunk=2048):
     return 2e-2 + 2.0**-9 * absdw + 2.0**-8 * rdw.abs()
 
 
-@pytest.mark.parametrize("label_term_outside", [1, 0])
+@pytest.mark.parametrize("label_term_outside", [2, 1, 0])
 def test_config3_full_size_against_the_whole_oracle(label_term_outside):
     """Llama-3-8B-shaped head at full size: T = 8 x 4096, H=4096, V=128256, tau=0.6, a response mask that zeroes a
     random suffix of each row (valid length U{512..4096}).  Every output is compared with the oracle.  At this
@@ -375,7 +375,7 @@ def test_config3_full_size_against_the_whole_oracle(label_term_outside):
         assert lib.lce_set_option(4, label_term_outside) == 0
         lp, ent, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
     finally:
-        lib.lce_set_option(4, 1)
+        lib.lce_set_option(4, 2)  # the default
     rlp, rent = O.lce_forward(h, w, y, tau, chunk=2048)
     rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, chunk=2048)
     assert (lp - rlp).abs().max() < 2e-2 and (ent - rent).abs().max() < 2e-2

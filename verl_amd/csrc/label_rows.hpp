@@ -11,6 +11,8 @@
 // The second sum needs the tokens grouped by label in a fixed order: a stable LSD radix sort of
 // (label row, position in the token list) pairs, 8 bits per pass, written here (no float atomics anywhere, and
 // no library call that a captured graph could not replay).
+// In the default mode G_t above is replaced by the label's whole entry of d_logits, softmax part included
+// (label_coef_kernel), and the tiles hold zero at the label.
 #pragma once
 
 #include "lce_kernels.hpp"
@@ -25,6 +27,47 @@ LCE_DEV uint32_t label_row(const LabelTerm& lt, int64_t tok, float& G) {
   G = lt.g_lp[tok * lt.g_stride] * lt.scale;
   const int64_t y = lt.labels[tok] - lt.v0;
   return (G != 0.f && y >= 0 && y < lt.V) ? (uint32_t)y : kNoRow;
+}
+
+// coef[t] = d_logits[t][label_t] in fp32, the whole entry: p * (C0 + C1 * x) + G with x = hidden[t] . W[label_t]
+// recomputed here (one wave per token, 16-byte loads, a fixed shuffle tree), p = exp(x / tau - logsumexp_t).  With it
+// the tiles leave the label's entry out altogether, so that for a token that is certain of its label the small
+// number G * (1 - p) is formed in fp32 instead of as the difference of G (fp32) and G * p (rounded to 16 bits).
+// Zero for tokens without upstream gradient and for labels outside this call's rows of W.  H a multiple of 8.
+template <typename T>
+__global__ __launch_bounds__(256) void label_coef_kernel(const T* h, int64_t ldh, const T* W, int64_t ldw, const int64_t* labels,
+                                                         int64_t v0, int64_t V, int64_t ntok, int64_t H, const float* maximum,
+                                                         const float* accumulate, const float* entropy_b, const float* g_lp,
+                                                         int64_t g_stride, float g_scale, const float* g_ent, float rcp_tau,
+                                                         float c, float* coef) {
+  static_assert(sizeof(T) == 2, "16-bit inputs");
+  typedef typename VecOf<T, 8>::type vec_t;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= ntok) return;
+  const float glp = g_lp[t * g_stride] * g_scale;
+  const float gent = g_ent ? g_ent[t] : 0.f;
+  const int64_t y = labels[t] - v0;
+  float out = 0.f;
+  if ((glp != 0.f || gent != 0.f) && y >= 0 && y < V) {  // (uniform over the wave)
+    const T* hr = h + t * ldh;
+    const T* wr = W + y * ldw;
+    float x = 0.f;
+    for (int64_t k = (int64_t)lane * 8; k < H; k += 64 * 8) {
+      const vec_t a = *reinterpret_cast<const vec_t*>(hr + k);
+      const vec_t b = *reinterpret_cast<const vec_t*>(wr + k);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x = __builtin_fmaf((float)a[e], (float)b[e], x);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
+    const float lse2 = (maximum[t] + logf(accumulate[t])) * kLog2e;
+    const float G = glp * rcp_tau;
+    const float C1 = -gent * rcp_tau * rcp_tau;
+    const float C0 = -G + gent * entropy_b[t] * rcp_tau;
+    out = fast_exp2(__builtin_fmaf(x, c, -lse2)) * __builtin_fmaf(x, C1, C0) + G;
+  }
+  if (lane == 0) coef[t] = out;
 }
 
 // keys[k] = label row of the k-th listed token (rows[k], or k itself without a list), vals[k] = that token;

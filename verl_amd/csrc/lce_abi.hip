@@ -29,7 +29,7 @@ int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
 int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
 int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
-int g_label_outside = 1;  // 16-bit inputs: one-hot part of d_logits added in fp32 outside the d_logits tiles
+int g_label_outside = 2;  // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
 int g_dw_transposed_reads = 1;  // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
 
 int fail(int code, const char* fmt, ...) {
@@ -220,7 +220,7 @@ int forward_splits_upper_bound(int64_t T) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_keys[2], off_vals[2], off_hist, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_coef, off_keys[2], off_vals[2], off_hist, total;
   int sort_items, sort_passes;  // label sort (0 items: the one-hot part stays inside the d_logits tiles)
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
@@ -296,6 +296,8 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
     L.off_vals[b] = o; o += align256((size_t)L.sort_items * 4);
   }
   L.off_hist = o;  o += align256((size_t)(L.sort_items / kSortBlock) * 256 * 4);
+  // per-token coefficient of the label's entry of d_logits, when the whole entry is kept out of the tiles
+  L.off_coef = o;  o += (L.sort_items && g_label_outside == 2) ? align256((size_t)T * 4) : 0;
   L.total = o;
   return L;
 }
@@ -357,6 +359,14 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   if (L.sort_items) {
     lt.labels = labels;
     ProfScope prof(PC_LABEL_ROWS, st);
+    if constexpr (sizeof(TIN) == 2) if (g_label_outside == 2) {
+      float* coef = reinterpret_cast<float*>(ws + L.off_coef);
+      hipLaunchKernelGGL(label_coef_kernel<TIN>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, h, ldh, W, ldw, labels, vocab_offset, V, T,
+                         H, maximum, accumulate, entropy_b, dlogprobs, lt.g_stride, reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f,
+                         dentropy, 1.0f / temperature, kLog2e / temperature, coef);
+      if ((rc = check_launch("label_coef_kernel"))) return rc;
+      lt.g_lp = coef; lt.g_stride = 1; lt.scale = 1.0f;
+    }
     const int nblocks = L.sort_items / kSortBlock;
     if (nblocks == 1) {
       hipLaunchKernelGGL(label_sort_single_kernel, dim3(1), dim3(256), 0, st, lt, rows, n_rows, T, L.sort_passes, skeys[0], svals[0],
@@ -410,7 +420,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_ent = dentropy;
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = L.tn ? nullptr : dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       d.rows = rows; d.n_rows = n_rows;
-      d.label_outside = lt.labels != nullptr;
+      d.label_outside = lt.labels != nullptr ? g_label_outside : 0;
       const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
       // faster on the launch while `hidden` is small enough to stay in the memory-side cache next to the
@@ -593,7 +603,10 @@ int lce_set_option(int key, int64_t value) {
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
     case LCE_OPT_DW_TRANSPOSED_READS: g_dw_transposed_reads = value != 0; return LCE_OK;
-    case LCE_OPT_LABEL_TERM_OUTSIDE: g_label_outside = value != 0; return LCE_OK;
+    case LCE_OPT_LABEL_TERM_OUTSIDE:
+      if (value < 0 || value > 2) return fail(LCE_E_ARG, "LCE_OPT_LABEL_TERM_OUTSIDE takes 0, 1 or 2");
+      g_label_outside = (int)value;
+      return LCE_OK;
     case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }

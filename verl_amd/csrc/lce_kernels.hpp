@@ -317,7 +317,8 @@ struct DsArgs {
   const int* rows;
   const int* n_rows;
   int label_outside;  // 1: the tiles hold the softmax terms only; the one-hot part g_lp / tau * 1[v == label] is added
-                      // elsewhere in fp32 (label_rows.hpp)
+                      // elsewhere in fp32 (label_rows.hpp); 2: the label's whole entry is left out of the tiles (zero
+                      // there) and added elsewhere in fp32; 0: everything inside the tiles
 };
 
 // The two gradient GEMMs sum over the vocabulary (d_hidden) and over the tokens (d_weight); any
@@ -378,12 +379,13 @@ LCE_DEV void store_run(T* dst, const float (&v)[N]) {
 }
 
 // d_logits of one accumulator element; SLOW adds the label one-hot and masks padded rows / tokens
+// (drop: the label's entry is not part of the tile at all, it is added elsewhere in fp32)
 template <bool SLOW>
-LCE_DEV float dlogit(float x, float c, float lse2, float C0, float C1, float G, bool hit, bool dead) {
+LCE_DEV float dlogit(float x, float c, float lse2, float C0, float C1, float G, bool hit, bool dead, bool drop) {
   const float pr = fast_exp2(__builtin_fmaf(x, c, -lse2));
   float dv = pr * __builtin_fmaf(x, C1, C0);
   if (SLOW) {
-    if (hit) dv += G;
+    if (hit) dv = drop ? 0.f : dv + G;
     if (dead) dv = 0.f;
   }
   return dv;
@@ -428,7 +430,7 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
       C1[j] = -gent * p.rcp_tau * p.rcp_tau;
       C0[j] = -G[j] + gent * p.entropy_b[tok] * p.rcp_tau;
       const int64_t y = p.labels[tok] - p.v0;
-      rel[j] = (!p.label_outside && y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
+      rel[j] = (p.label_outside != 1 && y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
     }
   }
   const bool tok_group_live = p.dST != nullptr && tok0 < p.tpad;  // the whole token group is inside dS^T's columns
@@ -448,7 +450,7 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
           d[j] = dlogit<SLOW>(acc[i][j][r], p.c, lse2[j], C0[j], C1[j], G[j], row == rel[j],
-                              !tok_ok[j] || vloc0 + row >= p.vrows);
+                              !tok_ok[j] || vloc0 + row >= p.vrows, p.label_outside == 2);
           stage[j][rr] = d[j];
         }
         if (tok_group_live) store_run<TIN, FN>(dst_t + (int64_t)(vloc0 + row) * p.ldST, d);
@@ -503,7 +505,7 @@ LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
 #pragma unroll
   for (int j = 0; j < Cfg::FN; ++j) {
     const int64_t tok = tok0 + j * 32 + ln;
-    if (tok < Tc && !p.label_outside) {
+    if (tok < Tc && p.label_outside != 1) {
       const int64_t y = p.labels[p.rows ? p.rows[tok] : tok] - p.v0;
       has_label |= (y >= vloc0 && y < vloc0 + Cfg::WM);
     }
