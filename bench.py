@@ -25,8 +25,8 @@ PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
 # cannot be read from inside this process.
 MEASURED_TRAFFIC = {
     "qwen2.5-7b-head-T16384": {
-        "lce_bwd_chunk_kernel": 8791985 * 1024 * 2.0 + 1380495 * 1024 * 1.0,
-        "lce_fwd_kernel": 13577739 * 1024 * 2.0 + 7160 * 1024 * 1.0,
+        "lce_bwd_chunk_kernel": 8927984 * 1024 * 2.0 + 1379224 * 1024 * 1.0,
+        "lce_fwd_kernel": 13709236 * 1024 * 2.0 + 7159 * 1024 * 1.0,
     },
     "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 537764 * 1024 * 2.0 + 1024 * 1024 * 1.0},
 }
