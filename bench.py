@@ -42,6 +42,8 @@ WORKLOADS = {
     "llama3-8b-actor-step-T262144": (262144, 4096, 128256, 1.0, 0.02, 64, 256, True),
     # log-prob pass with few tokens: one streaming read of W, HBM-bound
     "qwen2.5-7b-head-T64-fwd": (64, 3584, 152064, 1.0, 0.02, 0, 0, False, True),
+    # the log-prob passes that run under no_grad (old_log_prob, ref_log_prob): forward only at the full token count
+    "qwen2.5-7b-head-T16384-fwd": (16384, 3584, 152064, 1.0, 0.02, 0, 0, False, True),
     "small": (2048, 1024, 32768, 1.0, 0.02, 0, 0, False),
 }
 
@@ -322,9 +324,29 @@ def main():
         if k in executed:
             v["executed_tflops"] = executed[k] * V * H / (v["ms_per_step"] * 1e-3) / 1e12
     if fwd_only:
-        # one pass over W: the HBM roofline bounds it
         k = kernels["lce_fwd_kernel"]
         nbytes = (V * H + T * H) * 2.0
+        flops = 2.0 * T * V * H
+        if flops / nbytes > PEAK_BF16 / PEAK_HBM:
+            # enough tokens per weight row: the matrix pipe bounds it
+            out = {
+                "metric": "tokens/s, forward (log-prob + entropy); % of bf16 MFMA peak",
+                "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                "ms_per_step": ms_per_step, "step_ms": step_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                "dtype": "bf16", "data": "synthetic",
+                "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
+                "algorithmic_tflops": flops / (elapsed / args.steps) / 1e12,
+                "frac_of_bf16_peak": flops / (elapsed / args.steps) / PEAK_BF16,
+                "roofline": {"bound": "mfma", "kernel": "lce_fwd_kernel", "achieved": flops / (k["avg_ms"] * 1e-3) / 1e12,
+                             "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flops / (k["avg_ms"] * 1e-3) / PEAK_BF16,
+                             "traffic": MEASURED_TRAFFIC.get("qwen2.5-7b-head-T16384", {}).get("lce_fwd_kernel") if T == 16384 else None,
+                             "avg_launch_ms": k["avg_ms"], "flops_per_launch": flops},
+                "kernels": kernels,
+                "cpu_baseline": None,
+            }
+            print(json.dumps(out), flush=True)
+            return
+        # one pass over W: the HBM roofline bounds it
         out = {
             "metric": "tokens/s, forward (log-prob + entropy) with few tokens; % of HBM peak",
             "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
