@@ -928,7 +928,7 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
   hipLaunchKernelGGL(ppo_finish_kernel, dim3(1), dim3(256), 0, st, p.partials, rows, p.segs, row_len, g, row_tot,
                      row_weight, out);
   if ((rc = check_launch("ppo_finish_kernel"))) return rc;
-  hipLaunchKernelGGL(ppo_scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g_log_prob, g_entropy, rows, row_len,
+  hipLaunchKernelGGL(ppo_scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g_log_prob, g_entropy, row_len,
                      p.segs, p.seg_len, row_weight);
   return check_launch("ppo_scale_kernel");
 }

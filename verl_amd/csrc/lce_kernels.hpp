@@ -1366,7 +1366,7 @@ __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs,
   }
 }
 
-__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t rows, int64_t row_len, int segs, int64_t seg_len,
+__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t row_len, int segs, int64_t seg_len,
                                  const float* row_weight) {
   const int64_t row = (int64_t)blockIdx.x / segs;
   const int64_t c0 = ((int64_t)blockIdx.x % segs) * seg_len;
