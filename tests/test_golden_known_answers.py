@@ -76,3 +76,54 @@ def test_uniform_logits_kernels(case):
     lp = F.logprobs_from_logits(z.float(), torch.tensor([0, V // 2, V - 1], device="cuda:0"))
     assert ent.cpu().tolist() == pytest.approx([float(case["entropy"])] * 3, rel=1e-5)
     assert lp.cpu().tolist() == pytest.approx([float(case["logprob"])] * 3, rel=1e-5)
+
+
+PPO = GOLD["ppo"]
+AGG_MODES = ("token-mean", "token-sum", "seq-mean-token-sum", "seq-mean-token-sum-norm", "seq-mean-token-mean")
+
+
+def _ppo_inputs(device, dtype):
+    t = lambda k: torch.tensor(PPO[k], dtype=dtype, device=device)
+    return t("log_prob"), t("entropy"), t("old_log_prob"), t("advantages"), t("mask"), t("ref_log_prob")
+
+
+def test_ppo_oracle_against_the_known_answers():
+    """Clipped loss per token (every branch: unclipped, clipped above / below, dual clip, the +-20 clamp), the four KL
+    estimators, the five aggregation modes and the masked-mean metrics, evaluated with scalar arithmetic at 40 digits."""
+    lp, ent, old, adv, mask, ref = _ppo_inputs("cpu", torch.float64)
+    for mode in AGG_MODES:
+        pg, met = O.policy_loss_vanilla(old, lp, adv, mask, mode, 0.2, PPO["clip_ratio_low"], PPO["clip_ratio_high"],
+                                        PPO["clip_ratio_c"])  # fmt: skip
+        assert pg.item() == pytest.approx(float(PPO["pg_loss"][mode]), rel=1e-12)
+        assert O.agg_loss(ent, mask, mode).item() == pytest.approx(float(PPO["entropy_loss"][mode]), rel=1e-9)
+        for kl in ("kl", "abs", "mse", "low_var_kl"):
+            got = O.agg_loss(O.kl_penalty(lp, ref, kl), mask, mode).item()
+            assert got == pytest.approx(float(PPO["kl_loss"][kl][mode]), rel=1e-9), (kl, mode)
+    assert met["actor/pg_clipfrac"] == pytest.approx(float(PPO["pg_clipfrac"]), rel=1e-9)
+    assert met["actor/pg_clipfrac_lower"] == pytest.approx(float(PPO["pg_clipfrac_lower"]), rel=1e-9)
+    assert met["actor/ppo_kl"] == pytest.approx(float(PPO["ppo_kl"]), rel=1e-9)
+    for kl in ("kl", "abs", "mse", "low_var_kl"):
+        want = torch.tensor([[float(v) for v in row] for row in PPO["kl"][kl]], dtype=torch.float64)
+        torch.testing.assert_close(O.kl_penalty(lp, ref, kl), want, rtol=1e-12, atol=1e-15)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", AGG_MODES)
+@pytest.mark.parametrize("kl", ["kl", "abs", "mse", "low_var_kl"])
+def test_ppo_kernels_against_the_known_answers(mode, kl):
+    from verl_amd.trainer.ppo.core_algos import agg_loss
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    lp, ent, old, adv, mask, ref = _ppo_inputs("cuda:0", torch.float32)
+    loss, met = fused_ppo_loss(lp, ent, old, adv, mask, clip_ratio_low=PPO["clip_ratio_low"], clip_ratio_high=PPO["clip_ratio_high"],
+                               clip_ratio_c=PPO["clip_ratio_c"], entropy_coeff=0.5, loss_agg_mode=mode, ref_log_prob=ref,
+                               kl_loss_type=kl, kl_loss_coef=0.25)  # fmt: skip
+    pg, el, kll = float(PPO["pg_loss"][mode]), float(PPO["entropy_loss"][mode]), float(PPO["kl_loss"][kl][mode])
+    assert met["actor/pg_loss"].item() == pytest.approx(pg, rel=2e-6)
+    assert met["actor/entropy_loss"].item() == pytest.approx(el, rel=2e-6)
+    assert met["kl_loss"].item() == pytest.approx(kll, rel=2e-6)
+    assert loss.item() == pytest.approx(pg - 0.5 * el + 0.25 * kll, rel=2e-6, abs=1e-6)
+    assert met["actor/pg_clipfrac"].item() == pytest.approx(float(PPO["pg_clipfrac"]), rel=1e-6)
+    assert met["actor/pg_clipfrac_lower"].item() == pytest.approx(float(PPO["pg_clipfrac_lower"]), rel=1e-6)
+    assert met["actor/ppo_kl"].item() == pytest.approx(float(PPO["ppo_kl"]), rel=1e-6)
+    assert agg_loss(ent, mask, mode).item() == pytest.approx(el, rel=2e-6)
