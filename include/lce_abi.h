@@ -167,6 +167,8 @@ int lce_num_variants(void);
  * LCE_OPT_DW_TRANSPOSED_READS (default 1, bf16 only): the d_weight GEMM reads the token-major d_logits with
  * transposing LDS reads; 0 builds a second, vocab-major copy of the d_logits for it (changes the workspace size:
  * set it before querying lce_backward_workspace_bytes).
+ * LCE_OPT_DLOGITS_FEW_TOKEN_TILES (default 1, 16-bit inputs): with at most 128 tokens the d_logits tiles of the backward
+ * use the narrow token tiles and deep LDS ring of the few-token forward; 0 = the backward's own 256 x 256 tiles.
  * LCE_OPT_LABEL_TERM_OUTSIDE (default 2, 16-bit inputs only): 1 = the one-hot part g_logprob / temperature * 1[v == label]
  * of the gradient of the logits is added to d_hidden and to the label rows of d_weight in fp32 instead of being rounded
  * to 16 bits with the rest of the d_logits tile; 2 = the label's whole entry of d_logits (one-hot and softmax part,
@@ -177,7 +179,8 @@ enum {
   LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
   LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
   LCE_OPT_DW_TRANSPOSED_READS = 3,
-  LCE_OPT_LABEL_TERM_OUTSIDE = 4
+  LCE_OPT_LABEL_TERM_OUTSIDE = 4,
+  LCE_OPT_DLOGITS_FEW_TOKEN_TILES = 5
 };
 int lce_set_option(int key, int64_t value);
 

@@ -29,6 +29,7 @@ int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
 bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
 int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
 int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
+int g_ds_few_tokens = 1;     // d_logits tiles of a backward with at most 128 tokens: narrow token tiles, deeper ring
 int g_label_outside = 2;  // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
 int g_dw_transposed_reads = 1;  // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
 
@@ -320,6 +321,19 @@ BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk
   return bwd_layout_for(T, H, V, esz, vchunk, gt, gv);
 }
 
+// The d_logits tiles of a backward with few tokens stream W once, like the forward with few tokens, and gain from
+// the same narrow token tiles with a deeper ring.  SmallCfg must permute the vocabulary inside a wave tile as Cfg
+// does (same WM), because the gradient GEMMs that read dS run with Cfg.
+template <typename SmallCfg, typename Cfg>
+int launch_ds_few_tokens(DsArgs<typename Cfg::TIN> d, int64_t T, int nvt, hipStream_t st) {
+  static_assert(SmallCfg::WM == Cfg::WM && SmallCfg::FM == Cfg::FM && SmallCfg::BM == Cfg::BM, "same vocabulary order in dS");
+  const int ntt = (int)((T + SmallCfg::BN - 1) / SmallCfg::BN);
+  d.map = TileMap::make(ntt, nvt, block_rows(ntt), 0);
+  allow_lds(lce_bwd_ds_kernel<SmallCfg>, SmallCfg::LDS_BYTES);
+  hipLaunchKernelGGL(lce_bwd_ds_kernel<SmallCfg>, dim3(d.map.total), dim3(SmallCfg::NTHREADS), SmallCfg::LDS_BYTES, st, d);
+  return check_launch("lce_bwd_ds_kernel");
+}
+
 template <typename Cfg>
 int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                   int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
@@ -489,6 +503,15 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       continue;
     }
     ProfScope prof(PC_BWD_CHUNK, st);
+    if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
+      if (g_ds_few_tokens && p.n_gw + p.n_gh == 0 && L.tn && T <= 128) {  // the first launch: d_logits tiles only
+        const int nvt = (int)((p.ds.vrows + Cfg::BM - 1) / Cfg::BM);
+        rc = T <= 64 ? launch_ds_few_tokens<typename VariantT64<TIN>::Cfg, Cfg>(p.ds, T, nvt, st)
+                     : launch_ds_few_tokens<typename VariantT128<TIN>::Cfg, Cfg>(p.ds, T, nvt, st);
+        if (rc) return rc;
+        continue;
+      }
+    }
     hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
@@ -607,6 +630,7 @@ int lce_set_option(int key, int64_t value) {
       if (value < 0 || value > 2) return fail(LCE_E_ARG, "LCE_OPT_LABEL_TERM_OUTSIDE takes 0, 1 or 2");
       g_label_outside = (int)value;
       return LCE_OK;
+    case LCE_OPT_DLOGITS_FEW_TOKEN_TILES: g_ds_few_tokens = value != 0; return LCE_OK;
     case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
