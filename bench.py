@@ -21,7 +21,8 @@ if ROOT not in sys.path:
 PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
 # HBM-side bytes per launch (fetch + write) of the MFMA kernels on the default workload, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run
-# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt, profiles/lce_fwd_kernel_qwen2.5-7b-head-T64-fwd.txt); counters
+# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt, profiles/lce_fwd_kernel_qwen2.5-7b-head-T64-fwd.txt,
+# profiles/lce_kernels_qwen2.5-7b-head-T64.txt); counters
 # cannot be read from inside this process.
 MEASURED_TRAFFIC = {
     "qwen2.5-7b-head-T16384": {
@@ -29,6 +30,9 @@ MEASURED_TRAFFIC = {
         "lce_fwd_kernel": 13709236 * 1024 * 2.0 + 7159 * 1024 * 1.0,
     },
     "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 537764 * 1024 * 2.0 + 1024 * 1024 * 1.0},
+    # (average of the backward's two launches: d_logits tiles, then both gradient GEMMs;
+    # profiles/lce_kernels_qwen2.5-7b-head-T64.txt)
+    "qwen2.5-7b-head-T64": {"lce_bwd_chunk_kernel": ((537574 + 625946) * 1024 * 2.0 + (19008 + 1111246) * 1024 * 1.0) / 2},
 }
 WORKLOADS = {
     # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step[, forward only])
@@ -42,6 +46,8 @@ WORKLOADS = {
     "llama3-8b-actor-step-T262144": (262144, 4096, 128256, 1.0, 0.02, 64, 256, True),
     # log-prob pass with few tokens: one streaming read of W, HBM-bound
     "qwen2.5-7b-head-T64-fwd": (64, 3584, 152064, 1.0, 0.02, 0, 0, False, True),
+    # few tokens, forward + backward: every kernel streams W (or writes d_weight) once, HBM-bound
+    "qwen2.5-7b-head-T64": (64, 3584, 152064, 1.0, 0.02, 0, 0, False),
     # the log-prob passes that run under no_grad (old_log_prob, ref_log_prob): forward only at the full token count
     "qwen2.5-7b-head-T16384-fwd": (16384, 3584, 152064, 1.0, 0.02, 0, 0, False, True),
     "small": (2048, 1024, 32768, 1.0, 0.02, 0, 0, False),
@@ -374,6 +380,17 @@ def main():
         "flops_per_launch": flops_per_launch,
     }
     algorithmic = 6.0 * T * V * H / (elapsed / args.steps)
+    if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM:
+        # few tokens: the step is four streaming passes over [V, H] in the input dtype (W read by the forward, by the
+        # d_logits tiles and by the d_hidden GEMM; d_weight written), and HBM bounds it.  The backward's two launches
+        # (d_logits tiles; both gradient GEMMs) account for three of the four.
+        k = kernels["lce_bwd_chunk_kernel"]
+        nbytes = 3.0 * V * H * 2.0 / k["launches_per_step"]
+        roofline = {"bound": "hbm", "kernel": "lce_bwd_chunk_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
+                    "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
+                    "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("lce_bwd_chunk_kernel"),
+                    "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes,
+                    "step_bytes": 4.0 * V * H * 2.0, "step_GBps": 4.0 * V * H * 2.0 / (elapsed / args.steps) / 1e9}
     out = {
         "metric": "fwd+bwd tokens/s, 7B lm-head logprob+entropy; % of bf16 MFMA peak",
         "value": tokens_per_s,
