@@ -180,7 +180,10 @@ enum {
   LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
   LCE_OPT_DW_TRANSPOSED_READS = 3,
   LCE_OPT_LABEL_TERM_OUTSIDE = 4,
-  LCE_OPT_DLOGITS_FEW_TOKEN_TILES = 5
+  LCE_OPT_DLOGITS_FEW_TOKEN_TILES = 5,
+  LCE_OPT_DLOGITS_STRIP = 6,
+  LCE_OPT_DHIDDEN_KSPLIT = 7,
+  LCE_OPT_WORKSPACE_BUDGET = 8
 };
 int lce_set_option(int key, int64_t value);
 

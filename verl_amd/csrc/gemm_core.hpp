@@ -109,6 +109,7 @@ struct Mma<float> {
 template <typename TIN_, int BM_, int BN_, int BKB_, int NSTAGE_, int WAVES_M_, int WAVES_N_, int SPLIT_ = 0, int TRANS_ = 0>
 struct GemmCfg {
   typedef TIN_ TIN;
+  static constexpr bool CORE16 = false;  // (the four-wave 16x16x32 mainloop is GemmCfg16, gemm_core16.hpp)
   static constexpr int BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
   static constexpr int SPLIT = SPLIT_;  // 0 whole stages; 1 split ring, A operand early; 2 split ring, B operand early
   static constexpr int TRANS = TRANS_;

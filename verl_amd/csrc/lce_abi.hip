@@ -12,6 +12,7 @@
 
 #include "label_rows.hpp"
 #include "lce_kernels.hpp"
+#include "lce_kernels16.hpp"
 
 using namespace lce;
 
@@ -21,17 +22,39 @@ bool known_dtype(int dtype) { return dtype == LCE_DTYPE_BF16 || dtype == LCE_DTY
 size_t esize(int dtype) { return dtype == LCE_DTYPE_F32 ? 4 : 2; }
 
 thread_local char g_err[512] = "";
-// Defaults: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it only up
-// to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed
-// (the XCD's workgroups drift apart and lose L2 sharing), so large forwards keep the 2-stage ring.
-constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2;
-int g_variant_fwd = kDefaultVariantFwd, g_variant_bwd = kDefaultVariantBwd;
-bool g_variant_forced = false;  // lce_set_variant was called: no size-based choice of the forward's tile
-int g_split_bwd = 0;          // diagnostic: launch the three sub-problems of a backward chunk separately
-int g_ds_tokens_first = -1;  // tile order of the d_logits pass; -1: by size
-int g_ds_few_tokens = 1;     // d_logits tiles of a backward with at most 128 tokens: narrow token tiles, deeper ring
-int g_label_outside = 2;  // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
-int g_dw_transposed_reads = 1;  // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
+// Tuning state.  Every entry point takes ONE snapshot of it under the mutex and works from that copy, so a setter
+// running on another thread can never change the workspace layout between a call's own size check and its launches.
+// (A setter between lce_backward_workspace_bytes and lce_backward can still make the two disagree: lce_backward
+// re-derives the size from its own snapshot and returns LCE_E_WORKSPACE instead of overrunning the buffer.)
+// Defaults of the 32x32x16 loops: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it
+// only up to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed (the XCD's
+// workgroups drift apart and lose L2 sharing), so large forwards keep the 2-stage ring.  Beyond 8192 tokens 16-bit
+// inputs run the four-wave 16x16x32 loop (variant 5) in both directions.
+constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2, kVariantCore16 = 5;
+constexpr int64_t kCore16MinTokens = 8192;  // variant 5 is the default above this many tokens
+struct Tuning {
+  int variant_fwd = kDefaultVariantFwd, variant_bwd = kDefaultVariantBwd;
+  bool variant_forced = false;   // lce_set_variant was called: no size-based choice of the tile
+  int split_bwd = 0;             // diagnostic: launch the three sub-problems of a backward chunk separately
+  int ds_tokens_first = -1;      // tile order of the d_logits pass; -1: by size
+  int ds_few_tokens = 1;         // d_logits tiles of a backward with at most 128 tokens: narrow token tiles, deeper ring
+  int label_outside = 2;         // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
+  int dh_ksplit = 0;             // K slices of the d_hidden GEMM; 0: chosen by shape
+  int ds_strip = 1;              // vocabulary tiles per workgroup of the d_logits pass on the 16x16x32 loop
+  int dw_transposed_reads = 1;   // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
+  int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
+};
+std::mutex g_tuning_mu;
+Tuning g_tuning;
+Tuning tuning_snapshot() {
+  std::lock_guard<std::mutex> l(g_tuning_mu);
+  return g_tuning;
+}
+// the mainloop variant a backward over T tokens of `esz`-byte elements runs with
+int bwd_variant(const Tuning& tu, int64_t T, size_t esz) {
+  if (tu.variant_forced) return tu.variant_bwd;
+  return (esz == 2 && T > kCore16MinTokens) ? kVariantCore16 : kDefaultVariantBwd;
+}
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -85,7 +108,10 @@ template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2,
 template <typename TIN> struct VariantT64 { typedef GemmCfg<TIN, 256, 64, 128, 4, 4, 2> Cfg; };
 template <typename TIN> struct VariantT128 { typedef GemmCfg<TIN, 256, 128, 128, 3, 4, 2> Cfg; };
 template <typename TIN> struct Variant4 { typedef GemmCfg<TIN, 256, 128, 128, 3, 2, 2> Cfg; };
-constexpr int kNumVariants = 5;
+// four waves of 128x128 on v_mfma_f32_16x16x32 (16-bit inputs; fp32 inputs run the split-ring 32x32x2 loop instead)
+template <typename TIN> struct Variant5 { typedef GemmCfg16<TIN> Cfg; };
+template <> struct Variant5<float> { typedef GemmCfg<float, 256, 256, 128, 5, 4, 2, 2> Cfg; };
+constexpr int kNumVariants = 6;
 
 template <typename K>
 void allow_lds(K kernel, int bytes) {
@@ -118,9 +144,15 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
   if (M <= 0 || N <= 0) return LCE_OK;
   if (K <= 0 || K % Cfg::BK != 0) return fail(LCE_E_ARG, "gemm: K=%lld must be a positive multiple of %d", (long long)K, Cfg::BK);
   const GemmArgs<TIN> p = make_gemm_args<Cfg>(A, lda, B, ldb, M, N, K, Cf, ldcf, Ct, ldct, out_mode);
-  allow_lds(gemm_nt_kernel<Cfg>, Cfg::LDS_BYTES);
   ProfScope prof(prof_cls, st);
-  hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  if constexpr (Cfg::CORE16) {
+    if (N % 4 != 0) return fail(LCE_E_ARG, "gemm: N=%lld must be a multiple of 4", (long long)N);
+    allow_lds(gemm16_nt_kernel<Cfg>, Cfg::LDS_BYTES);
+    hipLaunchKernelGGL(gemm16_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  } else {
+    allow_lds(gemm_nt_kernel<Cfg>, Cfg::LDS_BYTES);
+    hipLaunchKernelGGL(gemm_nt_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+  }
   return check_launch("gemm_nt_kernel");
 }
 
@@ -161,13 +193,18 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.label_offset = label_offset;
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
-  allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
   int rc;
   hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((T + 1023) / 1024)), dim3(256), 0, st, reinterpret_cast<uint32_t*>(p.xlabel), T);
   if ((rc = check_launch("fill_zero_kernel"))) return rc;
   {
     ProfScope prof(PC_FWD, st);
-    hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    if constexpr (Cfg::CORE16) {
+      allow_lds(lce_fwd16_kernel<Cfg>, Cfg::LDS_BYTES);
+      hipLaunchKernelGGL(lce_fwd16_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    } else {
+      allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
+      hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+    }
     rc = check_launch("lce_fwd_kernel");
   }
   if (rc) return rc;
@@ -221,7 +258,7 @@ int forward_splits_upper_bound(int64_t T) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_coef, off_keys[2], off_vals[2], off_hist, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_coef, off_keys[2], off_vals[2], off_hist, off_tokc, off_tokl, total;
   int sort_items, sort_passes;  // label sort (0 items: the one-hot part stays inside the d_logits tiles)
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
@@ -233,7 +270,7 @@ struct BwdLayout {
 // The d_weight GEMM can take the token-major d_logits and hidden as they are (transposing LDS reads exist
 // for 16-bit elements and are wired for the 8-wave 256 x 256 tile variants 1-3); otherwise a vocab-major copy of the
 // d_logits and a transposed hidden are built for it.
-bool dw_transposed_reads(size_t esz) { return esz == 2 && g_dw_transposed_reads && g_variant_bwd >= 1 && g_variant_bwd <= 3; }
+bool dw_transposed_reads(const Tuning& tu, int variant, size_t esz) { return esz == 2 && ((tu.dw_transposed_reads && variant >= 1 && variant <= 3) || variant == kVariantCore16); }
 
 // The d_hidden GEMM has only ceil(T/256) * ceil(H/256) output tiles, each with a K loop as long as the
 // vocabulary chunk.  With few tokens one such tile takes longer than a CU's share of the whole launch
@@ -248,18 +285,19 @@ int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
 }
 
 // layout for a given chunk width
-BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
+BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
   BwdLayout L;
-  L.tn = dw_transposed_reads(esz);
+  const int variant = bwd_variant(tu, T, esz);
+  L.tn = dw_transposed_reads(tu, variant, esz);
   // Measured: reading W through the transposing LDS reads costs the d_hidden GEMM about 2% of its rate, and
   // saves one transpose of W per call.  The transpose is the larger cost up to some thousands of tokens
   // (T=64: 1.95 -> 1.43 ms per forward + backward, T=4096: 15.7 -> 14.7 ms at H=3584, V=152064), the GEMM
   // rate beyond that (T=16384: +0.5 ms).
-  L.tn_dh = L.tn && T <= 8192;
+  L.tn_dh = L.tn && T <= 8192 && variant != kVariantCore16;  // (the 16x16x32 loop has no mixed mode: it always takes W^T)
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
-  L.ksplit = dh_ksplit(T, H, vchunk);
+  L.ksplit = tu.dh_ksplit > 0 ? tu.dh_ksplit : dh_ksplit(T, H, vchunk);
   L.nchunks = (int)((V + vchunk - 1) / vchunk);
   // Row strides are kept away from large powers of two (+128 bytes): with a 16 or 32 KiB stride the
   // 256 rows of an operand tile would all fall into the same L2 channel.
@@ -288,7 +326,7 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   L.off_inv = o;   o += align256((size_t)T * 4);
   L.off_nrows = o; o += 256;
   // (label row, token) pairs, two buffers each, and the per-block digit counts of one radix pass
-  L.sort_items = (esz == 2 && g_label_outside && T <= ((int64_t)1 << 30)) ? (int)round_up(T, kSortBlock) : 0;
+  L.sort_items = (esz == 2 && tu.label_outside && T <= ((int64_t)1 << 30)) ? (int)round_up(T, kSortBlock) : 0;
   int vbits = 1;
   while (vbits < 32 && ((int64_t)1 << vbits) < V) ++vbits;
   L.sort_passes = (vbits + 1 + 7) / 8;
@@ -298,7 +336,10 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
   }
   L.off_hist = o;  o += align256((size_t)(L.sort_items / kSortBlock) * 256 * 4);
   // per-token coefficient of the label's entry of d_logits, when the whole entry is kept out of the tiles
-  L.off_coef = o;  o += (L.sort_items && g_label_outside == 2) ? align256((size_t)T * 4) : 0;
+  L.off_coef = o;  o += (L.sort_items && tu.label_outside == 2) ? align256((size_t)T * 4) : 0;
+  // per-position constants of the d_logits tiles (16-bit inputs): 16 + 4 bytes per position
+  L.off_tokc = o;  o += esz == 2 ? align256((size_t)L.tpad * 16) : 0;
+  L.off_tokl = o;  o += esz == 2 ? align256((size_t)L.tpad * 4) : 0;
   L.total = o;
   return L;
 }
@@ -310,15 +351,16 @@ BwdLayout bwd_layout_for(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vc
 // then evened out over the number of chunks that width needs.
 // gt, gv: K-permutation groups that tokens / vocabulary are rounded up to (at most one workgroup
 // tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
-BwdLayout bwd_layout(int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
+BwdLayout bwd_layout(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
-    const double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
+    double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
+    if (tu.ws_budget > 0 && (double)tu.ws_budget < gate) gate = (double)tu.ws_budget;
     vchunk = round_up(V, 256);
-    while (vchunk > 2048 && (double)bwd_layout_for(T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
+    while (vchunk > 2048 && (double)bwd_layout_for(tu, T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
     const int64_t n = (V + vchunk - 1) / vchunk;
     vchunk = round_up((V + n - 1) / n, 256);
   }
-  return bwd_layout_for(T, H, V, esz, vchunk, gt, gv);
+  return bwd_layout_for(tu, T, H, V, esz, vchunk, gt, gv);
 }
 
 // The d_logits tiles of a backward with few tokens stream W once, like the forward with few tokens, and gain from
@@ -339,10 +381,10 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                   int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
                   const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                   typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st,
-                  int64_t vocab_offset = 0) {
+                  int64_t vocab_offset, const Tuning& tu) {
   // vocab_offset: W is the shard [vocab_offset, vocab_offset + V) of a larger vocabulary (labels are global ids)
   typedef typename Cfg::TIN TIN;
-  const BwdLayout L = bwd_layout(T, H, V, sizeof(TIN), vchunk, KPerm<Cfg>::GT, KPerm<Cfg>::GV);
+  const BwdLayout L = bwd_layout(tu, T, H, V, sizeof(TIN), vchunk, KPerm<Cfg>::GT, KPerm<Cfg>::GV);
   TIN* dS[2] = {reinterpret_cast<TIN*>(ws + L.off_dS[0]), reinterpret_cast<TIN*>(ws + L.off_dS[1])};
   TIN* dST[2] = {reinterpret_cast<TIN*>(ws + L.off_dST[0]), reinterpret_cast<TIN*>(ws + L.off_dST[1])};
   TIN* Wt = reinterpret_cast<TIN*>(ws + L.off_Wt);
@@ -373,7 +415,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   if (L.sort_items) {
     lt.labels = labels;
     ProfScope prof(PC_LABEL_ROWS, st);
-    if constexpr (sizeof(TIN) == 2) if (g_label_outside == 2) {
+    if constexpr (sizeof(TIN) == 2) if (tu.label_outside == 2) {
       float* coef = reinterpret_cast<float*>(ws + L.off_coef);
       hipLaunchKernelGGL(label_coef_kernel<TIN>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, h, ldh, W, ldw, labels, vocab_offset, V, T,
                          H, maximum, accumulate, entropy_b, dlogprobs, lt.g_stride, reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f,
@@ -400,6 +442,17 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       }
     }
   }
+  f32x4_t* tokc = nullptr;
+  int* tokl = nullptr;
+  if constexpr (Cfg::CORE16) {
+    tokc = reinterpret_cast<f32x4_t*>(ws + L.off_tokc);
+    tokl = reinterpret_cast<int*>(ws + L.off_tokl);
+    ProfScope prof(PC_ACTIVE_ROWS, st);
+    hipLaunchKernelGGL(ds_token_consts_kernel, dim3((unsigned)((L.tpad + 255) / 256)), dim3(256), 0, st, rows, n_rows, T, L.tpad, dlogprobs,
+                       (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f,
+                       dentropy, maximum, accumulate, entropy_b, labels, vocab_offset, V, 1.0f / temperature, tokc, tokl);
+    if ((rc = check_launch("ds_token_consts_kernel"))) return rc;
+  }
   // second operand of the d_weight GEMM (W^T for d_hidden follows chunk by chunk): the listed rows of hidden,
   // as they are (K-major, for the transposing reads), or transposed to h^T [H][T]
   if (L.tn) {
@@ -416,7 +469,15 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   const int ntt = (int)((T + Cfg::BN - 1) / Cfg::BN);
   // (the K-major d_weight tiles use the 160 KB split ring whatever ring the variant itself uses)
   const int chunk_lds = L.tn && Cfg::LDS_BYTES < 160 * 1024 ? 160 * 1024 : Cfg::LDS_BYTES;
-  allow_lds(lce_bwd_chunk_kernel<Cfg>, chunk_lds);
+  auto launch_chunk = [&](const BwdChunkArgs<TIN>& q) {
+    if constexpr (Cfg::CORE16) {
+      allow_lds(lce_bwd_chunk16_kernel<Cfg>, chunk_lds);
+      hipLaunchKernelGGL(lce_bwd_chunk16_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, q);
+    } else {
+      allow_lds(lce_bwd_chunk_kernel<Cfg>, chunk_lds);
+      hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, q);
+    }
+  };
   // launch c (0 <= c <= nchunks): d_logits of chunk c (if any) + the two gradient GEMMs of chunk c-1 (if any)
   for (int c = 0; c <= L.nchunks; ++c) {
     BwdChunkArgs<TIN> p;
@@ -434,13 +495,19 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.g_ent = dentropy;
       d.dS = dS[c & 1]; d.ldS = L.ldS; d.dST = L.tn ? nullptr : dST[c & 1]; d.ldST = L.ldST; d.tpad = L.tpad;
       d.rows = rows; d.n_rows = n_rows;
-      d.label_outside = lt.labels != nullptr ? g_label_outside : 0;
-      const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
+      d.label_outside = lt.labels != nullptr ? tu.label_outside : 0;
+      d.tokc = tokc; d.tokl = tokl; d.lab0 = v0;
+      d.strip = Cfg::CORE16 ? tu.ds_strip : 1;
+      if (Cfg::CORE16 && L.tn) {
+        // the compact copy of hidden built for the d_weight GEMM: the tiles read it without a row gather
+        d.h = Ht; d.ldh = L.ldHt; d.rows = nullptr;
+      }
+      const int nvt = ((int)((vrows + Cfg::BM - 1) / Cfg::BM) + d.strip - 1) / d.strip;  // columns of the map: strips of tiles
       // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
       // faster on the launch while `hidden` is small enough to stay in the memory-side cache next to the
       // chunk's other operands (T=16384, H=3584: 117 MB), along the tokens is 2% faster beyond that
       // (T=32768, H=4096 and T=65536, H=5120).
-      const int tokens_first = g_ds_tokens_first >= 0 ? g_ds_tokens_first : ((size_t)T * H * sizeof(TIN) > ((size_t)128 << 20));
+      const int tokens_first = tu.ds_tokens_first >= 0 ? tu.ds_tokens_first : ((size_t)T * H * sizeof(TIN) > ((size_t)128 << 20));
       d.map = TileMap::make(ntt, nvt, block_rows(ntt), tokens_first);
       p.n_ds = d.map.total;
     }
@@ -488,7 +555,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         swapped = true;
       }
     }
-    if (g_split_bwd) {
+    if (tu.split_bwd) {
       const int n[3] = {p.n_gw, p.n_gh, p.n_ds};
       const int cls[3] = {swapped ? PC_GEMM_DH : PC_GEMM_DW, swapped ? PC_GEMM_DW : PC_GEMM_DH, PC_BWD_DS};
       for (int k = 0; k < 3; ++k) {
@@ -497,14 +564,14 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         if (k == 1) q.gw = p.gh;  // sub-problem k is moved to the front slot of a single-problem launch
         if (k == 2) { q.n_gw = 0; q.n_gh = 0; } else { q.n_gw = n[k]; q.n_gh = 0; q.n_ds = 0; }
         ProfScope prof(cls[k], st);
-        hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(q.n_gw + q.n_gh + q.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, q);
+        launch_chunk(q);
         if ((rc = check_launch("lce_bwd_chunk_kernel(split)"))) return rc;
       }
       continue;
     }
     ProfScope prof(PC_BWD_CHUNK, st);
     if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
-      if (g_ds_few_tokens && p.n_gw + p.n_gh == 0 && L.tn && T <= 128) {  // the first launch: d_logits tiles only
+      if (tu.ds_few_tokens && p.n_gw + p.n_gh == 0 && L.tn && T <= 128) {  // the first launch: d_logits tiles only
         const int nvt = (int)((p.ds.vrows + Cfg::BM - 1) / Cfg::BM);
         rc = T <= 64 ? launch_ds_few_tokens<typename VariantT64<TIN>::Cfg, Cfg>(p.ds, T, nvt, st)
                      : launch_ds_few_tokens<typename VariantT128<TIN>::Cfg, Cfg>(p.ds, T, nvt, st);
@@ -512,7 +579,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         continue;
       }
     }
-    hipLaunchKernelGGL(lce_bwd_chunk_kernel<Cfg>, dim3(p.n_gw + p.n_gh + p.n_ds), dim3(Cfg::NTHREADS), chunk_lds, st, p);
+    launch_chunk(p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
   {
@@ -554,17 +621,17 @@ template <template <typename> class Vt>
 int dispatch_dtype_backward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
                             int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* mx,
                             const float* ac, const float* eb, const float* glp, const float* gent, void* dh, void* dw,
-                            char* ws, int64_t vchunk, hipStream_t st, int64_t vocab_offset = 0) {
+                            char* ws, int64_t vchunk, hipStream_t st, int64_t vocab_offset, const Tuning& tu) {
   if (dtype == LCE_DTYPE_BF16)
     return backward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
                                                    reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st,
-                                                   vocab_offset);
+                                                   vocab_offset, tu);
   if (dtype == LCE_DTYPE_F16)
     return backward_impl<typename Vt<f16_t>::Cfg>((const f16_t*)h, ldh, (const f16_t*)W, ldw, labels, T, H, V, temperature,
                                                   reduction, mx, ac, eb, glp, gent, (f16_t*)dh, (f16_t*)dw, ws, vchunk, st,
-                                                  vocab_offset);
+                                                  vocab_offset, tu);
   return backward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
-                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st, vocab_offset);
+                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st, vocab_offset, tu);
 }
 
 template <template <typename> class Vt>
@@ -617,21 +684,36 @@ const char* lce_last_error(void) { return g_err; }
 int lce_num_variants(void) { return kNumVariants; }
 int lce_set_variant(int variant) {
   if (variant < -1 || variant >= kNumVariants) return fail(LCE_E_ARG, "variant %d out of range", variant);
-  g_variant_forced = variant >= 0;
-  g_variant_fwd = variant < 0 ? kDefaultVariantFwd : variant;
-  g_variant_bwd = variant < 0 ? kDefaultVariantBwd : variant;
+  std::lock_guard<std::mutex> l(g_tuning_mu);
+  g_tuning.variant_forced = variant >= 0;
+  g_tuning.variant_fwd = variant < 0 ? kDefaultVariantFwd : variant;
+  g_tuning.variant_bwd = variant < 0 ? kDefaultVariantBwd : variant;
   return LCE_OK;
 }
 int lce_set_option(int key, int64_t value) {
+  std::lock_guard<std::mutex> l(g_tuning_mu);
+  Tuning& t = g_tuning;
   switch (key) {
-    case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: g_split_bwd = value != 0; return LCE_OK;
-    case LCE_OPT_DW_TRANSPOSED_READS: g_dw_transposed_reads = value != 0; return LCE_OK;
+    case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: t.split_bwd = value != 0; return LCE_OK;
+    case LCE_OPT_DW_TRANSPOSED_READS: t.dw_transposed_reads = value != 0; return LCE_OK;
     case LCE_OPT_LABEL_TERM_OUTSIDE:
       if (value < 0 || value > 2) return fail(LCE_E_ARG, "LCE_OPT_LABEL_TERM_OUTSIDE takes 0, 1 or 2");
-      g_label_outside = (int)value;
+      t.label_outside = (int)value;
       return LCE_OK;
-    case LCE_OPT_DLOGITS_FEW_TOKEN_TILES: g_ds_few_tokens = value != 0; return LCE_OK;
-    case LCE_OPT_DLOGITS_TOKENS_FIRST: g_ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
+    case LCE_OPT_DLOGITS_FEW_TOKEN_TILES: t.ds_few_tokens = value != 0; return LCE_OK;
+    case LCE_OPT_DLOGITS_TOKENS_FIRST: t.ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
+    case LCE_OPT_DHIDDEN_KSPLIT:
+      if (value < 0 || value > 16) return fail(LCE_E_ARG, "LCE_OPT_DHIDDEN_KSPLIT takes 0..16");
+      t.dh_ksplit = (int)value;
+      return LCE_OK;
+    case LCE_OPT_DLOGITS_STRIP:
+      if (value < 1 || value > 64) return fail(LCE_E_ARG, "LCE_OPT_DLOGITS_STRIP takes 1..64");
+      t.ds_strip = (int)value;
+      return LCE_OK;
+    case LCE_OPT_WORKSPACE_BUDGET:
+      if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_WORKSPACE_BUDGET takes a byte count (0 = the built-in default)");
+      t.ws_budget = value;
+      return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
 }
@@ -691,18 +773,21 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
   char* ws = static_cast<char*>(workspace);
 #define LCE_FWD(Vt) dispatch_dtype_forward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum, accumulate, entropy_b, ws, st, label_offset, shard_out)
-  if (!g_variant_forced && T <= 64) return LCE_FWD(VariantT64);
-  if (!g_variant_forced && T <= 128) return LCE_FWD(VariantT128);
-  if (!g_variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
+  const Tuning tu = tuning_snapshot();
+  if (!tu.variant_forced && T <= 64) return LCE_FWD(VariantT64);
+  if (!tu.variant_forced && T <= 128) return LCE_FWD(VariantT128);
+  if (!tu.variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
+  if (!tu.variant_forced && esize(dtype) == 2 && T > kCore16MinTokens) return LCE_FWD(Variant5);
   // the split ring: measured 4-7% faster than the 2-stage ring up to 8192 tokens, equal (+-1%) beyond, and
   // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
-  if (!g_variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)))
+  if (!tu.variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)))
     return LCE_FWD(Variant2);
-  switch (g_variant_fwd) {
+  switch (tu.variant_fwd) {
     case 1: return LCE_FWD(Variant1);
     case 2: return LCE_FWD(Variant2);
     case 3: return LCE_FWD(Variant3);
     case 4: return LCE_FWD(Variant4);
+    case 5: return LCE_FWD(Variant5);
     default: return LCE_FWD(Variant0);
   }
 #undef LCE_FWD
@@ -757,7 +842,7 @@ int lce_merge_shards(const float* partials, int R, int64_t T, int reduction, flo
 
 size_t lce_backward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype, int64_t vchunk) {
   if (T <= 0 || H <= 0 || V <= 0) return 256;
-  return bwd_layout(T, H, V, esize(dtype), vchunk).total + 256;
+  return bwd_layout(tuning_snapshot(), T, H, V, esize(dtype), vchunk).total + 256;
 }
 
 // shared body of lce_backward and lce_backward_shard
@@ -779,15 +864,17 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
   if (!d_hidden || !maximum || !accumulate || !entropy_b || !dlogprobs) return fail(LCE_E_ARG, "null pointer");
   if (!aligned16(d_hidden) || !aligned16(d_weight)) return fail(LCE_E_ARG, "gradients must be 16-byte aligned");
   if (vchunk < 0) return fail(LCE_E_ARG, "vchunk must be >= 0");
-  if (!workspace || workspace_bytes < lce_backward_workspace_bytes(T, H, V, dtype, vchunk))
-    return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, lce_backward_workspace_bytes(T, H, V, dtype, vchunk));
+  const Tuning tu = tuning_snapshot();
+  const size_t need = bwd_layout(tu, T, H, V, esz, vchunk).total + 256;
+  if (!workspace || workspace_bytes < need) return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, need);
   char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
-#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st, vocab_offset)
-  switch (g_variant_bwd) {
+#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st, vocab_offset, tu)
+  switch (bwd_variant(tu, T, esz)) {
     case 1: return LCE_BWD(Variant1);
     case 2: return LCE_BWD(Variant2);
     case 3: return LCE_BWD(Variant3);
     case 4: return LCE_BWD(Variant4);
+    case 5: return LCE_BWD(Variant5);
     default: return LCE_BWD(Variant0);
   }
 #undef LCE_BWD
@@ -825,6 +912,7 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
     case 2: return LCE_GEMM(Variant2);
     case 3: return LCE_GEMM(Variant3);
     case 4: return LCE_GEMM(Variant4);
+    case 5: return LCE_GEMM(Variant5);
     default: return fail(LCE_E_ARG, "variant %d out of range", variant);
   }
 #undef LCE_GEMM
@@ -838,8 +926,15 @@ int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
   if (lda < round_up(M, 256) || ldb < round_up(N, 256)) return fail(LCE_E_ARG, "gemm_tn: rows must be allocated in whole 256-column tiles");
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   GemmArgs<bf16_t> p = make_gemm_args<Cfg>((const bf16_t*)A, lda, (const bf16_t*)B, ldb, M, N, K, C, ldc, nullptr, 0, 0);
-  allow_lds(gemm_tn_kernel<Cfg>, Cfg::LDS_BYTES);
   ProfScope prof(PC_GEMM_DW, st);
+  if (tuning_snapshot().variant_bwd == kVariantCore16) {  // the same product on the four-wave 16x16x32 loop
+    typedef GemmCfg16<bf16_t> C16;
+    if (N % 4 != 0) return fail(LCE_E_ARG, "gemm_tn: N must be a multiple of 4");
+    allow_lds(gemm16_tn_kernel<C16>, C16::LDS_BYTES);
+    hipLaunchKernelGGL(gemm16_tn_kernel<C16>, dim3(p.map.total), dim3(C16::NTHREADS), C16::LDS_BYTES, st, p);
+    return check_launch("gemm16_tn_kernel");
+  }
+  allow_lds(gemm_tn_kernel<Cfg>, Cfg::LDS_BYTES);
   hipLaunchKernelGGL(gemm_tn_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
   return check_launch("gemm_tn_kernel");
 }

@@ -319,6 +319,14 @@ struct DsArgs {
   int label_outside;  // 1: the tiles hold the softmax terms only; the one-hot part g_lp / tau * 1[v == label] is added
                       // elsewhere in fp32 (label_rows.hpp); 2: the label's whole entry is left out of the tiles (zero
                       // there) and added elsewhere in fp32; 0: everything inside the tiles
+  // Per-position constants prepared once per backward (ds_token_consts_kernel; used by the 16x16x32 tiles):
+  // tokc[k] = (logsumexp * log2 e, C0, C1, G) of the token at compact position k < tpad (positions without a token
+  // hold (1e30, 0, 0, 0), which makes every entry of their rows zero), tokl[k] = its label as a row of this call's
+  // weight or -1; lab0 = the chunk's first row in the same numbering.
+  const f32x4_t* tokc;
+  const int* tokl;
+  int64_t lab0;
+  int strip;  // vocabulary tiles that one workgroup walks (the map's columns are strips)
 };
 
 // The two gradient GEMMs sum over the vocabulary (d_hidden) and over the tokens (d_weight); any
