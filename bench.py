@@ -19,21 +19,34 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16 = 2500e12  # MI355X dense bf16 MFMA peak, FLOP/s
-# HBM-side bytes per launch (fetch + write) of the MFMA kernels on the default workload, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy in the same run
-# (profiles/lce_kernels_qwen2.5-7b-head-T16384.txt, profiles/lce_fwd_kernel_qwen2.5-7b-head-T64-fwd.txt,
-# profiles/lce_kernels_qwen2.5-7b-head-T64.txt); counters
-# cannot be read from inside this process.
-MEASURED_TRAFFIC = {
-    "qwen2.5-7b-head-T16384": {
-        "lce_bwd_chunk_kernel": 8927984 * 1024 * 2.0 + 1379224 * 1024 * 1.0,
-        "lce_fwd_kernel": 13709236 * 1024 * 2.0 + 7159 * 1024 * 1.0,
-    },
-    "qwen2.5-7b-head-T64-fwd": {"lce_fwd_kernel": 537764 * 1024 * 2.0 + 1024 * 1024 * 1.0},
-    # (average of the backward's two launches: d_logits tiles, then both gradient GEMMs;
-    # profiles/lce_kernels_qwen2.5-7b-head-T64.txt)
-    "qwen2.5-7b-head-T64": {"lce_bwd_chunk_kernel": ((537574 + 625946) * 1024 * 2.0 + (19008 + 1111246) * 1024 * 1.0) / 2},
-}
+# HBM-side bytes per launch (fetch + write) of the dominant kernels come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (counters cannot be read from inside this process) and are kept in profiles/traffic.json together with the library state
+# they were measured at; a run whose state differs reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def library_state(lib, T, H, V, flags):
+    """What decides the tiling of a run: ABI version, the workspace sizes the library derives for this shape (they move
+    with the mainloop variant, the chunk width and the layout options) and the tuning flags given on the command line."""
+    return {
+        "abi": int(lib.lce_abi_version()),
+        "forward_workspace_bytes": int(lib.lce_forward_workspace_bytes(T, H, V, 0)),
+        "backward_workspace_bytes": int(lib.lce_backward_workspace_bytes(T, H, V, 0, 0)),
+        "flags": flags,
+    }
+
+
+def measured_traffic(workload, kernel, state):
+    try:
+        table = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return None
+    rec = table.get(workload, {}).get(kernel)
+    if not rec or rec.get("state") != state:
+        return None
+    return rec.get("bytes_per_launch")
+
+
 WORKLOADS = {
     # name: (T, H, V, temperature, weight std, sequences, shortest valid length, PPO loss in the step[, forward only])
     # `sequences` > 0: T is that many equally long rows, each with a valid prefix of U{shortest..row}
@@ -54,10 +67,20 @@ WORKLOADS = {
 }
 
 
+def cpu_model_name() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(seconds_budget: float = 20.0):
     """The oracle's torch restatement (materialised fp32 logits) on the host cores: forward on the
     CPU-runnable reference case (T=1024, H=896, V=151936), bounded to a sample of rows sized so the
-    whole leg takes about `seconds_budget`; reported in tokens/s."""
+    whole leg takes about `seconds_budget`: one warm-up, then the median of five runs; reported in tokens/s."""
     import torch
 
     from oracle import lce_oracle as O
@@ -76,22 +99,27 @@ def cpu_baseline(seconds_budget: float = 20.0):
     y = torch.randint(0, V, (T,), generator=g)
     rows = 128
     t0 = time.perf_counter()
-    O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)  # warm-up, also sizes the sample
+    O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)  # sizes the sample
     dt = time.perf_counter() - t0
-    rows = int(max(128, min(T, rows * (seconds_budget / 3.0) / max(dt, 1e-3))))
+    runs = 5
+    rows = int(max(128, min(T, rows * (seconds_budget / (runs + 1.0)) / max(dt, 1e-3))))
     rows = (rows // 128) * 128
+    O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)  # warm-up at the sample size
     times = []
-    for _ in range(3):
+    for _ in range(runs):
         t0 = time.perf_counter()
         O.lce_forward(h[:rows], w, y[:rows], 1.0, chunk=128)
         times.append(time.perf_counter() - t0)
-    med = sorted(times)[1]
+    med = sorted(times)[runs // 2]
     return {
         "value": rows / med,
         "unit": "tokens/s (forward only, fp32)",
         "cores": cores,
+        "torch_num_threads": torch.get_num_threads(),
+        "cpu_model": cpu_model_name(),
         "kind": "port",
-        "sample": f"oracle torch restatement, forward, first {rows} of T=1024 rows, H=896, V=151936, fp32, median of 3",
+        "sample": f"oracle torch restatement, forward, first {rows} of T=1024 rows, H=896, V=151936, fp32, 1 warm-up + median of {runs}",
+        "runs_s": [round(t, 4) for t in times],
         "gflops": 2.0 * rows * H * V / med / 1e9,
     }
 
@@ -101,6 +129,8 @@ PEAK_HBM = 8e12  # MI355X HBM3E peak, bytes/s
 LOGITS_WORKLOADS = {
     # name: (rows, vocabulary): logits that already exist in HBM, bf16
     "logits-twins-R8192-V152064": (8192, 152064),
+    # the same through logprobs_and_entropy_from_logits: one forward pass, one backward pass, one d_logits
+    "logits-twins-combined-R8192-V152064": (8192, 152064, True),
 }
 
 
@@ -114,7 +144,8 @@ def run_logits_workload(args, name):
 
     lib = _abi.load()
     dev = torch.device("cuda:0")
-    R, V = LOGITS_WORKLOADS[name]
+    R, V = LOGITS_WORKLOADS[name][:2]
+    combined = len(LOGITS_WORKLOADS[name]) > 2 and LOGITS_WORKLOADS[name][2]
     g = torch.Generator(device=dev).manual_seed(1234 + 6)
     z = (torch.randn(R, V, device=dev, generator=g) * 3).bfloat16().requires_grad_(True)
     y = torch.randint(0, V, (R,), device=dev, generator=g)
@@ -123,8 +154,11 @@ def run_logits_workload(args, name):
 
     def step():
         z.grad = None
-        lp = F.logprobs_from_logits(z, y)
-        ent = F.entropy_from_logits(z)
+        if combined:
+            lp, ent = F.logprobs_and_entropy_from_logits(z, y)
+        else:
+            lp = F.logprobs_from_logits(z, y)
+            ent = F.entropy_from_logits(z)
         torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
     for _ in range(args.warmup):
@@ -164,7 +198,7 @@ def run_logits_workload(args, name):
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": name, "R": R, "V": V, "pass": "2 x fwd + 2 x bwd (+ torch's accumulation of the two d_logits)"},
+        "config": {"workload": name, "R": R, "V": V, "pass": "1 x fwd + 1 x bwd (one autograd node)" if combined else "2 x fwd + 2 x bwd (+ torch's accumulation of the two d_logits)"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM, "traffic": None, "avg_launch_ms": kernels[dom]["avg_ms"],
                      "bytes_per_launch": bytes_per_launch[dom]},
@@ -187,6 +221,7 @@ def main():
     ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
     ap.add_argument("--no-transposed-reads", action="store_true", help="diagnostic: d_weight GEMM from a vocab-major copy of the d_logits")
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE", help="diagnostic: lce_set_option(KEY, VALUE)")
+    ap.add_argument("--print-state", action="store_true", help="print the library state that keys profiles/traffic.json and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -218,6 +253,12 @@ def main():
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
     T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload][:8]
+    flags = {"variant": args.variant, "vchunk": args.vchunk, "split_backward": bool(args.split_backward),
+             "options": sorted(args.option + (["3=0"] if args.no_transposed_reads else []) + (["2=1"] if args.dlogits_tokens_first else []))}
+    state = library_state(lib, T, H, V, flags)
+    if args.print_state:
+        print(json.dumps({"workload": args.workload, "state": state}), flush=True)
+        return
     fwd_only = len(WORKLOADS[args.workload]) > 8 and WORKLOADS[args.workload][8]
     g = torch.Generator(device=dev).manual_seed(1234 + 2)
     h = torch.randn(T, H, device=dev, generator=g).bfloat16().requires_grad_(True)
@@ -345,7 +386,7 @@ def main():
                 "frac_of_bf16_peak": flops / (elapsed / args.steps) / PEAK_BF16,
                 "roofline": {"bound": "mfma", "kernel": "lce_fwd_kernel", "achieved": flops / (k["avg_ms"] * 1e-3) / 1e12,
                              "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flops / (k["avg_ms"] * 1e-3) / PEAK_BF16,
-                             "traffic": MEASURED_TRAFFIC.get("qwen2.5-7b-head-T16384", {}).get("lce_fwd_kernel") if T == 16384 else None,
+                             "traffic": measured_traffic(args.workload, "lce_fwd_kernel", state),
                              "avg_launch_ms": k["avg_ms"], "flops_per_launch": flops},
                 "kernels": kernels,
                 "cpu_baseline": None,
@@ -361,7 +402,7 @@ def main():
             "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
             "roofline": {"bound": "hbm", "kernel": "lce_fwd_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                          "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
-                         "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("lce_fwd_kernel"),
+                         "traffic": measured_traffic(args.workload, "lce_fwd_kernel", state),
                          "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes},
             "kernels": kernels,
             "cpu_baseline": None,
@@ -375,11 +416,13 @@ def main():
         "peak": PEAK_BF16 / 1e12,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16,
-        "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(dom),
+        "traffic": measured_traffic(args.workload, dom, state),
         "avg_launch_ms": mfma[dom]["avg_ms"],
         "flops_per_launch": flops_per_launch,
     }
-    algorithmic = 6.0 * T * V * H / (elapsed / args.steps)
+    # Algorithmic FLOPs of the step: forward 2*T*V*H, backward 4*Ta*V*H over the Ta tokens that carry an upstream gradient
+    # (the mandated recompute of the logits is executed but not counted).  With Ta = T this is the reference's 6*T*V*H.
+    algorithmic = (2.0 * T + 4.0 * t_active) * V * H / (elapsed / args.steps)
     if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM:
         # few tokens: the step is four streaming passes over [V, H] in the input dtype (W read by the forward, by the
         # d_logits tiles and by the d_hidden GEMM; d_weight written), and HBM bounds it.  The backward's two launches
@@ -388,7 +431,7 @@ def main():
         nbytes = 3.0 * V * H * 2.0 / k["launches_per_step"]
         roofline = {"bound": "hbm", "kernel": "lce_bwd_chunk_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                     "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
-                    "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("lce_bwd_chunk_kernel"),
+                    "traffic": measured_traffic(args.workload, "lce_bwd_chunk_kernel", state),
                     "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes,
                     "step_bytes": 4.0 * V * H * 2.0, "step_GBps": 4.0 * V * H * 2.0 / (elapsed / args.steps) / 1e9}
     out = {
@@ -408,8 +451,12 @@ def main():
         "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau,
                    "pass": "fwd+ppo_loss+bwd" if ppo else "fwd+bwd", "tokens_with_gradient": t_active},
         "memory": memory,
-        "algorithmic_tflops": algorithmic / 1e12,  # 6*T*V*H per step, the reference's accounting per token
+        "algorithmic_tflops": algorithmic / 1e12,
         "frac_of_bf16_peak": algorithmic / PEAK_BF16,
+        # tokens without upstream gradient are skipped by the backward: `value` counts them (they are part of the batch),
+        # the FLOP figures above do not; 6*T*V*H per step over every token is given separately and is NOT a fraction of peak
+        "row_skip": t_active < T,
+        "per_token_accounting_tflops": 6.0 * T * V * H / (elapsed / args.steps) / 1e12,
         # what the kernels execute: forward on T tokens, recompute + two GEMMs on the tokens with gradient
         "executed_tflops": (2.0 * T + 6.0 * t_active) * V * H / (elapsed / args.steps) / 1e12,
         "roofline": roofline,

@@ -150,3 +150,15 @@ def test_process_group_of_one_rank_is_the_single_gpu_path():
     finally:
         if created:
             dist.destroy_process_group()
+
+
+def test_logits_twins_name_the_gpu_only_precondition():
+    """The reference's twins run on any device (its own CPU tests call them); these are HIP kernels without a fallback
+    and say so with a named error instead of a bare assert."""
+    from verl_amd.utils import torch_functional as F
+
+    z = torch.zeros(2, 8)
+    for call in (lambda: F.entropy_from_logits(z), lambda: F.logprobs_from_logits(z, torch.zeros(2, dtype=torch.long)),
+                 lambda: F.calculate_sum_pi_squared_from_logits(z)):
+        with pytest.raises(_abi.LceError, match="GPU tensors only"):
+            call()

@@ -687,3 +687,28 @@ def test_extreme_logits_closed_forms(dtype):
         i = int(excess.argmax())
         assert excess.max() <= 0, (name, i // H, i % H, got.reshape(-1)[i].item(), want.reshape(-1)[i].item(),
                                    bound.reshape(-1)[i].item())
+
+
+def test_every_backward_method_runs_and_split_dlogits_m_raises():
+    """set_backward_method (verl/utils/kernel/kernels.py:146-180): every BackwardEnum value the reference implements
+    gives the oracle's gradients here (they all select the one HIP schedule); _Split_Dlogits_M raises
+    NotImplementedError in the backward, as in the reference (:1726-1727)."""
+    from verl_amd.utils.kernel import kernels
+
+    T, H, V, tau = 513, 256, 2049, 0.9
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=21)
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    try:
+        for method in (kernels.BackwardEnum._Total_Fuse_MN, kernels.BackwardEnum._Total_Separate, kernels.BackwardEnum._Split_Dlogits_N):
+            kernels.set_backward_method(method)
+            assert kernels._config._backward == method
+            _, _, dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+            torch.testing.assert_close(dh.float(), rdh, atol=2e-2, rtol=4e-2)
+            torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
+            assert_bf16_bar(dh, rdh)
+            assert_bf16_bar(dw, rdw)
+        kernels.set_backward_method(kernels.BackwardEnum._Split_Dlogits_M)
+        with pytest.raises(NotImplementedError, match="_Split_Dlogits_M"):
+            _run(h, w, y, tau, g_lp, g_ent)
+    finally:
+        kernels.set_backward_method(kernels.BackwardEnum._Split_Dlogits_N)

@@ -159,3 +159,57 @@ def test_sum_pi_squared_at_the_reference_tests_cases(shape):
     torch.testing.assert_close(got.double(), want, atol=1e-5, rtol=1e-5)
     with pytest.raises(NotImplementedError):  # fp64 logits: the kernels take bf16, fp16 and fp32
         F.calculate_sum_pi_squared_from_logits(big.double())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_autograd_path_saves_the_row_statistics(dtype):
+    """Through autograd the forward must hand its row statistics to the backward (one pass instead of two): the
+    decision is taken from ctx.needs_input_grad, because grad mode is off inside autograd.Function.forward."""
+    from verl_amd.utils import torch_functional as F
+
+    R, V = 37, 4099
+    g = torch.Generator().manual_seed(3)
+    z = (torch.randn(R, V, generator=g) * 2).to(dtype).to(DEV).requires_grad_(True)
+    y = torch.randint(0, V, (R,), generator=g).to(DEV)
+    g_lp = torch.randn(R, generator=g).to(DEV)
+    lp = F.logprobs_from_logits(z, y)
+    saved = lp.grad_fn.saved_tensors
+    assert len(saved) == 3 and saved[2] is not None and saved[2].shape == (R, 2)
+    lp.backward(g_lp.to(lp.dtype))
+    want = O.logits_backward(z.detach(), y, g_lp.to(lp.dtype).float(), torch.zeros(R, device=DEV))
+    tol = dict(atol=1e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(z.grad.float(), want, **tol)
+    with torch.no_grad():
+        assert F.logprobs_from_logits(z, y).grad_fn is None
+    ent = F.entropy_from_logits(z)
+    assert ent.grad_fn.saved_tensors[1] is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(5, 7, 1000), (64, 152064), (3, 33)])
+def test_combined_twin_one_pass_one_gradient(dtype, shape):
+    """logprobs_and_entropy_from_logits: the values of the two twins, and a backward that writes the gradient of the
+    logits once (checked against the oracle's closed form, which is also what the two separate nodes add up to)."""
+    from verl_amd.utils import torch_functional as F
+
+    V = shape[-1]
+    g = torch.Generator().manual_seed(V)
+    z = (torch.randn(*shape, generator=g) * 2).to(dtype).to(DEV)
+    y = torch.randint(0, V, shape[:-1], generator=g).to(DEV)
+    g_lp = torch.randn(*shape[:-1], generator=g).to(DEV)
+    g_ent = torch.randn(*shape[:-1], generator=g).to(DEV)
+    z1 = z.clone().requires_grad_(True)
+    lp, ent = F.logprobs_and_entropy_from_logits(z1, y)
+    assert lp.shape == shape[:-1] and ent.shape == shape[:-1] and lp.dtype == dtype and ent.dtype == dtype
+    assert torch.equal(lp, F.logprobs_from_logits(z, y)) and torch.equal(ent, F.entropy_from_logits(z))
+    torch.autograd.backward([lp, ent], [g_lp.to(dtype), g_ent.to(dtype)])
+    want = O.logits_backward(z.reshape(-1, V), y.reshape(-1), g_lp.to(dtype).float().reshape(-1), g_ent.to(dtype).float().reshape(-1))
+    tol = dict(atol=1e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(z1.grad.float().reshape(-1, V), want, **tol)
+    # only one of the two upstream gradients
+    z2 = z.clone().requires_grad_(True)
+    lp2, ent2 = F.logprobs_and_entropy_from_logits(z2, y, entropy_dtype=torch.float32)
+    assert ent2.dtype == torch.float32
+    ent2.backward(g_ent)
+    want2 = O.logits_backward(z.reshape(-1, V), y.reshape(-1), torch.zeros_like(g_lp).reshape(-1), g_ent.reshape(-1))
+    torch.testing.assert_close(z2.grad.float().reshape(-1, V), want2, **tol)

@@ -28,8 +28,17 @@ def _as_rows(logits: torch.Tensor):
     return rows, V
 
 
-def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool):
-    assert logits.is_cuda, "verl_amd.utils.torch_functional runs on the GPU only"
+def _require_gpu(logits: torch.Tensor) -> None:
+    """The reference's twins run on any device; these are HIP kernels and there is no eager fallback."""
+    if not logits.is_cuda:
+        raise _abi.LceError(
+            "verl_amd.utils.torch_functional runs on GPU tensors only (hand-written HIP kernels, no CPU or eager "
+            f"fallback); got a tensor on {logits.device}"
+        )
+
+
+def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool, want_stats: bool):
+    _require_gpu(logits)
     code = _abi.dtype_code(logits.dtype)
     rows, V = _as_rows(logits)
     R = rows.shape[0]
@@ -37,7 +46,8 @@ def _logits_forward(logits, labels, want_logprobs: bool, want_entropy: bool):
     lp = torch.empty((R,), device=dev, dtype=torch.float32) if want_logprobs else None
     ent = torch.empty((R,), device=dev, dtype=torch.float32) if want_entropy else None
     # row statistics for the backward (it then needs one pass instead of two)
-    stats = torch.empty((R, 2), device=dev, dtype=torch.float32) if (torch.is_grad_enabled() and logits.requires_grad) else None
+    # (the caller decides: inside autograd.Function.forward grad mode is off, so it cannot be read here)
+    stats = torch.empty((R, 2), device=dev, dtype=torch.float32) if want_stats else None
     y = None
     if want_logprobs:
         y = labels.reshape(-1).to(torch.int64).contiguous()
@@ -71,7 +81,7 @@ def _logits_backward(rows, y, stats, g_lp, g_ent, out_shape, out_dtype):
 class _LogprobsFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels):
-        rows, y, lp, _, stats = _logits_forward(logits, labels, True, False)
+        rows, y, lp, _, stats = _logits_forward(logits, labels, True, False, ctx.needs_input_grad[0])
         ctx.save_for_backward(rows, y, stats)
         ctx.shape, ctx.dtype = logits.shape, logits.dtype
         return lp.reshape(logits.shape[:-1]).to(logits.dtype)
@@ -85,7 +95,7 @@ class _LogprobsFromLogits(torch.autograd.Function):
 class _EntropyFromLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, out_dtype):
-        rows, _, _, ent, stats = _logits_forward(logits, None, False, True)
+        rows, _, _, ent, stats = _logits_forward(logits, None, False, True, ctx.needs_input_grad[0])
         ctx.save_for_backward(rows, stats)
         ctx.shape, ctx.dtype = logits.shape, logits.dtype
         return ent.reshape(logits.shape[:-1]).to(out_dtype)
@@ -94,6 +104,34 @@ class _EntropyFromLogits(torch.autograd.Function):
     def backward(ctx, g):
         rows, stats = ctx.saved_tensors
         return _logits_backward(rows, None, stats, None, g, ctx.shape, ctx.dtype), None
+
+
+class _LogprobsAndEntropyFromLogits(torch.autograd.Function):
+    """Both row reductions from one read of the logits, and ONE gradient of the logits in the backward."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, entropy_dtype):
+        rows, y, lp, ent, stats = _logits_forward(logits, labels, True, True, ctx.needs_input_grad[0])
+        ctx.save_for_backward(rows, y, stats)
+        ctx.shape, ctx.dtype = logits.shape, logits.dtype
+        ctx.set_materialize_grads(False)
+        return lp.reshape(logits.shape[:-1]).to(logits.dtype), ent.reshape(logits.shape[:-1]).to(entropy_dtype)
+
+    @staticmethod
+    def backward(ctx, g_lp, g_ent):
+        rows, y, stats = ctx.saved_tensors
+        if g_lp is None and g_ent is None:
+            return None, None, None
+        return _logits_backward(rows, y if g_lp is not None else None, stats, g_lp, g_ent, ctx.shape, ctx.dtype), None, None
+
+
+def logprobs_and_entropy_from_logits(logits, labels, entropy_dtype=None):
+    """``(logprobs_from_logits(logits, labels), entropy_from_logits(logits))`` from a single pass over the logits, with
+    a backward that writes the gradient of the logits once.  The reference calls the two functions back to back on the
+    same logits (``verl/workers/engine/fsdp/transformer_impl.py:1400-1449``); as two autograd nodes each writes a full
+    ``[rows, V]`` gradient and autograd adds them.  ``entropy_dtype``: dtype of the entropy (default: that of
+    ``logits``; ``torch.float32`` gives what ``entropy_from_logits_with_chunking`` returns)."""
+    return _LogprobsAndEntropyFromLogits.apply(logits, labels, logits.dtype if entropy_dtype is None else entropy_dtype)
 
 
 def logprobs_from_logits(logits, labels, inplace_backward=True):
@@ -131,7 +169,7 @@ def calculate_sum_pi_squared_from_logits(logits: torch.Tensor) -> torch.Tensor:
     shape ``logits.shape[:-1]``, dtype of ``logits``.  One pass over the logits.  The reference calls it on
     the actor's logits while collecting log-probs (no graph); differentiating through it is not wired and
     raises instead of returning a detached value."""
-    assert logits.is_cuda, "verl_amd.utils.torch_functional runs on the GPU only"
+    _require_gpu(logits)
     if torch.is_grad_enabled() and logits.requires_grad:
         raise NotImplementedError("calculate_sum_pi_squared_from_logits has no backward; call it under torch.no_grad()")
     rows, V = _as_rows(logits)
