@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 5
+#define LCE_ABI_VERSION 6
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1, LCE_DTYPE_F16 = 2 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -49,6 +49,18 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
                 int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
                 float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
                 void* stream);
+
+/* The same forward for callers that cannot allocate device memory and have no workspace to hand over (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * partial statistics go to a buffer of LCE_STATIC_SCRATCH_BYTES that is part of the library's own device image (one
+ * copy per GPU, held until the process ends); the call allocates nothing and returns LCE_E_WORKSPACE when
+ * lce_forward_workspace_bytes(T, H, V, dtype) exceeds that size (beyond about 116000 tokens).  All calls on one GPU share the
+ * buffer: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  The first call on
+ * a device looks the buffer's address up, so make one call outside a graph capture before capturing. */
+#define LCE_STATIC_SCRATCH_BYTES (8u << 20)
+int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T, int64_t H,
+                       int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy, float* maximum,
+                       float* accumulate, float* entropy_b, void* stream);
 
 /* Backward.  Replaces efficient_entropy_backward (verl/utils/kernel/kernels.py:1518-1729): its
  * d_logits kernel (:1380-1515) and the two vendor GEMMs per vocab split (:1714-1724).

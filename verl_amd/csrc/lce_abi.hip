@@ -665,6 +665,33 @@ int check_common(const void* hidden, int64_t ldh, const void* weight, int64_t ld
 
 }  // namespace
 
+// Scratch memory of lce_forward_static: device memory that lives in the library's own image, so that the entry point
+// needs no caller workspace and allocates nothing.  Every GPU that runs the library holds its own copy of the array at
+// its own address (found once per device with hipGetSymbolAddress); the array's name itself is only a host-side
+// stand-in and is never passed to a kernel.
+static __device__ __align__(256) unsigned char scratch[LCE_STATIC_SCRATCH_BYTES];
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+// device address of `scratch` on the current device
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(LCE_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(LCE_E_ARG, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> l(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail(LCE_E_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return LCE_OK;
+}
+}  // namespace
+
 extern "C" {
 
 #ifdef LCE_DBG_TIMING
@@ -799,6 +826,23 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
                 void* stream) {
   return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
                        accumulate, entropy_b, workspace, workspace_bytes, stream, 0, nullptr);
+}
+
+int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T, int64_t H,
+                       int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy, float* maximum,
+                       float* accumulate, float* entropy_b, void* stream) {
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  const size_t need = lce_forward_workspace_bytes(T, H, V, dtype);
+  if (need > (size_t)LCE_STATIC_SCRATCH_BYTES)
+    return fail(LCE_E_WORKSPACE, "lce_forward_static: T=%lld needs %zu bytes of scratch, the built-in buffer holds %zu; use lce_forward with a workspace",
+                (long long)T, need, (size_t)LCE_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  // (what must start at zero, the label logits, is cleared by a fill kernel inside the forward: nothing of the previous
+  // call's contents is read)
+  return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
+                       accumulate, entropy_b, ws, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr);
 }
 
 int lce_forward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
