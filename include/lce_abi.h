@@ -157,6 +157,23 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
                  float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
                  float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same loss on PACKED model outputs: folds in the response slice that the no-padding engines apply between the
+ * head and the loss, no_padding_2_padding (verl/workers/utils/padding.py:97-141): for sequence r with prompt length
+ * P_r > 0 and response length R_r, packed end offset E_r = sum_{q <= r} (P_q + R_q), the padded element (r, c) is
+ * log_prob_packed[E_r - R_r - 1 + c] for c < R_r (the model output left-shifted by one token) and 0 beyond.
+ *   log_prob_packed, entropy_packed (may be NULL with g_entropy_packed) [total_nnz] fp32: what the fused head returns
+ *   response_start [rows] int64 = E_r - R_r - 1, response_len [rows] int64 = R_r (0 allowed), both on the device
+ *   everything else as in lce_ppo_loss, [rows, row_len] with row_len = max_response_len
+ *   g_log_prob_packed, g_entropy_packed [total_nnz]: the gradients IN PACKED ORDER (zero at every position that no
+ *   response token maps to), i.e. exactly the dlogprobs / dentropy vectors lce_backward takes: no gather or scatter
+ *   of per-token data remains between the two kernels. */
+int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packed, int64_t total_nnz, const int64_t* response_start,
+                        const int64_t* response_len, const float* old_log_prob, const float* advantages, const float* mask,
+                        const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef, int64_t rows, int64_t row_len,
+                        int agg_mode, float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
+                        float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
+                        float* g_log_prob_packed, float* g_entropy_packed, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Diagnostic: C[M, N] (fp32, row stride ldc) = A[M, K] . B[N, K]^T with the library's MFMA
  * mainloop (the same code that the entry points above use).  K a multiple of 64 (bf16) / 32 (fp32).
  * No counterpart in the reference; exists so the mainloop can be tested and timed on its own. */

@@ -22,6 +22,7 @@ What each function follows in the reference tree (paths relative to the referenc
 * ``policy_loss_vanilla``    verl/trainer/ppo/core_algos.py:1286-1376
 * ``kl_penalty``             verl/trainer/ppo/core_algos.py:2188-2251
 * ``ppo_actor_loss``         verl/workers/utils/losses.py:57-153 (policy loss minus entropy bonus plus KL penalty)
+* ``no_padding_2_padding``   verl/workers/utils/padding.py:97-141 (response slice of a packed model output)
 
 How each is pinned (see tests/test_oracle_*.py): the reference's own known-answer vector for the
 padded-vocab regression (tests/utils/test_linear_cross_entropy.py:352-395, closed form
@@ -33,7 +34,8 @@ for the gradients, the invariant ``sum_v dz = 0``, for ``sum_pi_squared_from_log
 ``lce_oracle.c``, and the reference's known answers for ``agg_loss`` / ``masked_mean``
 (tests/trainer/ppo/test_loss_aggregation_on_cpu.py:23-65, tests/utils/test_torch_functional.py:61-72);
 ``kl_penalty`` by its definitions evaluated with ``math.exp`` on scalars, ``k3 >= 0``, ``k3 = d^2/2 + O(d^3)``,
-``E_pi[k1] = E_pi[k3] = KL`` on a small categorical distribution and autograd for the straight-through variants.
+``E_pi[k1] = E_pi[k3] = KL`` on a small categorical distribution and autograd for the straight-through variants;
+``no_padding_2_padding`` by a packed batch written out by hand (response lengths 3, 1 and 0) and the reference's two assertions.
 No function here is "parity unpinned".
 """
 
@@ -334,6 +336,24 @@ def ppo_actor_loss(
         metrics["kl_coef"] = kl_loss_coef
     metrics["actor/pg_loss"] = pg.detach().item()
     return loss, metrics
+
+
+def no_padding_2_padding(values, prompt_lens, response_lens, max_response_len: Optional[int] = None):
+    """verl/workers/utils/padding.py:97-141: the response slice of a packed per-token model output.  Sequence r
+    occupies values[E_{r-1} : E_r], E_r = cumsum(prompt_lens + response_lens); its response part, left-shifted by one
+    token (the output at position i predicts token i + 1), is values[E_r - R_r - 1 : E_r - 1], right-padded with zeros
+    to max_response_len and stacked to [batch, max_response_len]."""
+    prompt_lens = torch.as_tensor(prompt_lens)
+    response_lens = torch.as_tensor(response_lens)
+    if max_response_len is None:
+        max_response_len = int(response_lens.max().item())
+    offsets = (prompt_lens + response_lens).cumsum(dim=0)
+    assert offsets[-1].item() == values.shape[0]
+    assert not prompt_lens.eq(0).any(), f"seq_offset - resp_len - 1 assumes prompt_len > 0. Got {prompt_lens}"
+    rows = []
+    for resp_len, end in zip(response_lens.tolist(), offsets.tolist()):
+        rows.append(torch.nn.functional.pad(values[end - resp_len - 1 : end - 1], (0, max_response_len - resp_len)))
+    return torch.stack(rows, dim=0)
 
 
 def padded_vocab_known_answer(V: int):

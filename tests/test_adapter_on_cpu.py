@@ -38,6 +38,9 @@ def captured(monkeypatch):
         return torch.zeros(labels.numel()), torch.ones(labels.numel())
 
     monkeypatch.setattr(dense_common, "linear_cross_entropy", fake)
+    from verl_amd.utils.experimental import torch_functional as experimental
+
+    monkeypatch.setattr(experimental, "linear_cross_entropy", fake)
     return calls
 
 
@@ -67,9 +70,24 @@ def test_patch_selection(captured, capsys):
     assert M.forward is orig
     monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend="bogus")
     assert M.forward is orig
-    for backend in ("triton", "torch", "liger", "hip"):
+    # the reference installs its triton forward for "triton" and its torch forward for "torch" / "liger"
+    # (verl/models/transformers/monkey_patch.py:281-291); the two differ in the shape and dtype of what they return
+    for backend, fwd in (("triton", dense_common.forward_with_hip_backend), ("hip", dense_common.forward_with_hip_backend),
+                         ("torch", dense_common.forward_with_torch_backend), ("liger", dense_common.forward_with_torch_backend)):
         monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend=backend)
-        assert M.forward is dense_common.forward_with_hip_backend and m._verl_fused_kernels_backend == backend
+        assert M.forward is fwd and m._verl_fused_kernels_backend == backend
     m.config.model_type = "qwen2_vl"
     with pytest.raises(NotImplementedError):
         monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend="hip")
+
+
+def test_torch_backend_returns_batch_shaped_outputs(captured):
+    """forward_with_torch_backend goes through FusedLinearForPPO (verl/models/transformers/dense_common.py:119-129):
+    outputs shaped like input_ids, entropy in the hidden dtype, so that output.log_probs[:, -R-1:-1] slices responses."""
+    m = _Model()
+    m._verl_fused_kernels_backend = "torch"
+    ids = torch.tensor([[5, 6, 7, 8], [1, 2, 3, 4]])
+    out = dense_common.forward_with_torch_backend(m, input_ids=ids, return_dict=True, temperature=0.5)
+    assert out.log_probs.shape == (2, 4) and out.entropy.shape == (2, 4) and out.entropy.dtype == torch.float32
+    assert captured["labels"].tolist() == [6, 7, 8, 5, 2, 3, 4, 1] and captured["temperature"] == 0.5
+    assert out.log_probs[:, -3:-1].shape == (2, 2)

@@ -237,3 +237,70 @@ def test_actor_step_fused_end_to_end():
     torch.testing.assert_close(loss, rloss, atol=1e-4, rtol=1e-4)
     assert (hh.grad.float() - h2.grad).abs().max() <= 2e-2 * h2.grad.abs().max()
     assert (ww.grad.float() - w2.grad).abs().max() <= 2e-2 * w2.grad.abs().max()
+
+
+def _packed_case(prompt, resp, R, seed):
+    g = torch.Generator().manual_seed(seed)
+    B, total = len(prompt), int(sum(prompt) + sum(resp))
+    lp = -torch.rand(total, generator=g) * 3
+    ent = torch.rand(total, generator=g) * 5
+    old = -torch.rand(B, R, generator=g) * 3
+    adv = torch.randn(B, 1, generator=g).expand(B, R).contiguous()
+    ref = -torch.rand(B, R, generator=g) * 3
+    mask = (torch.arange(R)[None, :] < torch.tensor(resp)[:, None]).float()
+    mask = mask * (torch.rand(B, R, generator=g) > 0.1).float()  # holes inside the responses too
+    return [t.to(DEV) for t in (lp, ent, old, adv, ref, mask)]
+
+
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean"])
+@pytest.mark.parametrize("with_kl", [False, True])
+def test_packed_outputs_response_slice_inside_the_kernel(mode, with_kl):
+    """fused_ppo_loss_packed against oracle slice (no_padding_2_padding, verl/workers/utils/padding.py:97-141) + oracle
+    loss: ragged prompts and responses, response lengths 0 and 1, a row as long as the padded width, holes in the mask;
+    the gradients come back in packed order and are exactly zero where no response position maps to."""
+    from verl_amd.workers.utils.losses import fused_ppo_loss_packed
+
+    prompt, resp = [3, 1, 7, 2, 1, 4, 260], [5, 1, 0, 9, 300, 2, 17]
+    R = 300
+    lp, ent, old, adv, ref, mask = _packed_case(prompt, resp, R, seed=5)
+    P, Rl = torch.tensor(prompt, device=DEV), torch.tensor(resp, device=DEV)
+    kw = dict(clip_ratio=0.2, entropy_coeff=1e-3, loss_agg_mode=mode)
+    if with_kl:
+        kw.update(ref_log_prob=ref, kl_loss_type="low_var_kl", kl_loss_coef=0.01)
+    lp1, ent1 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    loss, met = fused_ppo_loss_packed(lp1, ent1, P, Rl, old, adv, mask, clip_ratio_c=3.0, **kw)
+    (loss * 1.3).backward()
+    lp2, ent2 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    rloss, rmet = O.ppo_actor_loss(O.no_padding_2_padding(lp2, prompt, resp, R), O.no_padding_2_padding(ent2, prompt, resp, R),
+                                   old, adv, mask, **kw)
+    (rloss * 1.3).backward()
+    torch.testing.assert_close(loss, rloss, atol=1e-6, rtol=1e-5)
+    for k, v in met.items():
+        if k != "kl_coef":
+            assert v.item() == pytest.approx(rmet[k], rel=1e-5, abs=1e-6), k
+    assert lp1.grad.shape == lp.shape and ent1.grad.shape == ent.shape
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-8, rtol=1e-5)
+    torch.testing.assert_close(ent1.grad, ent2.grad, atol=1e-9, rtol=1e-5)
+    assert ((lp2.grad == 0) <= (lp1.grad == 0)).all()  # exact zeros wherever the oracle's gradient is zero
+    # the same numbers as the padded entry point on the oracle's slice
+    from verl_amd.workers.utils.losses import fused_ppo_loss
+
+    loss_p, _ = fused_ppo_loss(O.no_padding_2_padding(lp, prompt, resp, R), O.no_padding_2_padding(ent, prompt, resp, R), old, adv, mask,
+                               clip_ratio_c=3.0, **kw)
+    torch.testing.assert_close(loss.detach(), loss_p, atol=0, rtol=0)
+
+
+def test_packed_outputs_reference_assertions():
+    from verl_amd.workers.utils.losses import fused_ppo_loss_packed
+
+    prompt, resp, R = [2, 1, 3], [3, 1, 0], 4
+    lp, ent, old, adv, ref, mask = _packed_case(prompt, resp, R, seed=6)
+    P, Rl = torch.tensor(prompt, device=DEV), torch.tensor(resp, device=DEV)
+    with pytest.raises(AssertionError, match="prompt_len > 0"):  # verl/workers/utils/padding.py:128
+        fused_ppo_loss_packed(lp, ent, torch.tensor([2, 0, 4], device=DEV), Rl, old, adv, mask)
+    with pytest.raises(AssertionError):  # lengths that do not add up to total_nnz (:127)
+        fused_ppo_loss_packed(lp[:-1], ent[:-1], P, Rl, old, adv, mask)
+    with pytest.raises(AssertionError, match="longer than max_response_len"):
+        fused_ppo_loss_packed(lp, ent, P, Rl, old[:, :2], adv[:, :2], mask[:, :2])
+    loss, _ = fused_ppo_loss_packed(lp, None, P, Rl, old, adv, mask)  # entropy is optional as in fused_ppo_loss
+    assert torch.isfinite(loss)

@@ -138,3 +138,25 @@ def test_actor_loss_with_kl_term_is_the_sum_of_its_parts():
         want = pg - 0.1 * O.agg_loss(ent, mask, mode) + 0.3 * O.agg_loss(O.kl_penalty(lp, ref, "k3"), mask, mode)
         torch.testing.assert_close(loss, want)
         assert met["kl_coef"] == 0.3 and met["kl_loss"] == pytest.approx(O.agg_loss(O.kl_penalty(lp, ref, "k3"), mask, mode).item())
+
+
+def test_response_slice_of_packed_outputs_hand_written_batch():
+    """no_padding_2_padding (verl/workers/utils/padding.py:97-141) on a packed batch written out by hand: three
+    sequences with (prompt, response) lengths (2, 3), (1, 1), (3, 0); the packed per-token values are 100 * sequence +
+    position.  The response part is left-shifted by one token: sequence 0 occupies packed[0:5] and its response slice
+    is positions 1..3 (the outputs that PREDICT the three response tokens at positions 2..4)."""
+    values = torch.tensor([0.0, 1, 2, 3, 4, 100, 101, 200, 201, 202])
+    out = O.no_padding_2_padding(values, [2, 1, 3], [3, 1, 0], max_response_len=4)
+    want = torch.tensor([[1.0, 2, 3, 0], [100, 0, 0, 0], [0, 0, 0, 0]])
+    assert torch.equal(out, want)
+    # default width = the longest response
+    assert torch.equal(O.no_padding_2_padding(values, [2, 1, 3], [3, 1, 0]), want[:, :3])
+    # the reference's two assertions
+    with pytest.raises(AssertionError, match="prompt_len > 0"):
+        O.no_padding_2_padding(values, [2, 0, 3], [3, 2, 0])
+    with pytest.raises(AssertionError):
+        O.no_padding_2_padding(values[:-1], [2, 1, 3], [3, 1, 0])
+    # a slice never takes the last token's output of its sequence and never reaches into the previous sequence
+    v = torch.arange(12.0)
+    got = O.no_padding_2_padding(v, [1, 1], [5, 5])
+    assert torch.equal(got, torch.tensor([[0.0, 1, 2, 3, 4], [6, 7, 8, 9, 10]]))

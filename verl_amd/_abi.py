@@ -37,6 +37,7 @@ SYMBOLS = {
     "lce_logits_sum_pi_squared": (_i, [_p, _i64, _i64, _i64, _i, _p, _p]),
     "lce_ppo_loss_workspace_bytes": (_sz, [_i64, _i64]),
     "lce_ppo_loss": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _f, _i64, _i64, _i, _f, _f, _f, _f, _f, _f, _f, _f, _p, _p, _p, _p, _sz, _p]),
+    "lce_ppo_loss_packed": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _f, _i64, _i64, _i, _f, _f, _f, _f, _f, _f, _f, _f, _p, _p, _p, _p, _sz, _p]),
     "lce_gemm_nt": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _i, _p]),
     "lce_gemm_tn": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),
     "lce_set_variant": (_i, [_i]),

@@ -1039,12 +1039,13 @@ size_t lce_ppo_loss_workspace_bytes(int64_t rows, int64_t row_len) {
          ppo_align((size_t)rows * sizeof(float));
 }
 
-int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
-                 const float* mask, const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef,
-                 int64_t rows, int64_t row_len, int agg_mode,
-                 float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
-                 float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
-                 float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream) {
+// shared body of lce_ppo_loss and lce_ppo_loss_packed
+static int ppo_entry(const float* log_prob, const float* entropy, const int64_t* pk_start, const int64_t* pk_len, int64_t total_nnz,
+                     const float* old_log_prob, const float* advantages, const float* mask, const float* is_weights,
+                     const float* ref_log_prob, int kl_type, float kl_coef, int64_t rows, int64_t row_len, int agg_mode, float clip_low,
+                     float clip_high, float clip_c, float entropy_coeff, float dp_size, float batch_num_tokens,
+                     float global_batch_size, float loss_scale_factor, float* out, float* g_log_prob, float* g_entropy,
+                     void* workspace, size_t workspace_bytes, void* stream) {
   if (rows <= 0 || row_len <= 0) return fail(LCE_E_ARG, "ppo loss: rows and row_len must be positive");
   if (rows > ((int64_t)1 << 30) || row_len > ((int64_t)1 << 40) / rows) return fail(LCE_E_ARG, "ppo loss: too many elements");
   if (!mask || !out) return fail(LCE_E_ARG, "null pointer");
@@ -1055,6 +1056,8 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
     return fail(LCE_E_ARG, "without log_prob the call aggregates `entropy` alone");
   }
   if ((entropy == nullptr) != (g_entropy == nullptr)) return fail(LCE_E_ARG, "entropy and g_entropy go together");
+  if ((pk_start == nullptr) != (pk_len == nullptr)) return fail(LCE_E_ARG, "packed layout: starts and lengths go together");
+  if (pk_start && total_nnz < 0) return fail(LCE_E_ARG, "packed layout: total_nnz must be >= 0");
   const int kl_base = kl_type & ~LCE_PPO_KL_STRAIGHT_THROUGH;
   if (kl_base < LCE_PPO_KL_NONE || kl_base > LCE_PPO_KL_K3 || (kl_base == LCE_PPO_KL_NONE && kl_type != LCE_PPO_KL_NONE))
     return fail(LCE_E_ARG, "ppo loss: unknown kl_type %d", kl_type);
@@ -1081,19 +1084,52 @@ int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_l
   p.kl_straight_through = (kl_type & LCE_PPO_KL_STRAIGHT_THROUGH) != 0 && kl_base != LCE_PPO_KL_K2;
   p.clip_low = clip_low; p.clip_high = clip_high; p.clip_c = clip_c; p.entropy_coeff = entropy_coeff;
   p.g_log_prob = g_log_prob; p.g_entropy = g_entropy;
+  p.pk_start = pk_start; p.pk_len = pk_len; p.total_nnz = total_nnz;
   PpoAgg g;
   g.mode = agg_mode; g.dp_size = dp_size; g.batch_num_tokens = batch_num_tokens; g.global_batch_size = global_batch_size;
   g.loss_scale_factor = loss_scale_factor; g.entropy_coeff = entropy_coeff;
   g.kl_coef = kl_base != LCE_PPO_KL_NONE ? kl_coef : 0.f;
+  int rc;
+  if (pk_start && total_nnz > 0) {
+    // packed gradients: the positions no response token maps to (prompts, the last token of each sequence) are zeros
+    for (float* gp : {g_log_prob, g_entropy}) {
+      if (!gp) continue;
+      hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((total_nnz + 1023) / 1024 < 4096 ? (total_nnz + 1023) / 1024 : 4096)), dim3(256), 0, st,
+                         reinterpret_cast<uint32_t*>(gp), total_nnz);
+      if ((rc = check_launch("fill_zero_kernel"))) return rc;
+    }
+  }
   hipLaunchKernelGGL(ppo_terms_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
-  int rc = check_launch("ppo_terms_kernel");
-  if (rc) return rc;
+  if ((rc = check_launch("ppo_terms_kernel"))) return rc;
   hipLaunchKernelGGL(ppo_finish_kernel, dim3(1), dim3(256), 0, st, p.partials, rows, p.segs, row_len, g, row_tot,
                      row_weight, out);
   if ((rc = check_launch("ppo_finish_kernel"))) return rc;
-  hipLaunchKernelGGL(ppo_scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g_log_prob, g_entropy, row_len,
-                     p.segs, p.seg_len, row_weight);
+  hipLaunchKernelGGL(ppo_scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p, row_weight);
   return check_launch("ppo_scale_kernel");
+}
+
+int lce_ppo_loss(const float* log_prob, const float* entropy, const float* old_log_prob, const float* advantages,
+                 const float* mask, const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef,
+                 int64_t rows, int64_t row_len, int agg_mode,
+                 float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
+                 float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
+                 float* g_log_prob, float* g_entropy, void* workspace, size_t workspace_bytes, void* stream) {
+  return ppo_entry(log_prob, entropy, nullptr, nullptr, 0, old_log_prob, advantages, mask, is_weights, ref_log_prob, kl_type, kl_coef, rows,
+                   row_len, agg_mode, clip_low, clip_high, clip_c, entropy_coeff, dp_size, batch_num_tokens, global_batch_size,
+                   loss_scale_factor, out, g_log_prob, g_entropy, workspace, workspace_bytes, stream);
+}
+
+int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packed, int64_t total_nnz, const int64_t* response_start,
+                        const int64_t* response_len, const float* old_log_prob, const float* advantages, const float* mask,
+                        const float* is_weights, const float* ref_log_prob, int kl_type, float kl_coef, int64_t rows, int64_t row_len,
+                        int agg_mode, float clip_low, float clip_high, float clip_c, float entropy_coeff, float dp_size,
+                        float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
+                        float* g_log_prob_packed, float* g_entropy_packed, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!log_prob_packed || !response_start || !response_len) return fail(LCE_E_ARG, "ppo loss (packed): null pointer");
+  return ppo_entry(log_prob_packed, entropy_packed, response_start, response_len, total_nnz, old_log_prob, advantages, mask, is_weights,
+                   ref_log_prob, kl_type, kl_coef, rows, row_len, agg_mode, clip_low, clip_high, clip_c, entropy_coeff, dp_size,
+                   batch_num_tokens, global_batch_size, loss_scale_factor, out, g_log_prob_packed, g_entropy_packed, workspace,
+                   workspace_bytes, stream);
 }
 
 int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, int64_t R, int64_t V, int dtype,

@@ -1201,7 +1201,22 @@ struct PpoArgs {
   float* g_log_prob;  // unscaled d(sum of masked losses)/d log_prob
   float* g_entropy;   // may be null
   float* partials;    // [rows * segs][8]
+  // Packed model outputs (both null: log_prob, entropy and the two gradients are [rows][row_len] like everything else).
+  // Otherwise log_prob / entropy / g_log_prob / g_entropy are [total_nnz] vectors over the packed sequences and element
+  // (row, c) lives at pk_start[row] + c for c < pk_len[row]; beyond that the value is the padding constant 0 and there is
+  // no gradient to write (the response slice of verl/workers/utils/padding.py:97-141, left-shifted by one token:
+  // pk_start = end of the sequence - response length - 1).
+  const int64_t* pk_start;
+  const int64_t* pk_len;
+  int64_t total_nnz;
 };
+
+// index of element (row, c) in the model-output vectors, or -1 for a padding position of the packed layout
+LCE_DEV int64_t ppo_out_index(const PpoArgs& p, int64_t row, int64_t c) {
+  if (!p.pk_start) return row * p.row_len + c;
+  const int64_t i = p.pk_start[row] + c;
+  return (c < p.pk_len[row] && i >= 0 && i < p.total_nnz) ? i : -1;
+}
 
 // Per-token terms and unscaled gradients; workgroup (row, seg) reduces its segment of one row to
 // partials[row * segs + seg][0..6] = sums of (loss, entropy, clipped, -log ratio, dual-clipped, 1, kl) x mask.
@@ -1213,24 +1228,27 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
   const int64_t c1 = c0 + p.seg_len < p.row_len ? c0 + p.seg_len : p.row_len;
   for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
     const int64_t t = row * p.row_len + c;
+    const int64_t to = ppo_out_index(p, row, c);
     const float m = p.mask[t];
     const bool on = m != 0.f;  // values outside the mask never reach a sum (NaNs there are harmless)
     float loss = 0.f, dloss = 0.f, nkl = 0.f, clipped = 0.f, dual_clipped = 0.f;
     if (p.log_prob) {
-      const float lp = p.log_prob[t], A = p.advantages[t];
+      const float lp = to >= 0 ? p.log_prob[to] : 0.f, A = p.advantages[t];
       const float d = lp - p.old_log_prob[t];
       nkl = fminf(fmaxf(d, -20.f), 20.f);
       const float r = __expf(nkl);
-      const float dr = (d > -20.f && d < 20.f) ? r : 0.f;          // d ratio / d log_prob
+      // (the clamps pass the gradient ON their bounds, as torch.clamp's backward does, and the maximum / minimum split
+      // it evenly at a tie, as torch.maximum / torch.min do: the reference's autograd at the kinks)
+      const float dr = (d >= -20.f && d <= 20.f) ? r : 0.f;        // d ratio / d log_prob
       const float rc = fminf(fmaxf(r, 1.f - p.clip_low), 1.f + p.clip_high);
-      const float drc = (r > 1.f - p.clip_low && r < 1.f + p.clip_high) ? dr : 0.f;
+      const float drc = (r >= 1.f - p.clip_low && r <= 1.f + p.clip_high) ? dr : 0.f;
       const float l1 = -A * r, l2 = -A * rc, l3 = -A * p.clip_c;
       const float lc1 = fmaxf(l1, l2);
       const float dlc1 = l1 > l2 ? -A * dr : (l2 > l1 ? -A * drc : -A * 0.5f * (dr + drc));
       const bool dual = A < 0.f;
       const float isw = p.is_weights ? p.is_weights[t] : 1.f;
       loss = (dual ? fminf(l3, lc1) : lc1) * isw;
-      dloss = ((dual && l3 < lc1) ? 0.f : dlc1) * isw;
+      dloss = (dual ? (l3 < lc1 ? 0.f : (l3 == lc1 ? 0.5f * dlc1 : dlc1)) : dlc1) * isw;
       clipped = l2 > l1 ? 1.f : 0.f;
       dual_clipped = (lc1 > l3 && dual) ? 1.f : 0.f;
       float kl = 0.f;
@@ -1256,13 +1274,13 @@ __global__ void ppo_terms_kernel(PpoArgs p) {
         if (p.kl_straight_through) dkl = e;
         dloss += p.kl_coef * dkl;
       }
-      p.g_log_prob[t] = on ? dloss * m : 0.f;
+      if (to >= 0) p.g_log_prob[to] = on ? dloss * m : 0.f;
       if (on) s[6] += kl * m;
     }
     float ent = 0.f;
     if (p.entropy) {
-      ent = p.entropy[t];
-      p.g_entropy[t] = on ? -p.entropy_coeff * m : 0.f;
+      ent = to >= 0 ? p.entropy[to] : 0.f;
+      if (to >= 0) p.g_entropy[to] = on ? -p.entropy_coeff * m : 0.f;
     }
     if (on) {
       s[0] += loss * m;
@@ -1374,16 +1392,16 @@ __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs,
   }
 }
 
-__global__ void ppo_scale_kernel(float* g_lp, float* g_ent, int64_t row_len, int segs, int64_t seg_len,
-                                 const float* row_weight) {
-  const int64_t row = (int64_t)blockIdx.x / segs;
-  const int64_t c0 = ((int64_t)blockIdx.x % segs) * seg_len;
-  const int64_t c1 = c0 + seg_len < row_len ? c0 + seg_len : row_len;
+__global__ void ppo_scale_kernel(PpoArgs p, const float* row_weight) {
+  const int64_t row = (int64_t)blockIdx.x / p.segs;
+  const int64_t c0 = ((int64_t)blockIdx.x % p.segs) * p.seg_len;
+  const int64_t c1 = c0 + p.seg_len < p.row_len ? c0 + p.seg_len : p.row_len;
   const float scale = row_weight[row];
   for (int64_t c = c0 + threadIdx.x; c < c1; c += blockDim.x) {
-    const int64_t t = row * row_len + c;
-    if (g_lp) g_lp[t] *= scale;
-    if (g_ent) g_ent[t] *= scale;
+    const int64_t t = ppo_out_index(p, row, c);
+    if (t < 0) continue;
+    if (p.g_log_prob) p.g_log_prob[t] *= scale;
+    if (p.g_entropy) p.g_entropy[t] *= scale;
   }
 }
 

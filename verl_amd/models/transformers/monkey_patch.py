@@ -1,20 +1,23 @@
 """Selects the fused-kernel forward for a HF causal LM.
 
 Same entry point as the reference's ``patch_forward_with_backends``
-(``verl/models/transformers/monkey_patch.py:234-291``).  Every backend name verl's configuration can
-carry (``triton``, ``torch``, ``liger``) and the explicit ``hip`` select the one HIP path here, so an
-existing ``fused_kernel_options.impl_backend`` keeps working.  Only dense text models are covered
-(the reference's VLM variants differ in how they build hidden states, not in the head).
+(``verl/models/transformers/monkey_patch.py:234-291``).  Every backend name verl's configuration can carry keeps
+working, with the output shape that backend has in the reference: ``triton`` (and the explicit ``hip``) install the
+forward that returns ``linear_cross_entropy``'s flat fp32 vectors, ``torch`` (verl's default ``impl_backend``) and
+``liger`` the one that goes through ``FusedLinearForPPO`` and returns ``[batch, seq]`` outputs with the entropy in the
+hidden dtype; all of them run the same HIP kernels.  Only dense text models are covered (the reference's VLM variants
+differ in how they build hidden states, not in the head).
 """
 
 from __future__ import annotations
 
-_BACKENDS = ("hip", "triton", "torch", "liger")
+_FLAT_BACKENDS = ("hip", "triton")
+_SHAPED_BACKENDS = ("torch", "liger")
 _VLM_TYPES = ("qwen2_5_vl", "qwen2_vl", "qwen3_vl", "qwen3_vl_moe", "glm4v", "qwen3_5", "qwen3_5_moe")
 
 
 def patch_forward_with_backends(model, use_fused_kernels: bool = False, fused_kernels_backend: str = None):
-    if not use_fused_kernels or fused_kernels_backend not in _BACKENDS:
+    if not use_fused_kernels or fused_kernels_backend not in _FLAT_BACKENDS + _SHAPED_BACKENDS:
         print(
             f"Skipping monkey patch for {model.__class__.__name__} as use_fused_kernels is "
             f"{use_fused_kernels} or fused_kernels_backend is {fused_kernels_backend}"
@@ -22,8 +25,9 @@ def patch_forward_with_backends(model, use_fused_kernels: bool = False, fused_ke
         return
     if getattr(model.config, "model_type", None) in _VLM_TYPES:
         raise NotImplementedError(f"model_type {model.config.model_type}: only dense text models are adapted")
-    from .dense_common import forward_with_hip_backend
+    from .dense_common import forward_with_hip_backend, forward_with_torch_backend
 
     model._verl_fused_kernels_backend = fused_kernels_backend
-    model.__class__.forward = forward_with_hip_backend
-    print(f"Using HIP backend for fused kernels in {model.__class__.__name__}")
+    flat = fused_kernels_backend in _FLAT_BACKENDS
+    model.__class__.forward = forward_with_hip_backend if flat else forward_with_torch_backend
+    print(f"Using HIP kernels behind the {fused_kernels_backend} backend for fused kernels in {model.__class__.__name__}")

@@ -59,7 +59,10 @@ class _FusedPPOLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, agg, kl,
-                clip_low, clip_high, clip_c, entropy_coeff):
+                clip_low, clip_high, clip_c, entropy_coeff, packed=None):
+        if packed is not None:
+            return _FusedPPOLoss._forward_packed(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights,
+                                                 ref_log_prob, agg, kl, clip_low, clip_high, clip_c, entropy_coeff, packed)
         lead = log_prob if log_prob is not None else entropy
         assert lead.is_cuda, "fused_ppo_loss runs on the GPU only"
         dev = lead.device
@@ -101,11 +104,56 @@ class _FusedPPOLoss(torch.autograd.Function):
         return out[0], out
 
     @staticmethod
+    def _forward_packed(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, agg, kl,
+                        clip_low, clip_high, clip_c, entropy_coeff, packed):
+        """log_prob / entropy are [total_nnz] model outputs over the packed sequences; everything else is
+        [batch, max_response_len]; packed = (response_start, response_len) int64 [batch] on the device."""
+        assert log_prob is not None and log_prob.is_cuda, "fused_ppo_loss_packed runs on the GPU only"
+        dev = log_prob.device
+        start, length = packed
+        rows, row_len = response_mask.shape
+        total = log_prob.numel()
+
+        def f32(t, n):
+            if t is None:
+                return None
+            t = t.detach().reshape(-1).to(torch.float32).contiguous()
+            assert t.numel() == n
+            return t
+
+        lp, ent = f32(log_prob, total), f32(entropy, total)
+        old, adv, mask = f32(old_log_prob, rows * row_len), f32(advantages, rows * row_len), f32(response_mask, rows * row_len)
+        isw, ref = f32(is_weights, rows * row_len), f32(ref_log_prob, rows * row_len)
+        mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor = agg
+        kl_type, kl_coef = kl
+        out = torch.empty(16, device=dev, dtype=torch.float32)
+        g_lp = torch.empty(total, device=dev, dtype=torch.float32)
+        g_ent = None if ent is None else torch.empty(total, device=dev, dtype=torch.float32)
+        lib = _abi.load()
+        with torch.cuda.device(dev):
+            ws_bytes = lib.lce_ppo_loss_workspace_bytes(rows, row_len)
+            ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+            rc = lib.lce_ppo_loss_packed(
+                lp.data_ptr(), _abi.ptr(ent), total, start.data_ptr(), length.data_ptr(), old.data_ptr(), adv.data_ptr(),
+                mask.data_ptr(), _abi.ptr(isw), _abi.ptr(ref), kl_type, kl_coef, rows, row_len, mode, clip_low, clip_high, clip_c,
+                entropy_coeff, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor, out.data_ptr(), g_lp.data_ptr(),
+                _abi.ptr(g_ent), ws.data_ptr(), ws_bytes, _abi.current_stream(dev),
+            )  # fmt: skip
+            _abi.check(rc, "lce_ppo_loss_packed")
+        empty = out.new_empty(0)
+        ctx.save_for_backward(g_lp, g_ent if g_ent is not None else empty)
+        ctx.has = (True, ent is not None)
+        ctx.shape = log_prob.shape
+        ctx.dtypes = (log_prob.dtype, None if entropy is None else entropy.dtype)
+        ctx.mark_non_differentiable(out)
+        return out[0], out
+
+    @staticmethod
     def backward(ctx, g_loss, _g_out):
         g_lp, g_ent = ctx.saved_tensors
         d_lp = (g_lp * g_loss).reshape(ctx.shape).to(ctx.dtypes[0]) if ctx.has[0] else None
         d_ent = (g_ent * g_loss).reshape(ctx.shape).to(ctx.dtypes[1]) if ctx.has[1] else None
-        return (d_lp, d_ent) + (None,) * 11
+        return (d_lp, d_ent) + (None,) * 12
 
 
 def fused_ppo_loss(
@@ -128,6 +176,7 @@ def fused_ppo_loss(
     ref_log_prob: Optional[torch.Tensor] = None,
     kl_loss_coef: float = 0.001,
     kl_loss_type: str = "low_var_kl",
+    _packed=None,
 ):
     """Returns ``(policy_loss, metrics)``: ``policy_loss = pg_loss - entropy_coeff * entropy_loss
     [+ kl_loss_coef * kl_loss]`` (a 0-dim tensor with autograd), ``metrics`` a dict of 0-dim tensors under the
@@ -144,7 +193,7 @@ def fused_ppo_loss(
     kl = (0, 0.0) if ref_log_prob is None else (kl_type_number(kl_loss_type), float(kl_loss_coef))
     loss, out = _FusedPPOLoss.apply(
         log_prob, entropy, old_log_prob, advantages, response_mask, rollout_is_weights, ref_log_prob, agg, kl,
-        float(lo), float(hi), float(clip_ratio_c), float(entropy_coeff),
+        float(lo), float(hi), float(clip_ratio_c), float(entropy_coeff), _packed,
     )  # fmt: skip
     metrics = {
         "actor/pg_loss": out[1],
@@ -158,3 +207,41 @@ def fused_ppo_loss(
         metrics["kl_loss"] = out[8]
         metrics["kl_coef"] = kl_loss_coef
     return loss, metrics
+
+
+def response_slices(prompt_lens: torch.Tensor, response_lens: torch.Tensor, total_nnz: int):
+    """``(start, length)`` per sequence of the response slice that ``no_padding_2_padding`` takes out of a packed model
+    output (``verl/workers/utils/padding.py:97-141``): ``start = end of the sequence - response length - 1`` (the
+    left shift by one token), with the reference's two assertions."""
+    prompt_lens = prompt_lens.to(torch.int64)
+    response_lens = response_lens.to(torch.int64)
+    sequence_offsets = (prompt_lens + response_lens).cumsum(dim=0)
+    assert sequence_offsets[-1].item() == total_nnz
+    assert not prompt_lens.eq(0).any(), f"seq_offset - resp_len - 1 assumes prompt_len > 0. Got {prompt_lens}"
+    return (sequence_offsets - response_lens - 1).contiguous(), response_lens.contiguous()
+
+
+def fused_ppo_loss_packed(
+    log_prob: torch.Tensor,
+    entropy: Optional[torch.Tensor],
+    prompt_lens: torch.Tensor,
+    response_lens: torch.Tensor,
+    old_log_prob: torch.Tensor,
+    advantages: torch.Tensor,
+    response_mask: torch.Tensor,
+    **kwargs,
+):
+    """``fused_ppo_loss`` for the no-padding engines: ``log_prob`` / ``entropy`` are the fused head's outputs over the
+    PACKED sequences, ``[total_nnz]``; ``prompt_lens`` / ``response_lens`` ``[batch]`` (integer tensors on the device);
+    ``old_log_prob``, ``advantages``, ``response_mask`` (and ``rollout_is_weights``, ``ref_log_prob``) stay
+    ``[batch, max_response_len]`` as the data batch holds them.  The kernel applies the response slice of
+    ``no_padding_2_padding`` (``verl/workers/utils/padding.py:97-141``) while it reads, and the gradients flow back in
+    packed order, so the backward of ``linear_cross_entropy`` starts from them without a gather or a scatter.
+    Same keyword arguments, return values and metrics as ``fused_ppo_loss``."""
+    assert log_prob.dim() == 1 and (entropy is None or entropy.shape == log_prob.shape), "packed outputs are [total_nnz]"
+    assert response_mask.dim() == 2 and old_log_prob.shape == response_mask.shape == advantages.shape
+    assert prompt_lens.shape == response_lens.shape == (response_mask.shape[0],)
+    dev = log_prob.device
+    start, length = response_slices(prompt_lens.to(dev), response_lens.to(dev), log_prob.numel())
+    assert int(length.max().item()) <= response_mask.shape[1], "a response is longer than max_response_len"
+    return fused_ppo_loss(log_prob, entropy, old_log_prob, advantages, response_mask, _packed=(start, length), **kwargs)
