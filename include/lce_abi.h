@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 6
+#define LCE_ABI_VERSION 7
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1, LCE_DTYPE_F16 = 2 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -76,6 +76,14 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
                  const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                  void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
                  void* stream);
+
+/* The same backward with both gradients returned in fp32, d_hidden [T, H] and d_weight [V, H] contiguous: what
+ * should_return_fp32_grad of efficient_entropy_backward asks for (verl/utils/kernel/kernels.py:1562-1567).  The sums are
+ * carried in fp32 anyway; here they are stored without the final rounding to the input dtype.  Same workspace. */
+int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T, int64_t H,
+                     int64_t V, int dtype, float temperature, int reduction, const float* maximum, const float* accumulate,
+                     const float* entropy_b, const float* dlogprobs, const float* dentropy, float* d_hidden, float* d_weight,
+                     void* workspace, size_t workspace_bytes, int64_t vchunk, void* stream);
 
 /* Vocabulary-parallel building blocks: what one rank of a tensor-parallel lm-head runs on its shard
  * W[vocab_offset : vocab_offset + V_local, :] of the vocabulary.  The exchange between the ranks (an
@@ -212,7 +220,8 @@ enum {
   LCE_OPT_DLOGITS_FEW_TOKEN_TILES = 5,
   LCE_OPT_DLOGITS_STRIP = 6,
   LCE_OPT_DHIDDEN_KSPLIT = 7,
-  LCE_OPT_WORKSPACE_BUDGET = 8
+  LCE_OPT_WORKSPACE_BUDGET = 8,
+  LCE_OPT_FEW_TOKEN_GEMMS = 9
 };
 int lce_set_option(int key, int64_t value);
 

@@ -50,6 +50,43 @@ def test_abi_version_and_error_string():
         assert lib.lce_backward_workspace_bytes(T, H, V, dt, 0) < 0.25 * T * V * esz + 4 * V * H, (T, H, V, dt)
 
 
+def test_default_chunk_rule_and_workspace_budget():
+    """Default: chunks of 8192 vocabulary columns (wider while one d_logits buffer stays within 256 MiB), so the backward's
+    workspace at config 2 is under 1 GiB; a byte budget (kernels.set_workspace_budget / LCE_OPT_WORKSPACE_BUDGET) makes
+    the library pick the widest chunk that fits, never exceeding its upper bound and never going below 2048 columns; an
+    explicit chunk width wins over both."""
+    from verl_amd.utils.kernel import kernels
+
+    lib = _abi.load()
+    T, H, V = 16384, 3584, 152064
+    gate = 0.25 * T * V * 2 + 4 * V * H
+    try:
+        default = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
+        assert default < (1 << 30)
+        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 8192) == default  # 19 chunks of 8192 columns
+        # few tokens: the whole vocabulary in one chunk (one single-buffered d_logits tile)
+        few = lib.lce_backward_workspace_bytes(64, H, V, 0, 0)
+        assert few == lib.lce_backward_workspace_bytes(64, H, V, 0, 152064)
+        sizes = []
+        for budget in (600 << 20, 1 << 30, 2 << 30, 1 << 40):
+            kernels.set_workspace_budget(budget)
+            n = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
+            sizes.append(n)
+            assert n < gate
+            if budget >= (700 << 20):
+                assert n <= min(budget, gate)
+        assert sizes == sorted(sizes) and sizes[0] < default < sizes[2] and sizes[3] > (2 << 30)
+        # a budget no chunk of at least 2048 columns fits: the floor is what is reported (and what lce_backward asks for)
+        kernels.set_workspace_budget(1 << 20)
+        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) == lib.lce_backward_workspace_bytes(T, H, V, 0, 2048)
+        # an explicit width is not touched by the budget
+        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 8192) == default
+    finally:
+        kernels.set_workspace_budget(0)
+    assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) == default
+    assert lib.lce_set_option(8, -1) != 0
+
+
 def test_signature_matches_reference():
     from verl_amd.utils.kernel.linear_cross_entropy import LinearCrossEntropy
     from verl_amd.utils.kernel import kernels
@@ -162,3 +199,39 @@ def test_logits_twins_name_the_gpu_only_precondition():
                  lambda: F.calculate_sum_pi_squared_from_logits(z)):
         with pytest.raises(_abi.LceError, match="GPU tensors only"):
             call()
+
+
+def test_metric_aggregation_kinds_of_ppo_loss():
+    """verl/workers/utils/losses.py:71-84: any global normaliser switches the loss metrics to SUM; Metric folds as
+    verl/utils/metric/utils.py:72-160 (hand-computed numbers)."""
+    from verl_amd.trainer.ppo import core_algos as C
+    from verl_amd.utils.metric import AggregationType, Metric
+    from verl_amd.workers.utils.losses import metric_aggregation_for
+
+    assert metric_aggregation_for(1, None, None, None) == AggregationType.MEAN
+    assert metric_aggregation_for(2, None, None, None) == AggregationType.SUM
+    assert metric_aggregation_for(1, 100, None, None) == AggregationType.SUM
+    assert metric_aggregation_for(1, None, 8, None) == AggregationType.SUM
+    assert metric_aggregation_for(1, None, None, 512) == AggregationType.SUM
+    m = Metric("mean", 1.0)
+    m.append(torch.tensor(2.0))
+    m.append(Metric(AggregationType.MEAN, [3.0, 6.0]))
+    assert m.aggregate() == 3.0
+    assert Metric("sum", [1, 2, 3.5]).aggregate() == 6.5
+    assert Metric("min", [4, 2, 3]).aggregate() == 2 and Metric("max", [4, 2, 3]).aggregate() == 4
+    with pytest.raises(ValueError, match="mismatch"):
+        m.append(Metric("sum", 1.0))
+    with pytest.raises(ValueError, match="scalar"):
+        m.append(torch.zeros(2))
+    with pytest.raises(ValueError):
+        Metric("median")
+    # two ranks, two accumulation steps: SUM adds the per-step means over ranks, MAX looks at every value
+    assert Metric.aggregate_dp([Metric("sum", [1.0, 3.0]), Metric("sum", [3.0, 5.0])]) == 6.0
+    assert Metric.aggregate_dp([Metric("mean", [1.0, 3.0]), Metric("mean", [3.0, 5.0])]) == 3.0
+    assert Metric.aggregate_dp([Metric("max", [1.0, 9.0]), Metric("max", [3.0, 5.0])]) == 9.0
+    with pytest.raises(ValueError, match="same number of values"):
+        Metric.aggregate_dp([Metric("sum", [1.0]), Metric("sum", [1.0, 2.0])])
+    d = Metric.from_dict({"a": 1.0, "b": 2.0}, "mean")
+    assert d["b"].aggregate() == 2.0 and d["a"].aggregation == AggregationType.MEAN
+    with pytest.raises(ValueError, match="Unsupported loss mode: gpg"):
+        C.get_policy_loss_fn("gpg")

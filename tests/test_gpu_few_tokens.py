@@ -1,0 +1,137 @@
+"""Backward with at most 128 tokens and 16-bit inputs: both gradient GEMMs run as streaming kernels (one launch,
+d_weight rows written once in 64-byte runs, d_hidden from fp32 K-slice partials with W read in place) instead of
+the 256 x 256 tile kernels.  Same bar as every other backward (verl/utils/kernel/kernels.py:1380-1515,1666-1724 is
+the reference's schedule for these two products): 2e-2 absolute for bf16 against the oracle, bit-identical reruns,
+and agreement with the tile kernels that LCE_OPT_FEW_TOKEN_GEMMS = 0 selects."""
+
+import pytest
+import torch
+
+from oracle import lce_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+OPT_FEW_TOKEN_GEMMS = 9
+
+
+def _case(T, H, V, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    h = torch.randn(T, H, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(V, H, generator=g) * 0.05).to(dtype).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = torch.randn(T, generator=g).to(DEV)
+    g_ent = torch.randn(T, generator=g).to(DEV)
+    return h, w, y, g_lp, g_ent
+
+
+def _run(h, w, y, tau, g_lp, g_ent, few=1, vchunk=0, fp32_grad=False):
+    from verl_amd import _abi, linear_cross_entropy
+    from verl_amd.utils.kernel import kernels
+
+    lib = _abi.load()
+    hh, ww = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    try:
+        assert lib.lce_set_option(OPT_FEW_TOKEN_GEMMS, few) == 0
+        kernels.set_vocab_chunk(vchunk)
+        if fp32_grad:
+            lp, ent, mx, acc, eb = kernels.efficient_entropy_forward(h, w, y, 0, tau)
+            dh, dw = kernels.efficient_entropy_backward(g_lp, g_ent, h, w, y, mx, acc, eb, 0, True, tau)
+        else:
+            lp, ent = linear_cross_entropy(hh, ww, y, tau, "none")
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+            dh, dw = hh.grad, ww.grad
+        torch.cuda.synchronize()
+    finally:
+        kernels.set_vocab_chunk(0)
+        lib.lce_set_option(OPT_FEW_TOKEN_GEMMS, 1)
+    return dh, dw
+
+
+def _bar(got, want):
+    err = (got.double() - want.double()).abs()
+    lim = 2e-2 + 2.0**-7 * want.double().abs()
+    assert (err <= lim).all(), (err.max().item(), (err - lim).max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,V,vchunk", [
+    (1, 256, 5003, 0),        # one token: 63 zero rows pad the reduction of d_weight
+    (17, 3584, 20011, 0),     # vocabulary that is no multiple of the 64-column blocks, hidden of 14 column tiles
+    (64, 384, 50257, 0),      # hidden of one and a half column tiles
+    (64, 128, 32000, 4096),   # eight chunks: the d_hidden partials of later chunks are added to the first chunk's
+    (65, 1024, 32000, 0),     # just past 64 tokens: the 128-position kernels
+    (100, 2048, 128256, 0),
+    (128, 512, 100003, 8192),
+    (128, 128, 300, 0),       # a hidden narrower than a tile, a vocabulary narrower than the K slices
+])
+def test_against_the_oracle_and_the_tile_kernels(T, H, V, vchunk, dtype):
+    tau = 0.8
+    h, w, y, g_lp, g_ent = _case(T, H, V, dtype, seed=T + H)
+    dh, dw = _run(h, w, y, tau, g_lp, g_ent, few=1, vchunk=vchunk)
+    dh_again, dw_again = _run(h, w, y, tau, g_lp, g_ent, few=1, vchunk=vchunk)
+    dh_tiles, dw_tiles = _run(h, w, y, tau, g_lp, g_ent, few=0, vchunk=vchunk)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    _bar(dh, rdh)
+    _bar(dw, rdw)
+    assert torch.equal(dh, dh_again) and torch.equal(dw, dw_again)  # fixed summation order
+    # the two code paths sum d_weight over the same tokens in fp32 and round once: equal up to one 16-bit ulp
+    ulp = 2.0**-7 if dtype == torch.bfloat16 else 2.0**-10
+    assert ((dw.float() - dw_tiles.float()).abs() <= 1e-6 + ulp * dw_tiles.float().abs()).all()
+    assert ((dh.float() - dh_tiles.float()).abs() <= 2e-3 + 2 * ulp * dh_tiles.float().abs()).all()
+
+
+@pytest.mark.parametrize("T", [40, 120])
+@pytest.mark.parametrize("pattern", ["none", "single", "sparse", "tail"])
+def test_tokens_without_upstream_gradient(T, pattern):
+    """The token list is built on the device; the streaming kernels read its length there: k-steps of d_weight
+    beyond it are skipped (those rows of the compact hidden copy are not initialised), d_hidden rows of skipped
+    tokens are exactly zero."""
+    H, V, tau = 512, 30011, 0.9
+    h, w, y, g_lp, g_ent = _case(T, H, V, torch.bfloat16, seed=7 + T)
+    keep = torch.zeros(T, dtype=torch.bool, device=DEV)
+    if pattern == "single":
+        keep[T // 2] = True
+    elif pattern == "sparse":
+        keep[::7] = True
+    elif pattern == "tail":
+        keep[T - 33:] = True
+    g_lp, g_ent = g_lp * keep, g_ent * keep
+    dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    _bar(dh, rdh)
+    _bar(dw, rdw)
+    assert torch.count_nonzero(dh[~keep]) == 0
+    if pattern == "none":
+        assert torch.count_nonzero(dw) == 0 and torch.count_nonzero(dh) == 0
+
+
+@pytest.mark.parametrize("T", [64, 128])
+def test_fp32_gradients(T):
+    """should_return_fp32_grad: the streaming kernels write the fp32 accumulators of d_weight; they round to what the
+    16-bit call returns and are closer to the oracle on average."""
+    H, V, tau = 1024, 50257, 1.0
+    h, w, y, g_lp, g_ent = _case(T, H, V, torch.bfloat16, seed=3)
+    dh32, dw32 = _run(h, w, y, tau, g_lp, g_ent, fp32_grad=True)
+    dh16, dw16 = _run(h, w, y, tau, g_lp, g_ent)
+    assert dh32.dtype == torch.float32 and dw32.dtype == torch.float32
+    assert torch.equal(dh32.bfloat16(), dh16)
+    # d_weight: the same accumulators, so equal after rounding, except on the rows of the labels, where the 16-bit call
+    # rounds twice (the softmax terms, then their sum with the one-hot terms that are added in fp32): one ulp of the
+    # result there, or half an ulp of the softmax terms where the two parts cancel (entries of 1e-4 off by 1e-6; bound 2e-4)
+    label_row = torch.zeros(V, dtype=torch.bool, device=DEV)
+    label_row[y] = True
+    assert torch.equal(dw32.bfloat16()[~label_row], dw16[~label_row])
+    assert ((dw32.bfloat16().float() - dw16.float()).abs() <= 2e-4 + 2.0**-7 * dw16.float().abs())[label_row].all()
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    assert (dw32 - rdw).abs().mean() < (dw16.float() - rdw).abs().mean()
+
+
+def test_full_vocabulary_config2_head():
+    """qwen2.5-7b head (H=3584, V=152064) at 64 tokens, the shape the few-token bench line is quoted on: both gradients
+    whole against the oracle."""
+    T, H, V, tau = 64, 3584, 152064, 1.0
+    h, w, y, g_lp, g_ent = _case(T, H, V, torch.bfloat16, seed=11)
+    dh, dw = _run(h, w, y, tau, g_lp, g_ent)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau)
+    _bar(dh, rdh)
+    _bar(dw, rdw)

@@ -712,3 +712,37 @@ def test_every_backward_method_runs_and_split_dlogits_m_raises():
             _run(h, w, y, tau, g_lp, g_ent)
     finally:
         kernels.set_backward_method(kernels.BackwardEnum._Split_Dlogits_N)
+
+
+@pytest.mark.parametrize("T", [700, 9001])  # the 32x32x16 path and the 16x16x32 path
+def test_should_return_fp32_grad_gives_the_fp32_accumulators(T):
+    """should_return_fp32_grad (verl/utils/kernel/kernels.py:1562-1567): the gradients leave as fp32 without the final
+    rounding to bf16.  They round to exactly what the default call returns (same accumulators, one rounding fewer), and
+    they are closer to the oracle than bf16 storage allows: wherever an entry is large enough for its bf16 spacing to
+    matter, the fp32 result must beat the bf16 one."""
+    from verl_amd.utils.kernel import kernels
+
+    H, V, tau = 256, 3001, 1.1
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=T)
+    lp, ent, mx, acc, eb = kernels.efficient_entropy_forward(h, w, y, 0, tau)
+    dh16, dw16 = kernels.efficient_entropy_backward(g_lp.float(), g_ent.float(), h, w, y, mx, acc, eb, 0, False, tau)
+    dh32, dw32 = kernels.efficient_entropy_backward(g_lp.float(), g_ent.float(), h, w, y, mx, acc, eb, 0, True, tau)
+    assert dh32.dtype == torch.float32 and dw32.dtype == torch.float32 and dh32.shape == (T, H) and dw32.shape == (V, H)
+    assert torch.equal(dh32.bfloat16(), dh16)
+    # d_weight: equal after rounding on every row that is nobody's label.  On a label's row the 16-bit call rounds
+    # twice: the GEMM's sum of the softmax terms first, then that plus the label entries, which are added in fp32
+    # (|entry| <= (|g_logprob| + 20 |g_entropy|) / tau per token); the first rounding is half an ulp of the softmax sum
+    label_row = torch.zeros(V, dtype=torch.bool, device=DEV)
+    label_row[y] = True
+    assert torch.equal(dw32.bfloat16()[~label_row], dw16[~label_row])
+    entry = torch.zeros(V, H, device=DEV)
+    entry.index_add_(0, y, ((g_lp.float().abs() + 20 * g_ent.float().abs()) / tau)[:, None] * h.float().abs())
+    slack = 2.0**-7 * dw16.float().abs() + 2.0**-8 * (dw32.abs() + entry)
+    assert ((dw32.bfloat16().float() - dw16.float()).abs() <= slack).all()
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    for g32, g16, want in ((dh32, dh16, rdh), (dw32, dw16, rdw)):
+        e32, e16 = (g32 - want).abs(), (g16.float() - want).abs()
+        assert e32.max() < 2e-2
+        assert e32.mean() < e16.mean()
+        big = want.abs() > 0.25 * want.abs().max()  # entries whose bf16 spacing is the dominant error of the bf16 result
+        assert e32[big].mean() < 0.6 * e16[big].mean(), (e32[big].mean().item(), e16[big].mean().item())

@@ -304,3 +304,112 @@ def test_packed_outputs_reference_assertions():
         fused_ppo_loss_packed(lp, ent, P, Rl, old[:, :2], adv[:, :2], mask[:, :2])
     loss, _ = fused_ppo_loss_packed(lp, None, P, Rl, old, adv, mask)  # entropy is optional as in fused_ppo_loss
     assert torch.isfinite(loss)
+
+
+class _ActorConfig:
+    """The fields of the reference's ActorConfig that ppo_loss reads (verl/workers/utils/losses.py:57-155)."""
+
+    def __init__(self, **kw):
+        self.clip_ratio, self.clip_ratio_low, self.clip_ratio_high, self.clip_ratio_c = 0.2, None, None, 3.0
+        self.entropy_coeff, self.loss_agg_mode, self.loss_scale_factor = 1e-3, "token-mean", None
+        self.use_kl_loss, self.kl_loss_coef, self.kl_loss_type = False, 0.01, "low_var_kl"
+        self.policy_loss = {"loss_mode": "vanilla"}
+        self.global_batch_info = {}
+        self.__dict__.update(kw)
+
+
+def _jagged(values, lens):
+    offsets = torch.cat([torch.zeros(1, dtype=torch.int64), torch.tensor(lens).cumsum(0)]).to(values.device)
+    return torch.nested.nested_tensor_from_jagged(values, offsets=offsets)
+
+
+@pytest.mark.parametrize("nested", [True, False])
+@pytest.mark.parametrize("globals_set", [False, True])
+def test_ppo_loss_entry_with_the_reference_signature(nested, globals_set):
+    """ppo_loss(config, model_output, data) on a nested (no-padding) batch and on a padded batch with attention_mask:
+    loss, gradients in packed order and every metric against the oracle's slice + loss; metric aggregation kinds as
+    verl/workers/utils/losses.py:71-84,124-126 (pg statistics MEAN; losses SUM once a global normaliser is set)."""
+    from verl_amd.utils.metric import AggregationType, Metric
+    from verl_amd.workers.utils.losses import ppo_loss
+
+    prompt, resp = [3, 1, 7, 2, 5], [5, 1, 12, 9, 2]
+    R = 12 if nested else 16
+    lp, ent, old, adv, ref, mask = _packed_case(prompt, resp, R, seed=11)
+    B, total = len(prompt), lp.numel()
+    ids = torch.arange(total, device=DEV)
+    data = {"response_mask": mask, "old_log_probs": old, "advantages": adv, "ref_log_prob": ref,
+            "dp_size": 2 if globals_set else 1, "batch_num_tokens": 77 if globals_set else None, "global_batch_size": None}
+    if nested:
+        data["prompts"] = _jagged(torch.arange(sum(prompt), device=DEV), prompt)
+        data["responses"] = _jagged(torch.arange(sum(resp), device=DEV), resp)
+        model_output = {"log_probs": _jagged(lp, [p + r for p, r in zip(prompt, resp)]), "entropy": None}
+    else:
+        Pw = 8
+        data["prompts"] = torch.zeros(B, Pw, dtype=torch.long, device=DEV)
+        data["responses"] = torch.zeros(B, R, dtype=torch.long, device=DEV)
+        am = torch.zeros(B, Pw + R, dtype=torch.long, device=DEV)
+        for b in range(B):
+            am[b, Pw - prompt[b] : Pw + resp[b]] = 1  # left-padded prompts, right-padded responses
+        data["attention_mask"] = am
+        model_output = {"log_probs": None, "entropy": None}
+    cfg = _ActorConfig(use_kl_loss=True, loss_agg_mode="token-mean")
+    lp1, ent1 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    if nested:
+        model_output["log_probs"] = _jagged(lp1, [p + r for p, r in zip(prompt, resp)])
+        model_output["entropy"] = _jagged(ent1, [p + r for p, r in zip(prompt, resp)])
+    else:
+        model_output["log_probs"], model_output["entropy"] = lp1, ent1
+    loss, metrics = ppo_loss(cfg, model_output, data)
+    loss.backward()
+    info = dict(dp_size=data["dp_size"], batch_num_tokens=data["batch_num_tokens"], global_batch_size=None, loss_scale_factor=None)
+    assert cfg.global_batch_info == info  # left on the config as the reference does (:70-73)
+    lp2, ent2 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    rloss, rmet = O.ppo_actor_loss(O.no_padding_2_padding(lp2, prompt, resp, R), O.no_padding_2_padding(ent2, prompt, resp, R), old, adv, mask,
+                                   clip_ratio=0.2, entropy_coeff=1e-3, loss_agg_mode="token-mean", ref_log_prob=ref,
+                                   kl_loss_type="low_var_kl", kl_loss_coef=0.01, **info)
+    rloss.backward()
+    torch.testing.assert_close(loss, rloss, atol=1e-6, rtol=1e-5)
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-8, rtol=1e-5)
+    torch.testing.assert_close(ent1.grad, ent2.grad, atol=1e-9, rtol=1e-5)
+    want = AggregationType.SUM if globals_set else AggregationType.MEAN
+    assert set(metrics) == {"actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower", "actor/pg_loss", "actor/entropy_loss", "kl_loss", "kl_coef"}
+    for k in ("actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower"):
+        assert isinstance(metrics[k], Metric) and metrics[k].aggregation == AggregationType.MEAN
+    for k in ("actor/pg_loss", "actor/entropy_loss", "kl_loss"):
+        assert metrics[k].aggregation == want
+    for k, v in metrics.items():
+        if k != "kl_coef":
+            assert v.aggregate() == pytest.approx(rmet[k], rel=1e-5, abs=1e-6), k
+    assert metrics["kl_coef"] == 0.01
+
+
+def test_ppo_loss_entry_refuses_what_has_no_fused_kernel():
+    from verl_amd.workers.utils.losses import ppo_loss
+
+    prompt, resp, R = [2, 1], [3, 1], 3
+    lp, ent, old, adv, ref, mask = _packed_case(prompt, resp, R, seed=12)
+    data = {"prompts": _jagged(torch.arange(3, device=DEV), prompt), "responses": _jagged(torch.arange(4, device=DEV), resp),
+            "response_mask": mask, "old_log_probs": old, "advantages": adv, "dp_size": 1, "batch_num_tokens": None, "global_batch_size": None}
+    with pytest.raises(NotImplementedError, match="only 'vanilla'"):
+        ppo_loss(_ActorConfig(policy_loss={"loss_mode": "gspo"}), {"log_probs": lp}, data)
+    with pytest.raises(NotImplementedError, match="sampler-correction"):
+        ppo_loss(_ActorConfig(), {"log_probs": lp, "sc_correction": lp}, data)
+    loss, metrics = ppo_loss(_ActorConfig(), {"log_probs": lp}, data)  # no entropy, no KL: just the policy loss
+    assert torch.isfinite(loss) and "actor/entropy_loss" not in metrics and "kl_loss" not in metrics
+
+
+def test_deprecated_compute_policy_loss_name():
+    """core_algos.py:1210-1282: positional cliprange arguments, a 4-tuple back, FutureWarning like the reference's decorator."""
+    from verl_amd.trainer.ppo import core_algos as C
+
+    lp, _, old, adv, mask = _case(6, 40, seed=21, spread=0.6)
+    with pytest.warns(FutureWarning, match="compute_policy_loss_vanilla"):
+        pg, clipfrac, kl, clipfrac_lower = C.compute_policy_loss(old, lp, adv, mask, 0.2, 0.1, 0.3, 2.5, "seq-mean-token-mean")
+    r, m = O.policy_loss_vanilla(old, lp, adv, mask, "seq-mean-token-mean", 0.2, clip_ratio_low=0.1, clip_ratio_high=0.3, clip_ratio_c=2.5)
+    torch.testing.assert_close(pg, r, atol=1e-6, rtol=1e-5)
+    assert clipfrac.item() == pytest.approx(m["actor/pg_clipfrac"], rel=1e-5, abs=1e-7)
+    assert kl.item() == pytest.approx(m["actor/ppo_kl"], rel=1e-5, abs=1e-7)
+    assert clipfrac_lower.item() == pytest.approx(m["actor/pg_clipfrac_lower"], rel=1e-5, abs=1e-7)
+    assert C.get_policy_loss_fn("vanilla") is C.compute_policy_loss_vanilla
+    with pytest.raises(ValueError, match="Unsupported loss mode: gpg"):
+        C.get_policy_loss_fn("gpg")

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LCE_LIBRARY_PATH") or os.path.join(_HERE, "lib", "liblce_gfx950.so")
 
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # every symbol include/lce_abi.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -23,6 +23,10 @@ SYMBOLS = {
     "lce_forward_static": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p]),
     "lce_backward_workspace_bytes": (_sz, [_i64, _i64, _i64, _i, _i64]),
     "lce_backward": (
+        _i,
+        [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _p],
+    ),
+    "lce_backward_f32": (
         _i,
         [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _p],
     ),

@@ -219,17 +219,19 @@ __global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm lt, co
 // One workgroup per sorted position; only the first position of a run works.  Runs after the d_weight GEMMs:
 // the rows are read back in the output dtype (rounded once by the GEMM that wrote the softmax terms, which are
 // small next to the one-hot sums on all but a few rows) and rounded once more with the sum added in fp32.
-template <typename T>
+// (TOUT: the dtype d_weight is returned in, the input dtype or fp32)
+template <typename T, typename TOUT>
 __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys, const int* toks, int n_items, LabelTerm lt, const T* h,
-                                                            int64_t ldh, int64_t H, T* dW) {
+                                                            int64_t ldh, int64_t H, TOUT* dW) {
   constexpr int N = 16 / (int)sizeof(T);
   typedef typename VecOf<T, N>::type vec_t;
   const int i = blockIdx.x;
   const uint32_t key = keys[i];
   if (key == kNoRow || (i > 0 && keys[i - 1] == key)) return;
-  T* row = dW + (int64_t)key * H;
+  TOUT* row = dW + (int64_t)key * H;
   for (int64_t c = (int64_t)threadIdx.x * N; c < H; c += 256 * N) {
-    const vec_t cur = *reinterpret_cast<const vec_t*>(row + c);
+    typedef typename VecOf<TOUT, N>::type ovec_t;
+    const ovec_t cur = *reinterpret_cast<const ovec_t*>(row + c);
     float acc[N];
 #pragma unroll
     for (int e = 0; e < N; ++e) acc[e] = 0.f;
@@ -242,7 +244,10 @@ __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys
     }
 #pragma unroll
     for (int e = 0; e < N; ++e) acc[e] += (float)cur[e];
-    store_run<T, N>(row + c, acc);
+    ovec_t out;
+#pragma unroll
+    for (int e = 0; e < N; ++e) out[e] = (TOUT)acc[e];
+    *reinterpret_cast<ovec_t*>(row + c) = out;
   }
 }
 

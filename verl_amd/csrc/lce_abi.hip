@@ -13,6 +13,7 @@
 #include "label_rows.hpp"
 #include "lce_kernels.hpp"
 #include "lce_kernels16.hpp"
+#include "few_tokens.hpp"
 
 using namespace lce;
 
@@ -29,9 +30,12 @@ thread_local char g_err[512] = "";
 // Defaults of the 32x32x16 loops: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it
 // only up to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed (the XCD's
 // workgroups drift apart and lose L2 sharing), so large forwards keep the 2-stage ring.  Beyond 8192 tokens 16-bit
-// inputs run the four-wave 16x16x32 loop (variant 5) in both directions.
+// inputs run the four-wave 16x16x32 loop (variant 5) in both directions (thresholds below).
 constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2, kVariantCore16 = 5;
-constexpr int64_t kCore16MinTokens = 8192;  // variant 5 is the default above this many tokens
+// variant 5 is the default above these token counts (measured at H=3584, V=152064: the forward gains 2-6% from 1024
+// tokens on; forward + backward breaks even at 4096 tokens, where the 32x32x16 path still saves the transpose of W, and
+// gains 4.5% at 8192)
+constexpr int64_t kCore16MinTokensFwd = 512, kCore16MinTokensBwd = 4096;
 struct Tuning {
   int variant_fwd = kDefaultVariantFwd, variant_bwd = kDefaultVariantBwd;
   bool variant_forced = false;   // lce_set_variant was called: no size-based choice of the tile
@@ -43,6 +47,7 @@ struct Tuning {
   int ds_strip = 1;              // vocabulary tiles per workgroup of the d_logits pass on the 16x16x32 loop
   int dw_transposed_reads = 1;   // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
+  int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
 };
 std::mutex g_tuning_mu;
 Tuning g_tuning;
@@ -53,7 +58,7 @@ Tuning tuning_snapshot() {
 // the mainloop variant a backward over T tokens of `esz`-byte elements runs with
 int bwd_variant(const Tuning& tu, int64_t T, size_t esz) {
   if (tu.variant_forced) return tu.variant_bwd;
-  return (esz == 2 && T > kCore16MinTokens) ? kVariantCore16 : kDefaultVariantBwd;
+  return (esz == 2 && T > kCore16MinTokensBwd) ? kVariantCore16 : kDefaultVariantBwd;
 }
 
 int fail(int code, const char* fmt, ...) {
@@ -130,7 +135,7 @@ GemmArgs<typename Cfg::TIN> make_gemm_args(const typename Cfg::TIN* A, int64_t l
   p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.M = M; p.N = N; p.K = K;
   p.Cf = Cf; p.ldcf = ldcf; p.Ct = Ct; p.ldct = ldct; p.out_mode = out_mode;
   p.ksplit = 1; p.kslice = K; p.cf_split_stride = 0;
-  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1; p.tn = 0; p.b_rows_valid = 0;
+  p.m_dev = nullptr; p.k_dev = nullptr; p.k_gran = 1; p.tn = 0; p.b_rows_valid = 0; p.perm_rows = 0;
   const int tm = (int)((M + Cfg::BM - 1) / Cfg::BM), tn = (int)((N + Cfg::BN - 1) / Cfg::BN);
   p.map = TileMap::make(tm, tn, block_rows(tm), 1);
   return p;
@@ -156,6 +161,23 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
   return check_launch("gemm_nt_kernel");
 }
 
+// Vocabulary splits of the forward with 256-token tiles.  A workgroup owns one (token tile, split) pair and walks the
+// split's vocabulary tiles itself, so the launch takes ceil(workgroups / CUs) rounds of ceil(tiles / splits) tiles
+// each: pick the split count with the fewest tile-times (ties: fewer splits, fewer partials to merge).  With 48 token
+// tiles (12288 tokens) the former rule, eight splits, gave 384 workgroups = two rounds of 75 tiles; sixteen splits give
+// three rounds of 38.
+constexpr int kNumCUs = 256;
+int forward_splits_256(int ntt, int nvt) {
+  int best = 1;
+  int64_t best_cost = -1;
+  for (int S = 1; S <= 256 && S <= nvt; ++S) {
+    const int64_t rounds = ((int64_t)ntt * S + kNumCUs - 1) / kNumCUs;
+    const int64_t cost = rounds * ((nvt + S - 1) / S);
+    if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = S; }
+  }
+  return best;
+}
+
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                  int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* logprobs, float* entropy,
@@ -169,7 +191,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   // splits: enough workgroups to fill 256 CUs, in multiples of the XCD block width
   const int br = block_rows(ntt), bc = 32 / br;
   const int nrb = (ntt + br - 1) / br;
-  int S = bc * ((8 + nrb - 1) / nrb);
+  int S = Cfg::BN == 256 ? forward_splits_256(ntt, nvt) : bc * ((8 + nrb - 1) / nrb);
   if (S > nvt) S = nvt;
   // The narrow token tiles serve the HBM-bound case (up to 128 tokens: one streaming read of W).  There each
   // split takes one contiguous range of rows, the same length for all, instead of whole tiles dealt round robin
@@ -245,9 +267,9 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
 }
 
 // upper bound of the number of vocabulary splits forward_impl picks, over the token-tile widths in use
-int forward_splits_upper_bound(int64_t T) {
-  int best = 1;
-  for (int bn = 64; bn <= 256; bn <<= 1) {
+int forward_splits_upper_bound(int64_t T, int64_t V) {
+  int best = forward_splits_256((int)((T + 255) / 256), (int)((V + 255) / 256));
+  for (int bn = 64; bn <= 128; bn <<= 1) {
     const int ntt = (int)((T + bn - 1) / bn);
     const int br = block_rows(ntt), bc = 32 / br, nrb = (ntt + br - 1) / br;
     const int S = bc * ((8 + nrb - 1) / nrb);
@@ -265,6 +287,7 @@ struct BwdLayout {
   bool tn;     // the gradient GEMMs read dS, a compact copy of hidden and W as they lie in memory (transposing LDS
                // reads for the K-major operands): no dS^T, no h^T
   bool tn_dh;  // ... and the d_hidden GEMM reads W as it lies in memory too: no W^T
+  bool few;    // at most 128 tokens, 16-bit inputs: both gradient GEMMs run as the streaming kernels of few_tokens.hpp
 };
 
 // The d_weight GEMM can take the token-major d_logits and hidden as they are (transposing LDS reads exist
@@ -276,6 +299,8 @@ bool dw_transposed_reads(const Tuning& tu, int variant, size_t esz) { return esz
 // vocabulary chunk.  With few tokens one such tile takes longer than a CU's share of the whole launch
 // (d_logits tiles + both GEMMs) and would set the launch's duration; the K range is then cut into
 // slices, with an fp32 partial each, so that a tile takes at most about half of that share.
+int64_t few_tile_columns(int64_t T) { return T <= 64 ? FewShape<64>::HW : FewShape<128>::HW; }
+
 int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
   const int64_t ntt = (T + 255) / 256, nht = (H + 255) / 256, nvt = (vchunk + 255) / 256;
   const int64_t work = ntt * nvt * H + nvt * nht * ntt * 256 + ntt * nht * vchunk;  // in K elements of 256x256 tiles
@@ -298,6 +323,17 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
   L.ksplit = tu.dh_ksplit > 0 ? tu.dh_ksplit : dh_ksplit(T, H, vchunk);
+  L.few = tu.few_token_gemms && L.tn && T <= 128;
+  if (L.few) {
+    // K slices of the streaming d_hidden kernel: its workgroups (column tiles x slices) fill the chip about twice
+    // over, which is what two resident workgroups per CU take in one round; at least 1024 columns per slice
+    const int64_t n_ht = (H + few_tile_columns(T) - 1) / few_tile_columns(T);
+    int64_t ks = (2 * kNumCUs) / n_ht;
+    const int64_t most = (vchunk + 1023) / 1024;
+    ks = ks > most ? most : ks;
+    L.ksplit = tu.dh_ksplit > 0 ? tu.dh_ksplit : (int)(ks < 1 ? 1 : ks > 40 ? 40 : ks);
+    L.tn_dh = true;  // W is read in place
+  }
   L.nchunks = (int)((V + vchunk - 1) / vchunk);
   // Row strides are kept away from large powers of two (+128 bytes): with a 16 or 32 KiB stride the
   // 256 rows of an operand tile would all fall into the same L2 channel.
@@ -353,10 +389,23 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
 // tile, which is what the size query assumes; the launch passes the tile variant's wave-tile sizes).
 BwdLayout bwd_layout(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
+    // Upper bound of the whole workspace: a quarter of one [T, V] tile plus one fp32 [V, H].  Below it the default is
+    // a chunk of 8192 columns, or wider while one d_logits buffer stays within 256 MiB (few tokens: the whole vocabulary
+    // in one chunk, which saves a pass over W per chunk).  Measured at config 2 on the 16x16x32 loop: 8192 columns cost
+    // 0.4% against the widest chunk the bound allows (56.2 against 56.0 ms per step) with 0.9 instead of 2.9 GiB of
+    // workspace; 4096 columns cost 6%.  A byte budget (LCE_OPT_WORKSPACE_BUDGET) replaces the default rule: the widest
+    // chunk whose workspace fits it, but never fewer than 2048 columns.
     double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
-    if (tu.ws_budget > 0 && (double)tu.ws_budget < gate) gate = (double)tu.ws_budget;
     vchunk = round_up(V, 256);
+    if (tu.ws_budget > 0) {
+      if ((double)tu.ws_budget < gate) gate = (double)tu.ws_budget;
+    } else {
+      int64_t cols = (((int64_t)256 << 20) / (T * (int64_t)esz)) / 256 * 256;
+      if (cols < 8192) cols = 8192;
+      if (cols < vchunk) vchunk = cols;
+    }
     while (vchunk > 2048 && (double)bwd_layout_for(tu, T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
+    if (vchunk < 2048) vchunk = 2048;
     const int64_t n = (V + vchunk - 1) / vchunk;
     vchunk = round_up((V + n - 1) / n, 256);
   }
@@ -376,11 +425,24 @@ int launch_ds_few_tokens(DsArgs<typename Cfg::TIN> d, int64_t T, int nvt, hipStr
   return check_launch("lce_bwd_ds_kernel");
 }
 
+// Both gradient GEMMs of one vocabulary chunk of a backward with at most 128 tokens, as one launch of the streaming
+// kernels (few_tokens.hpp): d_weight rows of the chunk in the output dtype, d_hidden as L.ksplit fp32 partials.
+template <typename Cfg, typename TOUT, int KT>
+int launch_few_gemms(const FewArgs<typename Cfg::TIN>& q, hipStream_t st) {
+  typedef typename Cfg::TIN TIN;
+  typedef FewShape<KT> S;
+  const int n_ht = (int)((q.H + S::HW - 1) / S::HW);
+  auto kern = lce_bwd_few_kernel<TIN, TOUT, KPerm<Cfg>, KT>;
+  allow_lds(kern, S::LDS_BYTES);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(q.n_dw + n_ht * q.ksplit)), dim3(256), S::LDS_BYTES, st, q);
+  return check_launch("lce_bwd_few_kernel");
+}
+
 template <typename Cfg>
 int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                   int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
                   const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
-                  typename Cfg::TIN* d_hidden, typename Cfg::TIN* d_weight, char* ws, int64_t vchunk, hipStream_t st,
+                  void* d_hidden, void* d_weight, bool grads_f32, char* ws, int64_t vchunk, hipStream_t st,
                   int64_t vocab_offset, const Tuning& tu) {
   // vocab_offset: W is the shard [vocab_offset, vocab_offset + V) of a larger vocabulary (labels are global ids)
   typedef typename Cfg::TIN TIN;
@@ -517,44 +579,69 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       const int64_t vrows = (V - v0) < L.vchunk ? (V - v0) : L.vchunk;
       // fp32 d_hidden partial [T][H] (+)= dS[T][Kc] . W[v0 : v0 + Kc][H]  (rows = listed tokens)
       const int64_t kc = round_up(vrows, KPerm<Cfg>::GV);
-      if (L.tn_dh) {
-        // W as it lies in memory (K-major for this product), fetched with transposing LDS reads
-        p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, W + v0 * ldw, ldw, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
-        p.gh.tn = 2;
-        p.gh.b_rows_valid = vrows;
-      } else {
-        // Wt = this chunk of W, transposed just before the launch (the previous launch, the last reader of the
-        // buffer, is complete by then)
-        ProfScope prof(PC_TRANSPOSE, st);
-        hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((kc + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
-                           st, W + v0 * ldw, ldw, vrows, H, Wt, L.ldWt, kc);
-        if ((rc = check_launch("transpose W"))) return rc;
-        p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+      bool few_done = false;  // (then nothing is left for the tile kernels but the d_logits of the next chunk)
+      if constexpr (sizeof(TIN) == 2) {
+        if (L.few) {
+          FewArgs<TIN> q;
+          q.dS = dS[cc & 1]; q.ldS = L.ldS; q.Ht = Ht; q.ldHt = L.ldHt; q.W = W + v0 * ldw; q.ldw = ldw;
+          q.vrows = vrows; q.ucols = kc; q.H = H;
+          q.kt = T <= 64 ? 64 : 128; q.nt = (int)T; q.n_rows = n_rows;
+          q.dW = grads_f32 ? static_cast<void*>(static_cast<float*>(d_weight) + v0 * H) : static_cast<void*>(static_cast<TIN*>(d_weight) + v0 * H);
+          q.dHp = dHacc; q.part_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
+          q.ksplit = L.ksplit; q.kslice = round_up((q.ucols + L.ksplit - 1) / L.ksplit, 64);
+          q.accumulate = cc == 0 ? 0 : 1;
+          q.n_dw = (int)(q.ucols / 64);
+          ProfScope prof(PC_BWD_CHUNK, st);
+          if (T <= 64) rc = grads_f32 ? launch_few_gemms<Cfg, float, 64>(q, st) : launch_few_gemms<Cfg, TIN, 64>(q, st);
+          else rc = grads_f32 ? launch_few_gemms<Cfg, float, 128>(q, st) : launch_few_gemms<Cfg, TIN, 128>(q, st);
+          if (rc) return rc;
+          few_done = true;
+        }
       }
-      p.gh.m_dev = n_rows;
-      if (L.ksplit > 1) {
-        p.gh.ksplit = L.ksplit;
-        p.gh.kslice = round_up((kc + L.ksplit - 1) / L.ksplit, Cfg::BK);
-        p.gh.cf_split_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
-      }
-      // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T
-      if (L.tn) {
-        // d_weight[v0 : v0 + vrows][H] = dS[tokens][vrows]^T . hidden[tokens][H], both operands K-major
-        p.gw = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Ht, L.ldHt, vrows, H, round_up(T, 64), nullptr, 0, d_weight + v0 * H, H, 2);
-        p.gw.tn = 1;
-        p.gw.k_dev = n_rows; p.gw.k_gran = 64;
-      } else {
-        p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, nullptr, 0, d_weight + v0 * H, H, 2);
-        p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
-      }
-      p.n_gh = p.gh.map.total * L.ksplit;
-      p.n_gw = p.gw.map.total;
-      if (p.gh.kslice > p.gw.K) {  // longer tiles go first
-        std::swap(p.gh, p.gw);
-        std::swap(p.n_gh, p.n_gw);
-        swapped = true;
+      if (!few_done) {
+        if (L.tn_dh) {
+          // W as it lies in memory (K-major for this product), fetched with transposing LDS reads
+          p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, W + v0 * ldw, ldw, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+          p.gh.tn = 2;
+          p.gh.b_rows_valid = vrows;
+        } else {
+          // Wt = this chunk of W, transposed just before the launch (the previous launch, the last reader of the
+          // buffer, is complete by then)
+          ProfScope prof(PC_TRANSPOSE, st);
+          hipLaunchKernelGGL((transpose_pad_kernel<Cfg, 2>), dim3((unsigned)((kc + 127) / 128), (unsigned)((H + 63) / 64)), dim3(256), 0,
+                             st, W + v0 * ldw, ldw, vrows, H, Wt, L.ldWt, kc);
+          if ((rc = check_launch("transpose W"))) return rc;
+          p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
+        }
+        p.gh.m_dev = n_rows;
+        if (L.ksplit > 1) {
+          p.gh.ksplit = L.ksplit;
+          p.gh.kslice = round_up((kc + L.ksplit - 1) / L.ksplit, Cfg::BK);
+          p.gh.cf_split_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
+        }
+        // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T   (written in the input dtype, or as fp32)
+        float* dw_f32 = grads_f32 ? static_cast<float*>(d_weight) + v0 * H : nullptr;
+        TIN* dw_t = grads_f32 ? nullptr : static_cast<TIN*>(d_weight) + v0 * H;
+        if (L.tn) {
+          // d_weight[v0 : v0 + vrows][H] = dS[tokens][vrows]^T . hidden[tokens][H], both operands K-major
+          p.gw = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Ht, L.ldHt, vrows, H, round_up(T, 64), dw_f32, H, dw_t, H, grads_f32 ? 0 : 2);
+          p.gw.tn = 1;
+          p.gw.perm_rows = 1;
+          p.gw.k_dev = n_rows; p.gw.k_gran = 64;
+        } else {
+          p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, dw_f32, H, dw_t, H, grads_f32 ? 0 : 2);
+          p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
+        }
+        p.n_gh = p.gh.map.total * L.ksplit;
+        p.n_gw = p.gw.map.total;
+        if (p.gh.kslice > p.gw.K) {  // longer tiles go first
+          std::swap(p.gh, p.gw);
+          std::swap(p.n_gh, p.n_gw);
+          swapped = true;
+        }
       }
     }
+    if (p.n_gw + p.n_gh + p.n_ds == 0) continue;
     if (tu.split_bwd) {
       const int n[3] = {p.n_gw, p.n_gh, p.n_ds};
       const int cls[3] = {swapped ? PC_GEMM_DH : PC_GEMM_DW, swapped ? PC_GEMM_DW : PC_GEMM_DH, PC_BWD_DS};
@@ -587,16 +674,25 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     ProfScope prof(PC_DH_FINISH, st);
     int64_t blocks = (T * (H / 4) + 255) / 256;
     if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(dh_finish_kernel<TIN>, dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit,
-                       (int64_t)(align256((size_t)T * H * 4) / 4), inv, T, H, d_hidden, lt, W, ldw);
+    const int64_t part_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
+    if (grads_f32)
+      hipLaunchKernelGGL((dh_finish_kernel<TIN, float>), dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit, part_stride, inv, T, H,
+                         static_cast<float*>(d_hidden), lt, W, ldw);
+    else
+      hipLaunchKernelGGL((dh_finish_kernel<TIN, TIN>), dim3((unsigned)blocks), dim3(256), 0, st, dHacc, L.ksplit, part_stride, inv, T, H,
+                         static_cast<TIN*>(d_hidden), lt, W, ldw);
     if ((rc = check_launch("dh_finish_kernel"))) return rc;
   }
   if (L.sort_items) {
     // one-hot part of d_weight: every chunk's rows hold their softmax terms by now
     ProfScope prof(PC_LABEL_ROWS, st);
     const int res = L.sort_passes & 1;
-    hipLaunchKernelGGL(dw_label_rows_kernel<TIN>, dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h, ldh, H,
-                       d_weight);
+    if (grads_f32)
+      hipLaunchKernelGGL((dw_label_rows_kernel<TIN, float>), dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h,
+                         ldh, H, static_cast<float*>(d_weight));
+    else
+      hipLaunchKernelGGL((dw_label_rows_kernel<TIN, TIN>), dim3(L.sort_items), dim3(256), 0, st, skeys[res], svals[res], L.sort_items, lt, h,
+                         ldh, H, static_cast<TIN*>(d_weight));
     if ((rc = check_launch("dw_label_rows_kernel"))) return rc;
   }
   return LCE_OK;
@@ -621,17 +717,17 @@ template <template <typename> class Vt>
 int dispatch_dtype_backward(int dtype, const void* h, int64_t ldh, const void* W, int64_t ldw, const int64_t* labels,
                             int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* mx,
                             const float* ac, const float* eb, const float* glp, const float* gent, void* dh, void* dw,
-                            char* ws, int64_t vchunk, hipStream_t st, int64_t vocab_offset, const Tuning& tu) {
+                            bool grads_f32, char* ws, int64_t vchunk, hipStream_t st, int64_t vocab_offset, const Tuning& tu) {
   if (dtype == LCE_DTYPE_BF16)
     return backward_impl<typename Vt<bf16_t>::Cfg>((const bf16_t*)h, ldh, (const bf16_t*)W, ldw, labels, T, H, V, temperature,
-                                                   reduction, mx, ac, eb, glp, gent, (bf16_t*)dh, (bf16_t*)dw, ws, vchunk, st,
+                                                   reduction, mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st,
                                                    vocab_offset, tu);
   if (dtype == LCE_DTYPE_F16)
     return backward_impl<typename Vt<f16_t>::Cfg>((const f16_t*)h, ldh, (const f16_t*)W, ldw, labels, T, H, V, temperature,
-                                                  reduction, mx, ac, eb, glp, gent, (f16_t*)dh, (f16_t*)dw, ws, vchunk, st,
+                                                  reduction, mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st,
                                                   vocab_offset, tu);
   return backward_impl<typename Vt<float>::Cfg>((const float*)h, ldh, (const float*)W, ldw, labels, T, H, V, temperature,
-                                                reduction, mx, ac, eb, glp, gent, (float*)dh, (float*)dw, ws, vchunk, st, vocab_offset, tu);
+                                                reduction, mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st, vocab_offset, tu);
 }
 
 template <template <typename> class Vt>
@@ -737,6 +833,7 @@ int lce_set_option(int key, int64_t value) {
       if (value < 1 || value > 64) return fail(LCE_E_ARG, "LCE_OPT_DLOGITS_STRIP takes 1..64");
       t.ds_strip = (int)value;
       return LCE_OK;
+    case LCE_OPT_FEW_TOKEN_GEMMS: t.few_token_gemms = value != 0; return LCE_OK;
     case LCE_OPT_WORKSPACE_BUDGET:
       if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_WORKSPACE_BUDGET takes a byte count (0 = the built-in default)");
       t.ws_budget = value;
@@ -775,9 +872,9 @@ int lce_profile_read(double* total_ms, int64_t* launches, int reset) {
 }
 
 size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
-  (void)H; (void)V; (void)dtype;
+  (void)H; (void)dtype;
   if (T <= 0) return 256;
-  return align256((size_t)forward_splits_upper_bound(T) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
+  return align256((size_t)forward_splits_upper_bound(T, V > 0 ? V : 1) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
 }
 
 // shared body of lce_forward and lce_forward_shard
@@ -804,7 +901,7 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
   if (!tu.variant_forced && T <= 64) return LCE_FWD(VariantT64);
   if (!tu.variant_forced && T <= 128) return LCE_FWD(VariantT128);
   if (!tu.variant_forced && T <= 512) return LCE_FWD(Variant1);  // W (the A operand) streams from HBM: give it the early slot
-  if (!tu.variant_forced && esize(dtype) == 2 && T > kCore16MinTokens) return LCE_FWD(Variant5);
+  if (!tu.variant_forced && esize(dtype) == 2 && T > kCore16MinTokensFwd) return LCE_FWD(Variant5);
   // the split ring: measured 4-7% faster than the 2-stage ring up to 8192 tokens, equal (+-1%) beyond, and
   // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
   if (!tu.variant_forced && (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)))
@@ -894,14 +991,14 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
                           int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
                           const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                           void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
-                          void* stream, int64_t vocab_offset) {
+                          void* stream, int64_t vocab_offset, bool grads_f32 = false) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const size_t esz = esize(dtype);
   if (!d_weight) return fail(LCE_E_ARG, "null d_weight");
   if (T == 0) {
-    const int64_t words = (int64_t)((size_t)V * H * esz / 4);
+    const int64_t words = (int64_t)((size_t)V * H * (grads_f32 ? 4 : esz) / 4);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<uint32_t*>(d_weight), words);
     return check_launch("fill_zero_kernel");
   }
@@ -912,7 +1009,7 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
   const size_t need = bwd_layout(tu, T, H, V, esz, vchunk).total + 256;
   if (!workspace || workspace_bytes < need) return fail(LCE_E_WORKSPACE, "backward workspace too small: %zu < %zu", workspace_bytes, need);
   char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
-#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, ws, vchunk, st, vocab_offset, tu)
+#define LCE_BWD(Vt) dispatch_dtype_backward<Vt>(dtype, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum, accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, grads_f32, ws, vchunk, st, vocab_offset, tu)
   switch (bwd_variant(tu, T, esz)) {
     case 1: return LCE_BWD(Variant1);
     case 2: return LCE_BWD(Variant2);
@@ -931,6 +1028,14 @@ int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ld
                  void* stream) {
   return backward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, maximum, accumulate, entropy_b,
                         dlogprobs, dentropy, d_hidden, d_weight, workspace, workspace_bytes, vchunk, stream, 0);
+}
+
+int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T, int64_t H,
+                     int64_t V, int dtype, float temperature, int reduction, const float* maximum, const float* accumulate,
+                     const float* entropy_b, const float* dlogprobs, const float* dentropy, float* d_hidden, float* d_weight,
+                     void* workspace, size_t workspace_bytes, int64_t vchunk, void* stream) {
+  return backward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, maximum, accumulate, entropy_b,
+                        dlogprobs, dentropy, d_hidden, d_weight, workspace, workspace_bytes, vchunk, stream, 0, true);
 }
 
 int lce_backward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,

@@ -556,6 +556,7 @@ struct GemmArgs {
   // epilogue leaves in KPerm::vocab order: row u of the tile is written to row KPerm::vocab_at(u) of C
   int tn;  // 0 NT (gemm_tile); 1 both operands K-major (gemm_tn_tile); 2 only B K-major, its rows in KPerm::vocab order (gemm_nb_tile)
   int64_t b_rows_valid;  // tn == 2: rows of B that exist (K may be rounded up beyond them; A is zero there)
+  int perm_rows;  // tn == 1 with fp32 output: row u of the tile goes to row KPerm::vocab_at(u) of Cf as well (out_mode 2 always does)
 };
 
 template <typename Cfg, int MODE, bool EDGE>
@@ -655,7 +656,7 @@ LCE_DEV void gemm_tn_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x16
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int u = acc_row(i, r, hh);  // row inside the wave tile
-        const int um = MODE == 2 ? (int)KPerm<PermCfg>::vocab_at(u) : u;
+        const int um = (MODE == 2 || p.perm_rows) ? (int)KPerm<PermCfg>::vocab_at(u) : u;
         const int64_t m = m0 + wave_m * Cfg::WM + um;
         if (EDGE && m >= p.M) continue;
         if (MODE == 2) p.Ct[m * p.ldct + n] = (TIN)acc[i][j][r];
@@ -824,8 +825,8 @@ struct LabelTerm {
 // without `inv`), or zeros where inv[t] < 0 (token without upstream gradient).  The sum runs in the
 // fixed order s = 0, 1, ..., so the result does not depend on scheduling.  H a multiple of 4.
 // With a label term, G_t * W[label_t][:] is added in fp32 before the one rounding.
-template <typename T>
-__global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, T* out,
+template <typename T, typename TOUT>
+__global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, TOUT* out,
                                  LabelTerm lt, const T* W, int64_t ldw) {
   const int64_t per_row = H / 4, n = ntok * per_row;
   for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += (int64_t)gridDim.x * blockDim.x) {
@@ -849,8 +850,8 @@ __global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const
         }
       }
     }
-    T* dst = out + t * H + c;
-    dst[0] = (T)a.x; dst[1] = (T)a.y; dst[2] = (T)a.z; dst[3] = (T)a.w;
+    TOUT* dst = out + t * H + c;
+    dst[0] = (TOUT)a.x; dst[1] = (TOUT)a.y; dst[2] = (TOUT)a.z; dst[3] = (TOUT)a.w;
   }
 }
 

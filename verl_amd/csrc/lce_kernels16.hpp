@@ -219,7 +219,7 @@ LCE_DEV void ds16_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x4_t (&a
   for (int j = 0; j < NB; ++j) {
     const float lse2 = tc[j][0], C0 = tc[j][1], C1 = tc[j][2], G = tc[j][3];
     // the label's entry: block pair rel / 32, lane group (rel / 4) % 4, value 4 ((rel / 16) % 2) + rel % 4 of the run
-    const int rel = LABEL ? lab[j] - (int)p.lab0 - vloc0 : -1;
+    const int rel = (LABEL && p.label_outside != 1) ? lab[j] - (int)p.lab0 - vloc0 : -1;  // (1: the tiles hold the softmax terms only)
     const int own_ip = (rel >= 0 && rel < Cfg::WM && ((rel >> 2) & 3) == g4) ? rel >> 5 : -1;
     const int own_q = ((rel >> 4) & 1) * 4 + (rel & 3);
     const int64_t tok = tok0 + j * 16 + l16;
@@ -418,7 +418,7 @@ LCE_DEV void gemm16_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, cha
 #pragma unroll
   for (int j = 0; j < Cfg::NB; ++j) {
     const int u = g.wave_n * Cfg::WN + j * 16 + (g.lane & 15);  // row inside the tile, in the operand's column order
-    const int64_t m = m0 + (p.out_mode == 2 ? (int64_t)KPerm<PermCfg>::vocab_at(u) : (int64_t)u);
+    const int64_t m = m0 + ((p.out_mode == 2 || p.perm_rows) ? (int64_t)KPerm<PermCfg>::vocab_at(u) : (int64_t)u);
     if (m >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < Cfg::NB; ++i) {

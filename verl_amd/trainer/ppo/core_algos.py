@@ -1,15 +1,17 @@
 """The two functions of the reference's ``verl/trainer/ppo/core_algos.py`` that sit directly behind the fused head:
-``agg_loss`` (``:1140-1206``) and ``compute_policy_loss_vanilla`` (``:1286-1376``), with the reference's names,
+``agg_loss`` (``:1140-1206``) and ``compute_policy_loss_vanilla`` (``:1286-1376``; its deprecated predecessor
+``compute_policy_loss``, ``:1210-1282``, and the registry lookup ``get_policy_loss_fn``, ``:70-85``), with the reference's names,
 argument order and return values, computed by the HIP PPO-loss kernels (``lce_ppo_loss``).  Both are
 differentiable; nothing here runs on the CPU."""
 
 from __future__ import annotations
 
+import warnings
 from typing import Any, Optional
 
 import torch
 
-from ...workers.utils.losses import _FusedPPOLoss, agg_numbers, fused_ppo_loss
+from ...workers.utils.losses import _cfg, _FusedPPOLoss, agg_numbers, fused_ppo_loss
 
 
 def agg_loss(
@@ -26,14 +28,6 @@ def agg_loss(
     # aggregation-only form of the kernel: loss = 0 - (-1) * agg(loss_mat)
     loss, _ = _FusedPPOLoss.apply(None, loss_mat, None, None, loss_mask, None, None, agg, (0, 0.0), 0.2, 0.2, 3.0, -1.0)
     return loss
-
-
-def _cfg(config, name, default=None):
-    if isinstance(config, dict):
-        return config.get(name, default)
-    if hasattr(config, name):
-        return getattr(config, name)
-    return config.get(name, default) if hasattr(config, "get") else default
 
 
 def compute_policy_loss_vanilla(
@@ -66,3 +60,41 @@ def compute_policy_loss_vanilla(
         k: metrics[k].detach().item() for k in ("actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower")
     }
     return pg_loss, pg_metrics
+
+
+def compute_policy_loss(
+    old_log_prob,
+    log_prob,
+    advantages,
+    response_mask,
+    cliprange=None,
+    cliprange_low=None,
+    cliprange_high=None,
+    clip_ratio_c=3.0,
+    loss_agg_mode: str = "token-mean",
+):
+    """Deprecated spelling of the vanilla loss (the reference warns with ``FutureWarning`` and so does this): no
+    config object, no IS weights, no global normalisers; returns the 4-tuple ``(pg_loss, pg_clipfrac, ppo_kl,
+    pg_clipfrac_lower)`` with the three statistics as 0-dim tensors, like the reference's ``masked_mean`` results."""
+    warnings.warn(
+        "Warning: Function 'verl_amd.trainer.ppo.core_algos.compute_policy_loss' is deprecated. Please use "
+        "'verl_amd.trainer.ppo.core_algos.compute_policy_loss_vanilla' instead.",
+        category=FutureWarning,
+        stacklevel=2,
+    )
+    pg_loss, m = fused_ppo_loss(
+        log_prob, None, old_log_prob, advantages, response_mask,
+        clip_ratio=cliprange, clip_ratio_low=cliprange_low, clip_ratio_high=cliprange_high, clip_ratio_c=clip_ratio_c,
+        loss_agg_mode=loss_agg_mode,
+    )  # fmt: skip
+    return pg_loss, m["actor/pg_clipfrac"], m["actor/ppo_kl"], m["actor/pg_clipfrac_lower"]
+
+
+POLICY_LOSS_REGISTRY = {"vanilla": compute_policy_loss_vanilla}
+
+
+def get_policy_loss_fn(name):
+    """Only the vanilla loss has a fused kernel; the message is the reference's."""
+    if name not in POLICY_LOSS_REGISTRY:
+        raise ValueError(f"Unsupported loss mode: {name}. Supported modes are: {list(POLICY_LOSS_REGISTRY.keys())}")
+    return POLICY_LOSS_REGISTRY[name]

@@ -79,6 +79,14 @@ def set_vocab_chunk(columns: int):
     _config._vocab_chunk = int(columns)
 
 
+def set_workspace_budget(num_bytes: int):
+    """Byte budget of the backward's workspace (process-wide; 0 = the library's default rule: chunks of 8192 vocabulary
+    columns, wider while one d_logits buffer stays within 256 MiB).  The library then picks the widest vocabulary chunk
+    whose workspace fits the budget (never fewer than 2048 columns) and never exceeds its own upper bound of a quarter of
+    one ``[T, V]`` tensor plus one fp32 ``[V, H]``.  An explicit ``set_vocab_chunk`` takes precedence."""
+    _abi.check(_abi.load().lce_set_option(8, int(num_bytes)), "lce_set_option")
+
+
 def _require_single_rank(dist_process_group) -> None:
     """The vocabulary is not sharded here: only ``None`` or a process group of exactly one rank is accepted."""
     if dist_process_group is None:
@@ -185,8 +193,11 @@ def efficient_entropy_backward(
     if dentropy is not None:
         assert dentropy.is_cuda and dentropy.device == dev and dentropy.shape == (T,)
         g_ent = dentropy.detach().to(torch.float32).contiguous()
-    d_hidden = torch.empty_like(hidden)
-    d_weight = torch.empty((V, H), device=dev, dtype=hidden.dtype)
+    # should_return_fp32_grad: both gradients straight from the fp32 accumulators, without the rounding to the input dtype
+    # (verl/utils/kernel/kernels.py:1562-1567)
+    grad_dtype = torch.float32 if should_return_fp32_grad else hidden.dtype
+    d_hidden = torch.empty((T, H), device=dev, dtype=grad_dtype)
+    d_weight = torch.empty((V, H), device=dev, dtype=grad_dtype)
     if T == 0:
         d_weight.zero_()
     else:
@@ -195,13 +206,12 @@ def efficient_entropy_backward(
             vchunk = _config._vocab_chunk
             ws_bytes = lib.lce_backward_workspace_bytes(T, H, V, code, vchunk)
             ws = torch.empty((ws_bytes,), device=dev, dtype=torch.uint8)
-            rc = lib.lce_backward(
+            entry = lib.lce_backward_f32 if should_return_fp32_grad else lib.lce_backward
+            rc = entry(
                 hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
                 code, float(temperature), reduction, maximum.data_ptr(), acc.data_ptr(), entropy_b.data_ptr(),
                 g_lp.data_ptr(), _abi.ptr(g_ent), d_hidden.data_ptr(), d_weight.data_ptr(), ws.data_ptr(), ws_bytes,
                 vchunk, _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_backward")
-    if should_return_fp32_grad:
-        d_hidden, d_weight = d_hidden.float(), d_weight.float()
     return d_hidden, d_weight

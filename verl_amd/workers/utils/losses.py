@@ -245,3 +245,130 @@ def fused_ppo_loss_packed(
     start, length = response_slices(prompt_lens.to(dev), response_lens.to(dev), log_prob.numel())
     assert int(length.max().item()) <= response_mask.shape[1], "a response is longer than max_response_len"
     return fused_ppo_loss(log_prob, entropy, old_log_prob, advantages, response_mask, _packed=(start, length), **kwargs)
+
+
+def _cfg(config, name, default=None):
+    """``config.name`` or ``config[name]``: the reference's configs are dataclasses that also answer ``.get``."""
+    if isinstance(config, dict):
+        return config.get(name, default)
+    if hasattr(config, name):
+        return getattr(config, name)
+    return config.get(name, default) if hasattr(config, "get") else default
+
+
+def _get(data, key, default=None):
+    try:
+        return data[key]
+    except KeyError:
+        return default
+
+
+def _has(data, key) -> bool:
+    try:
+        return key in data
+    except TypeError:
+        return _get(data, key) is not None
+
+
+def batch_lens(data):
+    """``(prompt_lens, response_lens)`` of a data batch the way ``no_padding_2_padding`` reads them
+    (``verl/workers/utils/padding.py:110-124``): from the offsets of nested ``prompts`` / ``responses``, or from the
+    two halves of ``attention_mask`` when the batch is padded."""
+    prompts, responses = data["prompts"], data["responses"]
+    if prompts.is_nested:
+        return prompts.offsets().diff(), responses.offsets().diff()
+    attention_mask = data["attention_mask"]
+    assert not attention_mask.is_nested
+    P = prompts.shape[1]
+    return attention_mask[:, :P].sum(dim=1), attention_mask[:, P:].sum(dim=1)
+
+
+def _padded(t: torch.Tensor, width: int) -> torch.Tensor:
+    """A batch field as ``[batch, width]``: nested (jagged) fields are padded with zeros like ``to_padded_tensor``."""
+    if t.is_nested:
+        t = torch.nested.to_padded_tensor(t, 0.0)
+    if t.shape[1] < width:
+        t = torch.nn.functional.pad(t, (0, width - t.shape[1]))
+    return t
+
+
+def metric_aggregation_for(dp_size, batch_num_tokens, global_batch_size, loss_scale_factor):
+    """``losses.py:71-84``: once any global normaliser is set the loss of a micro-batch is already a share of the
+    global mean, so its metric adds up over micro-batches (SUM); otherwise each is a local mean (MEAN)."""
+    from ...utils.metric import AggregationType
+
+    if dp_size > 1 or batch_num_tokens is not None or global_batch_size is not None or loss_scale_factor is not None:
+        return AggregationType.SUM
+    return AggregationType.MEAN
+
+
+def ppo_loss(config, model_output, data, dp_group=None):
+    """The reference's actor loss entry (``verl/workers/utils/losses.py:57-155``) on the fused kernels: same arguments,
+    same ``(policy_loss, metrics)`` with ``Metric`` values under the reference's keys and aggregation kinds.
+
+    ``model_output["log_probs"]`` / ``["entropy"]``: the head's outputs over the packed sequences (``[total_nnz]`` or
+    nested); ``data``: a mapping with ``prompts``, ``responses`` (nested, or padded together with
+    ``attention_mask``), ``response_mask``, ``old_log_probs``, ``advantages``, optionally ``rollout_is_weights`` and
+    ``ref_log_prob``, and the entries ``dp_size``, ``batch_num_tokens``, ``global_batch_size``.  ``config``: an
+    ``ActorConfig``-like object (``clip_ratio*``, ``entropy_coeff``, ``loss_agg_mode``, ``loss_scale_factor``,
+    ``use_kl_loss``, ``kl_loss_coef``, ``kl_loss_type``, ``policy_loss.loss_mode``, dict ``global_batch_info``).
+    The response slice, the policy loss, the entropy and KL terms and all metrics are ONE ``lce_ppo_loss_packed``
+    call; gradients come back in packed order.  Only ``loss_mode == "vanilla"`` has a fused kernel; other modes and
+    the sampler-correction outputs (``sc_*``) raise ``NotImplementedError`` instead of taking a slower path."""
+    from ...utils.metric import AggregationType, Metric
+
+    for key in ("sc_correction", "sc_sampler_head_mass", "sc_train_head_mass"):
+        if _has(model_output, key):
+            raise NotImplementedError(f"model output {key!r}: the fused PPO loss has no sampler-correction term")
+    loss_mode = _cfg(_cfg(config, "policy_loss", {}) or {}, "loss_mode", "vanilla")
+    if loss_mode != "vanilla":
+        raise NotImplementedError(f"policy loss mode {loss_mode!r}: only 'vanilla' has a fused kernel")
+
+    log_prob = model_output["log_probs"]
+    log_prob = log_prob.values() if log_prob.is_nested else log_prob
+    entropy = _get(model_output, "entropy")
+    if entropy is not None and entropy.is_nested:
+        entropy = entropy.values()
+
+    info = {
+        "dp_size": data["dp_size"],
+        "batch_num_tokens": data["batch_num_tokens"],
+        "global_batch_size": data["global_batch_size"],
+        "loss_scale_factor": _cfg(config, "loss_scale_factor"),
+    }
+    shared = _cfg(config, "global_batch_info")
+    if isinstance(shared, dict):  # the reference leaves them on the config for the policy-loss function
+        shared.update(info)
+    metric_aggregation = metric_aggregation_for(**info)
+
+    prompt_lens, response_lens = batch_lens(data)
+    response_mask = data["response_mask"]
+    width = response_mask.shape[1] if not response_mask.is_nested else int(response_lens.max().item())
+    response_mask = _padded(response_mask, width).to(bool)
+    use_kl = bool(_cfg(config, "use_kl_loss", False))
+    is_weights = _get(data, "rollout_is_weights")
+    policy_loss, m = fused_ppo_loss_packed(
+        log_prob, entropy, prompt_lens, response_lens,
+        _padded(data["old_log_probs"], width), _padded(data["advantages"], width), response_mask,
+        clip_ratio=_cfg(config, "clip_ratio"),
+        clip_ratio_low=_cfg(config, "clip_ratio_low"),
+        clip_ratio_high=_cfg(config, "clip_ratio_high"),
+        clip_ratio_c=_cfg(config, "clip_ratio_c", 3.0),
+        entropy_coeff=_cfg(config, "entropy_coeff", 0.0) if entropy is not None else 0.0,
+        loss_agg_mode=_cfg(config, "loss_agg_mode", "token-mean"),
+        rollout_is_weights=None if is_weights is None else _padded(is_weights, width),
+        ref_log_prob=_padded(data["ref_log_prob"], width) if use_kl else None,
+        kl_loss_coef=_cfg(config, "kl_loss_coef", 0.001),
+        kl_loss_type=_cfg(config, "kl_loss_type", "low_var_kl"),
+        **info,
+    )  # fmt: skip
+    metrics = Metric.from_dict(
+        {k: m[k] for k in ("actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower")}, AggregationType.MEAN
+    )
+    metrics["actor/pg_loss"] = Metric(metric_aggregation, m["actor/pg_loss"])
+    if entropy is not None:
+        metrics["actor/entropy_loss"] = Metric(metric_aggregation, m["actor/entropy_loss"])
+    if use_kl:
+        metrics["kl_loss"] = Metric(metric_aggregation, m["kl_loss"])
+        metrics["kl_coef"] = _cfg(config, "kl_loss_coef", 0.001)
+    return policy_loss, metrics
