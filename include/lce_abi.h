@@ -211,7 +211,19 @@ int lce_num_variants(void);
  * to 16 bits with the rest of the d_logits tile; 2 = the label's whole entry of d_logits (one-hot and softmax part,
  * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32; 0 keeps everything inside
  * the tile, which is the reference's data format (verl/utils/kernel/kernels.py:1666-1724).  Changes the workspace size
- * like the option above. */
+ * like the option above.
+ * LCE_OPT_DLOGITS_STRIP (default 1, 16-bit inputs on the 16x16x32 loop): vocabulary tiles that one workgroup of the
+ * d_logits pass walks before it ends (1..64).
+ * LCE_OPT_DHIDDEN_KSPLIT (default 0 = by shape): K slices of the d_hidden GEMM, each with its own fp32 partial that
+ * is summed in a fixed order afterwards (0..16; changes the workspace size).
+ * LCE_OPT_WORKSPACE_BUDGET (default 0 = the built-in rule, chunks of 8192 vocabulary columns or wider while one
+ * d_logits buffer stays within 256 MiB): a byte count; lce_backward_workspace_bytes with vocab_chunk <= 0 then
+ * returns the workspace of the widest chunk that fits it (never below 2048 columns, never above the bound
+ * 0.25 * T * V * esz + 4 * V * H), and lce_backward with vocab_chunk <= 0 uses that chunk.  An explicit vocab_chunk
+ * is not touched.  Takes the role of the reference's fixed vocab_per_split = 9504 (verl/utils/kernel/kernels.py:1666-1670).
+ * LCE_OPT_FEW_TOKEN_GEMMS (default 1, 16-bit inputs): with at most 128 tokens both gradient GEMMs of the backward run
+ * as one launch of streaming kernels (d_weight written once in 64-byte runs, d_hidden from fp32 K-slice partials with
+ * the weight read in place); 0 = the 256 x 256 tile kernels.  Changes the workspace size. */
 enum {
   LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
   LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
