@@ -149,6 +149,13 @@ def run_logits_workload(args, name):
     g = torch.Generator(device=dev).manual_seed(1234 + 6)
     z = (torch.randn(R, V, device=dev, generator=g) * 3).bfloat16().requires_grad_(True)
     y = torch.randint(0, V, (R,), device=dev, generator=g)
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB per launch
+        torch.cuda.synchronize()
+        del src, dst
     g_lp = torch.randn(R, device=dev, generator=g).bfloat16()
     g_ent = torch.randn(R, device=dev, generator=g).bfloat16()
 
