@@ -134,9 +134,9 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
     const int k = (*p.n_rows + 31) / 32;
     ks_n = k < ks_n ? k : ks_n;
   }
-  // B fragments (dS) are the same for every h tile: with 64 token positions they stay in registers (read once the
-  // tile has landed), with 128 they are re-read per tile (registers)
-  constexpr bool KEEP_B = KT <= 64;
+  // B fragments (dS) are the same for every h tile: they stay in registers (read once the tile has landed) unless 128
+  // token positions meet 256-column tiles (registers)
+  constexpr bool KEEP_B = KT <= 64 || HW <= 128;
   u32x4_t bf[KEEP_B ? KS : 1][4];
   auto read_b = [&](int ks, u32x4_t (&out)[4]) {
 #pragma unroll

@@ -312,9 +312,24 @@ template <typename Cfg, int MODE, bool EDGE>
 LCE_DEV void gemm16_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x4_t (&acc)[Cfg::NB][Cfg::NB], int64_t mw, int64_t nw) {
   typedef typename Cfg::TIN TIN;
   // mw, nw: this lane's row of block column 0 and its first column of block row 0
+  // accumulate modes: the old values of block column j + 1 are fetched before column j is added and stored, so that
+  // a lane always has eight 16-byte loads in flight (measured on the d_hidden GEMM of one 8192-column chunk, 16384 x
+  // 3584 x 8192: 0.900 -> 0.875 ms; the same GEMM storing without reading takes 0.837)
+  f32x4_t prev[2][Cfg::NB];
+  auto fetch = [&](int j) {
+    const int64_t m = mw + j * 16;
+#pragma unroll
+    for (int i = 0; i < Cfg::NB; ++i) {
+      const int64_t n = nw + i * 16;
+      prev[j & 1][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (!(EDGE && (m >= p.M || n >= p.N))) prev[j & 1][i] = *reinterpret_cast<const f32x4_t*>(p.Cf + m * p.ldcf + n);
+    }
+  };
+  if (MODE & 1) fetch(0);
 #pragma unroll
   for (int j = 0; j < Cfg::NB; ++j) {
     const int64_t m = mw + j * 16;
+    if ((MODE & 1) && j + 1 < Cfg::NB) fetch(j + 1);
     if (EDGE && m >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < Cfg::NB; ++i) {
@@ -322,8 +337,7 @@ LCE_DEV void gemm16_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x4_t
       if (EDGE && n >= p.N) continue;  // (N is a multiple of 4)
       f32x4_t v = acc[i][j];
       if (MODE & 1) {
-        const f32x4_t old = *reinterpret_cast<const f32x4_t*>(p.Cf + m * p.ldcf + n);
-        v += old;
+        v += prev[j & 1][i];
       }
       if (MODE & 2) {
         typedef typename VecOf<TIN, 4>::type vec_t;
