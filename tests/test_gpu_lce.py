@@ -425,6 +425,42 @@ def test_vocab_chunking_is_transparent(vchunk):
     torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
 
 
+@pytest.mark.parametrize("T", [700, 5000])  # the 32x32x16 loop and the 16x16x32 loop
+def test_workspace_budget_changes_the_chunking_not_the_result(T):
+    """kernels.set_workspace_budget: the backward asks torch for exactly what lce_backward_workspace_bytes reports
+    under the budget (peak memory moves with it), runs more, narrower chunks, and returns the same gradients:
+    d_weight bit for bit (each row is complete within its chunk), d_hidden to the rounding of one more fp32 sum."""
+    from verl_amd import _abi
+    from verl_amd.utils.kernel import kernels
+
+    lib = _abi.load()
+    H, V, tau = 512, 40000, 1.0
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=31)
+    default_bytes = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
+
+    def peak_of_one_step():
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        out = _run(h, w, y, tau, g_lp, g_ent)
+        return out[2], out[3], torch.cuda.max_memory_allocated() - base
+
+    dh0, dw0, peak_default = peak_of_one_step()
+    try:
+        kernels.set_workspace_budget(default_bytes // 3)
+        small_bytes = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
+        assert small_bytes < default_bytes
+        dh1, dw1, peak_small = peak_of_one_step()
+    finally:
+        kernels.set_workspace_budget(0)
+    assert peak_default - peak_small >= 0.8 * (default_bytes - small_bytes)  # the workspace is what shrank
+    assert torch.equal(dw0, dw1)
+    torch.testing.assert_close(dh0.float(), dh1.float(), atol=1e-3, rtol=2.0**-7)
+    rdh, rdw = O.lce_backward(g_lp.float(), g_ent.float(), h, w, y, tau)
+    torch.testing.assert_close(dh1.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(dw1.float(), rdw, atol=2e-2, rtol=4e-2)
+
+
 @pytest.mark.parametrize("T,H,V,vchunk,dtype", [
     (64, 256, 5000, 2048, torch.bfloat16),   # 16 K slices per chunk; the short last chunk leaves half of them empty
     (100, 128, 300, 0, torch.bfloat16),      # single chunk narrower than the slices: empty slices on the first chunk

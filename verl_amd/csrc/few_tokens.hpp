@@ -194,11 +194,7 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
         float d[8];
 #pragma unroll
         for (int x = 0; x < 8; ++x) d[x] = acc[2 * ip + (x >> 2)][j][x & 3];
-#ifdef LCE_FEW_STREAM
-        store_run<TOUT, 8, true>(static_cast<TOUT*>(p.dW) + vrow[j] * p.H + h, d);
-#else
-        store_run<TOUT, 8>(static_cast<TOUT*>(p.dW) + vrow[j] * p.H + h, d);
-#endif
+        store_run<TOUT, 8>(static_cast<TOUT*>(p.dW) + vrow[j] * p.H + h, d);  // (non-temporal stores: 2.9 instead of 4.1 TB/s)
       }
     }
   }
@@ -317,13 +313,7 @@ LCE_DEV void dh_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
 // which keeps the accumulators and the tile in flight within 128 registers a lane)
 template <int KT>
 struct FewShape {
-#ifndef LCE_FEW_HW_DW
-#define LCE_FEW_HW_DW (KT <= 64 ? 256 : 128)
-#endif
-#ifndef LCE_FEW_HW_DH
-#define LCE_FEW_HW_DH (KT <= 64 ? 256 : 128)
-#endif
-  static constexpr int NT = KT, HW = LCE_FEW_HW_DH, HW_DW = LCE_FEW_HW_DW;
+  static constexpr int NT = KT, HW = KT <= 64 ? 256 : 128, HW_DW = HW;
   static constexpr int DW = KT * 128 + KT * HW_DW * 2;
   static constexpr int DH = 64 * HW * 2 + NT * 128;
   static constexpr int LDS_BYTES = DW > DH ? DW : DH;

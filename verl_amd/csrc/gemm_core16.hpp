@@ -197,11 +197,7 @@ struct GemmCore16 {
                      u32x4_t (&af_n)[NB], u32x4_t (&bf_n)[NB], char* lds, int dma_slot, int64_t dma_ks) const {
     static_for(std::make_integer_sequence<int, NB * NB>{}, [&](auto mc) {
       constexpr int m = decltype(mc)::value;
-#ifdef LCE16_SNAKE
-      constexpr int i = m / NB, j = (i & 1) ? NB - 1 - m % NB : m % NB;  // boustrophedon: one operand changes per MFMA
-#else
       constexpr int i = m / NB, j = m % NB;
-#endif
       if constexpr (WAIT && (i == 0 || m % NB == 0)) {
         constexpr int need = i == 0 ? 1 + j : 8 + i;  // the last fragment this MFMA depends on
         constexpr int allow = (ALLI - upto(need)) + upto(frags_before(m) - 1);

@@ -48,24 +48,6 @@ LCE_DEV void fwd16_fold(const FwdArgs<typename Cfg::TIN>& p, const f32x4_t (&acc
         if (!FULL && vbase + 16 * i + 4 * g4 + r >= vend) v = -INFINITY;  // padded vocabulary rows
         x[i * 4 + r] = v;
       }
-#ifdef LCE16_FWD_NOEPI
-    float aj = a[j] + x[0], bj = b[j];
-#elif defined(LCE16_FWD_SERIAL)
-    float tmax = x[0];
-#pragma unroll
-    for (int q = 1; q < NB * 4; ++q) tmax = fmaxf(tmax, x[q]);
-    const float mn = fmaxf(m[j], tmax);
-    const float sc = fast_exp2((m[j] - mn) * p.c);
-    const float mc = mn * p.c;
-    float aj = a[j] * sc, bj = b[j] * sc;
-    m[j] = mn;
-#pragma unroll
-    for (int q = 0; q < NB * 4; ++q) {
-      const float e = fast_exp2(__builtin_fmaf(x[q], p.c, -mc));
-      aj += e;
-      bj = __builtin_fmaf(FULL ? x[q] : (x[q] == -INFINITY ? 0.f : x[q]), e, bj);
-    }
-#else
     // four independent chains each for the maximum and the two sums: one wave per SIMD has no neighbour to hide the
     // latency of a dependent chain of 32
     float t4[4] = {x[0], x[1], x[2], x[3]};
@@ -85,7 +67,6 @@ LCE_DEV void fwd16_fold(const FwdArgs<typename Cfg::TIN>& p, const f32x4_t (&acc
       b4[q & 3] = __builtin_fmaf(FULL ? x[q] : (x[q] == -INFINITY ? 0.f : x[q]), e, b4[q & 3]);
     }
     const float aj = (a4[0] + a4[1]) + (a4[2] + a4[3]), bj = (b4[0] + b4[1]) + (b4[2] + b4[3]);
-#endif
     a[j] = aj;
     b[j] = bj;
     // label logit: rare (a token's label falls in this wave tile with probability WM / V)
