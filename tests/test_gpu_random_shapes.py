@@ -20,6 +20,10 @@ def _case(seed):
     T = rnd.choice([1, 2, 31, 64, 255, 256, 257, 300, 511, 777, 1024, 1500, 2049])
     H = 128 * rnd.choice([1, 2, 3, 5, 8])
     V = rnd.choice([2, 17, 255, 256, 257, 1000, 4099, 8192, 12345, 20011])
+    if seed >= 1000:  # many tokens: the backward's 16x16x32 tiles (from 4096 tokens), ragged against their 256 x 256 tiles
+        T = rnd.choice([4096, 4097, 4500, 5000, 8191, 9001])
+        H = 128 * rnd.choice([1, 2, 3])
+        V = rnd.choice([255, 257, 1000, 4099, 12345])
     tau = rnd.choice([0.5, 0.6, 1.0, 1.5, 2.0])
     reduction = rnd.choice(["none", "none", "none", "sum", "mean"])
     mask = rnd.choice(["dense", "dense", "prefix", "random", "zero_lp"])
@@ -35,6 +39,11 @@ def test_random_shape(seed):
 @pytest.mark.parametrize("seed", range(96, 128))
 def test_random_shape_fp16(seed):
     _check(seed, torch.float16)
+
+
+@pytest.mark.parametrize("seed", range(1000, 1024))
+def test_random_shape_many_tokens(seed):
+    _check(seed, torch.float16 if seed % 4 == 3 else None)
 
 
 def _check(seed, force_dtype):
