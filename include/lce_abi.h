@@ -223,7 +223,11 @@ int lce_num_variants(void);
  * is not touched.  Takes the role of the reference's fixed vocab_per_split = 9504 (verl/utils/kernel/kernels.py:1666-1670).
  * LCE_OPT_FEW_TOKEN_GEMMS (default 1, 16-bit inputs): with at most 128 tokens both gradient GEMMs of the backward run
  * as one launch of streaming kernels (d_weight written once in 64-byte runs, d_hidden from fp32 K-slice partials with
- * the weight read in place); 0 = the 256 x 256 tile kernels.  Changes the workspace size. */
+ * the weight read in place); 0 = the 256 x 256 tile kernels.  Changes the workspace size.
+ * LCE_OPT_DHIDDEN_IN_PLACE (default 1, 16-bit inputs on the 16x16x32 loop): the d_hidden GEMM reads the weight as it
+ * lies in memory (K-major operand through transposing LDS reads); 0 = a transposed copy of every vocabulary chunk is
+ * built first (one more launch and H x chunk elements of workspace per chunk; same speed at T=16384).  Changes the
+ * workspace size. */
 enum {
   LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
   LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
@@ -233,7 +237,8 @@ enum {
   LCE_OPT_DLOGITS_STRIP = 6,
   LCE_OPT_DHIDDEN_KSPLIT = 7,
   LCE_OPT_WORKSPACE_BUDGET = 8,
-  LCE_OPT_FEW_TOKEN_GEMMS = 9
+  LCE_OPT_FEW_TOKEN_GEMMS = 9,
+  LCE_OPT_DHIDDEN_IN_PLACE = 10
 };
 int lce_set_option(int key, int64_t value);
 

@@ -45,7 +45,7 @@ LCE_DEV void static_for(std::integer_sequence<int, Is...>, F&& f) {
 }
 
 // TRANS_: 0 both operands K-contiguous (row-major A[m][k], B[n][k]); 1 both K-major in memory, A[k][m] and
-// B[k][n], fetched with the transposing LDS read (two ds_read_b64_tr_b16 per fragment).
+// B[k][n], fetched with the transposing LDS read (two ds_read_b64_tr_b16 per fragment); 2 only A K-major (mixed).
 template <typename TIN_, int TRANS_ = 0>
 struct GemmCfg16 {
   typedef TIN_ TIN;
@@ -65,6 +65,7 @@ struct GemmCore16 {
   typedef typename Cfg::TIN TIN;
   static constexpr int NB = Cfg::NB, HL = Cfg::HL, SLOT = Cfg::STAGE_BYTES;
   static constexpr bool TN = Cfg::TRANS == 1;
+  static constexpr bool TA = Cfg::TRANS != 0, TB = Cfg::TRANS == 1;  // which operand is K-major in memory
 
   const char* a_base;
   const char* b_base;
@@ -72,6 +73,9 @@ struct GemmCore16 {
   uint32_t a_rd, b_rd;      // per-lane LDS read offsets inside a slot (block 0, k-step 0)
   int64_t a_slab, b_slab;   // bytes from one K slab to the next in memory
   int wave, lane, wave_m, wave_n;
+  // mixed mode: row of A inside a slab that each load fetches, A's row stride in bytes and the number of its rows that exist
+  uint32_t va_tail[HL];         // mixed mode: va of the last slab of A that has rows, rows beyond them clamped
+  int64_t a_ks_full, a_ks_last;  // slabs below a_ks_full have all their 64 rows; a_ks_last: the last slab with any
 
   LCE_DEV void set_lane() {
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -152,11 +156,58 @@ struct GemmCore16 {
   }
   static LCE_DEV int tn_swz(int row) { return ((row & 3) * 4) ^ (((row >> 3) & 1) * 2); }
 
+  // Mixed: A[k][m0 + 0..256) K-major as in init_tn, B row-major as in init (rows n0 .. of an N-row matrix, clamped).
+  // LDS row r of an A slab holds memory row perm(r) of the slab (perm: a permutation of 0..63, the order in which B's
+  // K index was stored); rows at or beyond `kvalid` > 0 are replaced by rows that exist (B is zero there), and columns at
+  // or beyond `mcols` (a last tile of a width that is no multiple of 256) by the row's first chunk: in bounds, and they
+  // feed only results that the epilogue discards.
+  template <typename Perm>
+  LCE_DEV void init_mixed(const TIN* A, int64_t lda, int64_t m0, int64_t mcols, int64_t kvalid, Perm perm, const TIN* B, int64_t ldb,
+                          int64_t n0, int64_t N) {
+    static_assert(Cfg::TRANS == 2, "mixed mode");
+    set_lane();
+    a_base = reinterpret_cast<const char*>(A + m0);
+    b_base = reinterpret_cast<const char*>(B + n0 * ldb);
+    a_slab = 64 * lda * 2;
+    b_slab = Cfg::BKB;
+    a_ks_full = kvalid / 64;
+    a_ks_last = (kvalid - 1) / 64;
+    const int last_row = (int)(kvalid - 1 - a_ks_last * 64);  // of slab a_ks_last
+    const int rows_b = (int)((N - n0) < (int64_t)Cfg::BN ? (N - n0) : (int64_t)Cfg::BN);
+    const int lr = lane >> 3, pc = lane & 7;
+#pragma unroll
+    for (int j = 0; j < HL; ++j) {
+      const int rowa = (j * Cfg::NW + wave) * 2 + (lane >> 5);
+      const int ca = (lane & 31) ^ tn_swz(rowa);
+      const int prow = (int)perm(rowa);
+      const uint32_t col = (uint32_t)(((int64_t)ca * 8 < mcols ? ca : 0) * 16);
+      va[j] = (uint32_t)((int64_t)prow * lda * 2) + col;
+      va_tail[j] = (uint32_t)((int64_t)(prow < last_row ? prow : last_row) * lda * 2) + col;
+      const int rowb = (j * Cfg::NW + wave) * 8 + lr;
+      const int cb = pc ^ ((rowb >> 1) & 7);
+      const int rb = rowb < rows_b ? rowb : rows_b - 1;
+      vb[j] = (uint32_t)((int64_t)rb * ldb * 2) + (uint32_t)(cb * 16);
+    }
+    const int g = lane >> 4, e = (lane & 15) >> 2, q = lane & 3;
+    const int row = 8 * g + e;
+    a_rd = (uint32_t)(row * 512 + wave_m * Cfg::WM * 2) + (uint32_t)((((q >> 1) ^ tn_swz(row)) * 16) + (q & 1) * 8);
+    const int r16 = lane & 15;
+    b_rd = (uint32_t)(wave_n * Cfg::WN * 128) + (uint32_t)(r16 * 128 + ((g ^ (r16 >> 1)) * 16));
+  }
+
   // ---- instruction-level pieces ----------------------------------------------------------------------------
   // load j of one operand's half slab number `ks` into ring slot `slot`
   LCE_DEV void dma(char* lds, int slot, int64_t ks, bool is_b, int j) const {
     char* dst = lds + slot * SLOT + (j * Cfg::NW + wave) * 1024;
-    const char* src = (is_b ? b_base + ks * b_slab + vb[j] : a_base + ks * a_slab + va[j]);
+    const char* src;
+    if (Cfg::TRANS == 2 && !is_b) {
+      // slabs with rows that do not exist take the last slab that has any, with its rows clamped (branch-free: the
+      // hand-placed schedule of a k-step must stay one basic block)
+      const bool tail = ks >= a_ks_full;
+      src = a_base + (tail ? a_ks_last : ks) * a_slab + (tail ? va_tail[j] : va[j]);
+    } else {
+      src = (is_b ? b_base + ks * b_slab + vb[j] : a_base + ks * a_slab + va[j]);
+    }
     __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
   }
 
@@ -164,14 +215,14 @@ struct GemmCore16 {
   // loop, so the first row of eight needs a0 and every b, the later rows one more a each.
   static constexpr bool frag_is_a(int f) { return f == 0 || f > 8; }
   static constexpr int frag_blk(int f) { return f == 0 ? 0 : (f <= 8 ? f - 1 : f - 8); }
-  static constexpr int CI = TN ? 2 : 1;  // LDS instructions per fragment
+  static constexpr int CA = TA ? 2 : 1, CB = TB ? 2 : 1;  // LDS instructions per fragment of each operand
   // ra / rb: LDS address of the slot plus a_rd / b_rd; S: k-step inside the slab
   template <int F, int S>
   LCE_DEV void read_frag(uint32_t ra, uint32_t rb, u32x4_t (&af)[NB], u32x4_t (&bf)[NB]) const {
     constexpr bool is_a = frag_is_a(F);
     constexpr int blk = frag_blk(F);
     u32x4_t v;
-    if constexpr (TN) {
+    if constexpr (is_a ? TA : TB) {
       // block: 16 columns = 32 bytes further, inside the swizzled chunk bits; k-step: 32 rows; second half: 4 rows
       const uint32_t base = (is_a ? ra : rb) ^ (uint32_t)(blk * 32);
       const u32x2_t lo = tr_read<S * 16384>(base), hi = tr_read<S * 16384 + 2048>(base);
@@ -184,8 +235,8 @@ struct GemmCore16 {
   }
 
   // LDS instructions issued up to and including fragment f of a k-step (f = -1: none)
-  static constexpr int upto(int f) { return (f + 1) * CI; }
-  static constexpr int ALLI = 16 * CI;
+  static constexpr int upto(int f) { return f < 0 ? 0 : (f == 0 ? CA : (f <= 8 ? CA + CB * f : CA + 8 * CB + CA * (f - 8))); }
+  static constexpr int ALLI = 8 * (CA + CB);
   // fragments of the next k-step issued before MFMA m of this one: one after each even MFMA of the first half
   static constexpr int frags_before(int m) { return (m + 1) / 2 > 16 ? 16 : (m + 1) / 2; }
 

@@ -48,6 +48,7 @@ struct Tuning {
   int dw_transposed_reads = 1;   // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
   int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
+  int dh_in_place16 = 1;         // 16x16x32 backward: the d_hidden GEMM reads W in place (mixed mode) instead of a transposed chunk
 };
 std::mutex g_tuning_mu;
 Tuning g_tuning;
@@ -322,7 +323,8 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
   // saves one transpose of W per call.  The transpose is the larger cost up to some thousands of tokens
   // (T=64: 1.95 -> 1.43 ms per forward + backward, T=4096: 15.7 -> 14.7 ms at H=3584, V=152064), the GEMM
   // rate beyond that (T=16384: +0.5 ms).
-  L.tn_dh = L.tn && T <= 8192 && variant != kVariantCore16;  // (the 16x16x32 loop has no mixed mode: it always takes W^T)
+  // (on the 16x16x32 loop the transposing reads of one operand cost under 1 %: W is always read in place there)
+  L.tn_dh = L.tn && (variant == kVariantCore16 ? tu.dh_in_place16 != 0 : T <= 8192);
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
@@ -838,6 +840,7 @@ int lce_set_option(int key, int64_t value) {
       t.ds_strip = (int)value;
       return LCE_OK;
     case LCE_OPT_FEW_TOKEN_GEMMS: t.few_token_gemms = value != 0; return LCE_OK;
+    case LCE_OPT_DHIDDEN_IN_PLACE: t.dh_in_place16 = value != 0; return LCE_OK;
     case LCE_OPT_WORKSPACE_BUDGET:
       if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_WORKSPACE_BUDGET takes a byte count (0 = the built-in default)");
       t.ws_budget = value;

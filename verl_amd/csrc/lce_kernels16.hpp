@@ -349,7 +349,10 @@ LCE_DEV void gemm16_epilogue(const GemmArgs<typename Cfg::TIN>& p, const f32x4_t
   }
 }
 
-template <typename Cfg>
+// CoreCfg: Cfg itself, or its mixed twin GemmCfg16<TIN, 2>: then B is K-major as it lies in memory, B[k][n] with row
+// stride ldb, its rows in the order KPerm<Cfg>::vocab_at of A's columns (the d_hidden GEMM reading W in place: no W^T);
+// rows of B at or beyond p.b_rows_valid do not exist (A is zero in those columns).
+template <typename Cfg, typename CoreCfg = Cfg>
 LCE_DEV void gemm16_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* lds) {
   GemmArgs<typename Cfg::TIN> p = pin;
   if (p.m_dev) {
@@ -372,10 +375,15 @@ LCE_DEV void gemm16_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, char* 
   const TileMap map = p.m_dev ? p.map.with_rows((int)((p.M + Cfg::BM - 1) / Cfg::BM)) : p.map;
   if (!map.decode(bid, tm, tn)) return;
   const int64_t m0 = (int64_t)tm * Cfg::BM, n0 = (int64_t)tn * Cfg::BN;
-  GemmCore16<Cfg> g;
+  GemmCore16<CoreCfg> g;
   f32x4_t acc[Cfg::NB][Cfg::NB];
-  if (k0 < k1) {
-    g.init(p.B + k0, p.ldb, n0, p.N, p.A + k0, p.lda, m0, p.M);  // MFMA rows = n, MFMA columns = m
+  if (k0 < k1 && (CoreCfg::TRANS != 2 || k0 < p.b_rows_valid)) {
+    // MFMA rows = n, MFMA columns = m
+    if constexpr (CoreCfg::TRANS == 2)
+      g.init_mixed(p.B + k0 * p.ldb, p.ldb, n0, p.N - n0, p.b_rows_valid - k0, [](int r) { return KPerm<Cfg>::vocab_at(r); }, p.A + k0, p.lda,
+                   m0, p.M);
+    else
+      g.init(p.B + k0, p.ldb, n0, p.N, p.A + k0, p.lda, m0, p.M);
     g.run(lds, k1 - k0, acc);
   } else {  // empty K range: contributes zero (and still initialises what it owns)
     if (p.out_mode == 1) return;
@@ -472,6 +480,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void gemm16_tn_kernel(GemmArgs<typen
 template <typename Cfg>
 LCE_DEV void any_gemm16_tile(const GemmArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   if (p.tn == 1) gemm16_tn_tile<GemmCfg16<typename Cfg::TIN, 1>, Cfg>(p, bid, lds);
+  else if (p.tn == 2) gemm16_tile<Cfg, GemmCfg16<typename Cfg::TIN, 2>>(p, bid, lds);
   else gemm16_tile<Cfg>(p, bid, lds);
 }
 
