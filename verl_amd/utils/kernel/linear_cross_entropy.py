@@ -3,9 +3,11 @@
 Call-compatible with the reference's ``verl/utils/kernel/linear_cross_entropy.py:38-119``:
 ``linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None)
 -> (logprobs, entropy)``; outputs are fp32 and flattened to ``[T]`` (``logprobs`` is 0-dim for
-``"sum"`` / ``"mean"``), ``d_hidden`` is viewed back to ``hidden``'s shape, ``d_weight`` has
-``hidden.dtype``, the four non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never
-written to memory.
+``"sum"`` / ``"mean"``), ``d_hidden`` comes back in ``hidden``'s shape, ``d_weight`` has ``hidden.dtype``, the four
+non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory.
+
+The autograd node is a thin shell: everything it does besides argument checks and reshapes happens in the two host
+launchers of ``kernels.py`` (one C-ABI call each).
 """
 
 from __future__ import annotations
@@ -14,8 +16,20 @@ import typing
 
 import torch
 
+from . import kernels
+
+
+def _as_token_rows(hidden: torch.Tensor, labels: torch.Tensor):
+    """``[..., H]`` / ``[...]`` viewed as ``[T, H]`` / ``[T]`` (views, like the reference: a tensor that cannot be
+    viewed raises)."""
+    rows = hidden if hidden.dim() == 2 else hidden.view(-1, hidden.shape[-1])
+    flat = labels if labels.dim() == 1 else labels.view(-1)
+    return rows, flat
+
 
 class LinearCrossEntropy(torch.autograd.Function):
+    """``apply(hidden, weight, labels, temperature, reduction, dist_process_group)``."""
+
     @staticmethod
     def forward(
         ctx,
@@ -26,54 +40,29 @@ class LinearCrossEntropy(torch.autograd.Function):
         reduction: typing.Optional[str] = "none",
         dist_process_group=None,
     ):
+        # the reference's two type checks (:64-65), messages included: callers' tests match on them
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
-        with torch.cuda.nvtx.range("LinearCrossEntropy-forward"):
-            from . import kernels
-
-            REDUCTION = kernels.get_entropy_reduction_enum_number(reduction.lower())
-            original_hidden_shape = hidden.shape
-            if len(hidden.shape) != 2:
-                hidden = hidden.view(-1, hidden.shape[-1])
-            if len(labels.shape) != 1:
-                labels = labels.view(-1)
-            logprobs, entropy, _maximum, _accumulate, _entropy_b = kernels.efficient_entropy_forward(
-                hidden, weight, labels, REDUCTION, temperature, dist_process_group
-            )
-            ctx.save_for_backward(hidden, weight, labels, _maximum, _accumulate, _entropy_b)
-            ctx.original_hidden_shape = original_hidden_shape
-            ctx.REDUCTION = REDUCTION
-            ctx.dist_process_group = dist_process_group
-            ctx.should_return_fp32_grad = False
-            ctx.temperature = temperature
-            ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
+        mode = kernels.get_entropy_reduction_enum_number(reduction.lower())
+        rows, flat_labels = _as_token_rows(hidden, labels)
+        logprobs, entropy, *stats = kernels.efficient_entropy_forward(rows, weight, flat_labels, mode, temperature, dist_process_group)
+        ctx.save_for_backward(rows, weight, flat_labels, *stats)  # stats = (maximum, accumulate, entropy_b), fp32 [T]
+        ctx.call = (hidden.shape, mode, temperature, dist_process_group)
+        ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
         return logprobs, entropy
 
     @staticmethod
     def backward(ctx, dlogprobs: typing.Optional[torch.Tensor], dentropy: typing.Optional[torch.Tensor]):
-        from . import kernels
-
-        with torch.cuda.nvtx.range("LinearCrossEntropy-backward"):
-            (hidden, weight, labels, _maximum, _accumulate, _entropy_b) = ctx.saved_tensors
-            if dlogprobs is None:
-                shape = (hidden.shape[0],) if ctx.REDUCTION == 0 else ()
-                dlogprobs = torch.zeros(shape, device=hidden.device, dtype=torch.float32)
-            d_hidden, d_weight = kernels.efficient_entropy_backward(
-                dlogprobs,
-                dentropy,
-                hidden,
-                weight,
-                labels,
-                _maximum,
-                _accumulate,
-                _entropy_b,
-                ctx.REDUCTION,
-                ctx.should_return_fp32_grad,
-                ctx.temperature,
-                ctx.dist_process_group,
-            )
-            d_hidden = d_hidden.view(ctx.original_hidden_shape)
-        return (d_hidden, d_weight, None, None, None, None)
+        rows, weight, flat_labels, maximum, accumulate, entropy_b = ctx.saved_tensors
+        shape, mode, temperature, group = ctx.call
+        if dlogprobs is None:  # only the entropy was used downstream
+            dlogprobs = torch.zeros((rows.shape[0],) if mode == 0 else (), device=rows.device, dtype=torch.float32)
+        d_rows, d_weight = kernels.efficient_entropy_backward(
+            dlogprobs, dentropy, rows, weight, flat_labels, maximum, accumulate, entropy_b, mode,
+            False,  # should_return_fp32_grad: autograd wants the inputs' dtype
+            temperature, group,
+        )  # fmt: skip
+        return d_rows.view(shape), d_weight, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply
