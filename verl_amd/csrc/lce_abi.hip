@@ -285,7 +285,7 @@ int forward_splits_upper_bound(int64_t T, int64_t V) {
 
 struct BwdLayout {
   int64_t vchunk, tpad, vpad, ldS, ldST, ldWt, ldHt;
-  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_coef, off_keys[2], off_vals[2], off_hist, off_tokc, off_tokl, total;
+  size_t off_dS[2], off_dST[2], off_Wt, off_Ht, off_dHacc, off_rows, off_inv, off_nrows, off_acounts, off_coef, off_keys[2], off_vals[2], off_hist, off_tokc, off_tokl, total;
   int sort_items, sort_passes;  // label sort (0 items: the one-hot part stays inside the d_logits tiles)
   int nchunks;
   int ksplit;  // K splits of the d_hidden GEMM (each with its own fp32 partial)
@@ -367,6 +367,7 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
   L.off_rows = o;  o += align256((size_t)L.tpad * 4);
   L.off_inv = o;   o += align256((size_t)T * 4);
   L.off_nrows = o; o += 256;
+  L.off_acounts = o; o += align256((size_t)((T + kActiveBlock - 1) / kActiveBlock) * 4);  // per-block counts of the token list
   // (label row, token) pairs, two buffers each, and the per-block digit counts of one radix pass
   L.sort_items = (esz == 2 && tu.label_outside && T <= ((int64_t)1 << 30)) ? (int)round_up(T, kSortBlock) : 0;
   int vbits = 1;
@@ -469,8 +470,12 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   int* n_rows = compact ? reinterpret_cast<int*>(ws + L.off_nrows) : nullptr;
   if (compact) {
     ProfScope prof(PC_ACTIVE_ROWS, st);
-    hipLaunchKernelGGL(active_rows_kernel<1024>, dim3(1), dim3(1024), 0, st, dlogprobs,
-                       (int64_t)(reduction == LCE_REDUCTION_NONE ? 1 : 0), dentropy, T, rows, inv, n_rows);
+    int* acounts = reinterpret_cast<int*>(ws + L.off_acounts);
+    const unsigned nblk = (unsigned)((T + kActiveBlock - 1) / kActiveBlock);
+    const int64_t gstride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
+    hipLaunchKernelGGL(active_count_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, gstride, dentropy, T, acounts);
+    if ((rc = check_launch("active_count_kernel"))) return rc;
+    hipLaunchKernelGGL(active_rows_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, gstride, dentropy, T, acounts, rows, inv, n_rows);
     if ((rc = check_launch("active_rows_kernel"))) return rc;
   }
   // tokens grouped by label for the one-hot part of d_weight (added after the GEMMs)
