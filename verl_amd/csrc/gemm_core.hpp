@@ -19,9 +19,6 @@
 
 namespace lce {
 
-#ifdef LCE_DBG_TIMING
-__device__ unsigned long long lce_dbg_times[16];
-#endif
 
 typedef __bf16 bf16_t;
 typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
@@ -65,10 +62,6 @@ struct Mma;
 template <>
 struct Mma<bf16_t> {
   static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
-#ifdef LCE_DBG_NO_MFMA
-    asm volatile("" ::"v"(a), "v"(b));  // keeps the operand reads alive
-    return;
-#endif
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
                                                   acc, 0, 0, 0);
   }
@@ -78,10 +71,6 @@ struct Mma<bf16_t> {
 template <>
 struct Mma<f16_t> {
   static LCE_DEV void run(f32x16_t& acc, const u32x4_t& a, const u32x4_t& b) {
-#ifdef LCE_DBG_NO_MFMA
-    asm volatile("" ::"v"(a), "v"(b));
-    return;
-#endif
     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
                                                  acc, 0, 0, 0);
   }
@@ -261,9 +250,6 @@ struct GemmCore {
 
   // one of the PER wave-wide 16-byte-per-lane global->LDS loads of a slab (A loads first)
   LCE_DEV void dma_one(char* lds, int stage, int64_t kbyte, int idx) const {
-#ifdef LCE_DBG_NO_DMA
-    if (kbyte > 0) return;
-#endif
     char* sa = lds + stage * Cfg::STAGE_BYTES;
     if (idx < Cfg::A_LOADS) {
       __builtin_amdgcn_global_load_lds((gptr_t)(a_base + kbyte + la.voff[idx]),
@@ -276,9 +262,6 @@ struct GemmCore {
   }
   // split ring: load j of one operand's half slab into ring slot `slot`
   LCE_DEV void dma_half(char* lds, int slot, int64_t kbyte, bool is_b, int j) const {
-#ifdef LCE_DBG_NO_DMA
-    if (kbyte > 0) return;
-#endif
     char* sa = lds + slot * Cfg::STAGE_BYTES + (j * Cfg::NW + wave) * 1024;
     // kbyte counts BKB bytes per slab; K-major operands advance by 64 rows per slab instead
     if (is_b) {
@@ -303,9 +286,6 @@ struct GemmCore {
   // one of the N_READS operand reads of k-substep kk, in the order a0, b0..b(FN-1), a1..a(FM-1)
   // (sa, sb: the ring slots holding the A and the B operand; the same pointer unless the ring is split)
   LCE_DEV void read_one(const char* sa, const char* sb, int kk, int idx, u32x4_t (&af)[Cfg::FM], u32x4_t (&bf)[Cfg::FN]) const {
-#ifdef LCE_DBG_NO_READS
-    if (kk > 0) return;
-#endif
     if constexpr (Cfg::TRANS != 0) {
       const bool is_a = idx == 0 || idx > Cfg::FN;
       const int blk = idx == 0 ? 0 : (idx <= Cfg::FN ? idx - 1 : idx - Cfg::FN);
@@ -445,12 +425,6 @@ struct GemmCore {
     load_frags(lds, lds, 0, af[0], bf[0]);
     int stage = 0;
     int64_t kb_next = (int64_t)NS * Cfg::BKB;
-#ifdef LCE_DBG_TIMING
-    uint64_t dbg_compute = 0, dbg_vm = 0, dbg_bar = 0;
-    uint64_t dbg_last = __builtin_amdgcn_s_memtime();
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    const uint64_t dbg_t0 = dbg_last;
-#endif
     for (int it = 0; it < nk; ++it) {
       const char* s = lds + stage * Cfg::STAGE_BYTES;
 #pragma unroll
@@ -459,42 +433,15 @@ struct GemmCore {
       }
       // last substep of this slab: its fragments are in registers, so this wave is done with the stage
       const int nstage = stage + 1 == NS ? 0 : stage + 1;
-#ifdef LCE_DBG_TIMING
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      const uint64_t t1 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      wait_vm<Cfg::SPLIT ? 0 : (NS - 2) * PER>();
-      const uint64_t t2 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      __builtin_amdgcn_s_barrier();
-      const uint64_t t3 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      dbg_compute += t1 - dbg_last;  // last substep of the previous slab + substeps 0..KSUB-2 of this one
-      dbg_vm += t2 - t1;
-      dbg_bar += t3 - t2;
-      dbg_last = t3;
-#else
       wait_vm<Cfg::SPLIT ? 0 : (NS - 2) * PER>();  // slab it+1 has landed (only the younger slabs may be in flight)
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of the stage have returned
       __builtin_amdgcn_s_barrier();
-#endif
       substep<1>(acc, af[(KSUB - 1) & 1], bf[(KSUB - 1) & 1], lds + nstage * Cfg::STAGE_BYTES,
                     lds + nstage * Cfg::STAGE_BYTES, 0, af[0], bf[0], lds, stage, kb_next < last_kbyte ? kb_next : last_kbyte);
       kb_next += Cfg::BKB;
       stage = nstage;
     }
     wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
-#ifdef LCE_DBG_TIMING
-    if (lane == 0 && (wave == 0 || wave == Cfg::NW - 1)) {
-      const uint64_t t_end = __builtin_amdgcn_s_memtime();
-      unsigned long long* d = lce_dbg_times + (wave == 0 ? 0 : 8);
-      atomicAdd(d + 0, (unsigned long long)dbg_compute);
-      atomicAdd(d + 1, (unsigned long long)dbg_vm);
-      atomicAdd(d + 2, (unsigned long long)dbg_bar);
-      atomicAdd(d + 3, (unsigned long long)(t_end - dbg_t0));
-      atomicAdd(d + 4, (unsigned long long)nk);
-    }
-#endif
   }
 
   // K loop over the split ring.  One operand is "early" (E: A with SPLIT = 1, B with SPLIT = 2), the
@@ -523,12 +470,6 @@ struct GemmCore {
     u32x4_t af[2][Cfg::FM], bf[2][Cfg::FN];
     load_frags(lds + (A_EARLY ? 0 : Cfg::STAGE_BYTES), lds + (A_EARLY ? Cfg::STAGE_BYTES : 0), 0, af[0], bf[0]);
     int sa = 0;  // slot of this slab's early half; the late half is in the next slot
-#ifdef LCE_DBG_TIMING
-    uint64_t dbg_compute = 0, dbg_vm = 0, dbg_bar = 0;
-    uint64_t dbg_last = __builtin_amdgcn_s_memtime();
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    const uint64_t dbg_t0 = dbg_last;
-#endif
     for (int it = 0; it < nk; ++it) {
       const int sb = sa + 1 >= 5 ? sa + 1 - 5 : sa + 1;
       const int na = sa + 2 >= 5 ? sa + 2 - 5 : sa + 2;
@@ -541,41 +482,14 @@ struct GemmCore {
       substep<EARLY, 0, HL / 2>(acc, af[0], bf[0], pa, pb, 1, af[1], bf[1], lds, fa, kb);
       substep<EARLY, HL / 2, HL>(acc, af[1], bf[1], pa, pb, 2, af[0], bf[0], lds, fa, kb);
       substep<0>(acc, af[0], bf[0], pa, pb, 3, af[1], bf[1], lds, 0, 0);
-#ifdef LCE_DBG_TIMING
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      const uint64_t t1 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      wait_vm<HL>();
-      const uint64_t t2 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      __builtin_amdgcn_s_barrier();
-      const uint64_t t3 = __builtin_amdgcn_s_memtime();
-      __builtin_amdgcn_s_waitcnt(0xC07F);
-      dbg_compute += t1 - dbg_last;
-      dbg_vm += t2 - t1;
-      dbg_bar += t3 - t2;
-      dbg_last = t3;
-#else
       wait_vm<HL>();                       // slab it+1 has landed; E(it+2) may still be in flight
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's reads of both slots have returned
       __builtin_amdgcn_s_barrier();
-#endif
       substep<LATE, 0, HL>(acc, af[1], bf[1], lds + (A_EARLY ? na : nb) * Cfg::STAGE_BYTES, lds + (A_EARLY ? nb : na) * Cfg::STAGE_BYTES, 0,
                            af[0], bf[0], lds, sa, kb);
       sa = na;
     }
     wait_vm<0>();  // drain the redundant tail fetches before LDS is reused
-#ifdef LCE_DBG_TIMING
-    if (lane == 0 && (wave == 0 || wave == Cfg::NW - 1)) {
-      const uint64_t t_end = __builtin_amdgcn_s_memtime();
-      unsigned long long* d = lce_dbg_times + (wave == 0 ? 0 : 8);
-      atomicAdd(d + 0, (unsigned long long)dbg_compute);
-      atomicAdd(d + 1, (unsigned long long)dbg_vm);
-      atomicAdd(d + 2, (unsigned long long)dbg_bar);
-      atomicAdd(d + 3, (unsigned long long)(t_end - dbg_t0));
-      atomicAdd(d + 4, (unsigned long long)nk);
-    }
-#endif
   }
 
   // s_waitcnt lgkmcnt(n) only; n is a constant after unrolling, the switch folds away

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void label_coef_kernel(const T* h, int64_t ldh
 
 // keys[k] = label row of the k-th listed token (rows[k], or k itself without a list), vals[k] = that token;
 // positions from the list's length up to n_items are filled with kNoRow.
-__global__ __launch_bounds__(256) void label_keys_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int n_items,
+inline __global__ __launch_bounds__(256) void label_keys_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int n_items,
                                                          uint32_t* keys, int* vals) {
   const int k = blockIdx.x * 256 + threadIdx.x;
   if (k >= n_items) return;
@@ -136,13 +136,13 @@ LCE_DEV void sort_scatter_block(const uint32_t* kin, const int* vin, uint32_t* k
   }
 }
 
-__global__ __launch_bounds__(256) void sort_hist_kernel(const uint32_t* keys, int shift, int nblocks, int* gh) {
+inline __global__ __launch_bounds__(256) void sort_hist_kernel(const uint32_t* keys, int shift, int nblocks, int* gh) {
   __shared__ int h[256];
   sort_hist_block(keys, shift, blockIdx.x, nblocks, gh, h);
 }
 
 // exclusive scan of gh[0 .. n) in place, one workgroup of 1024 threads
-__global__ __launch_bounds__(1024) void sort_scan_kernel(int* gh, int n) {
+inline __global__ __launch_bounds__(1024) void sort_scan_kernel(int* gh, int n) {
   __shared__ int part[1024];
   const int tid = threadIdx.x;
   const int per = (n + 1023) / 1024;
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(1024) void sort_scan_kernel(int* gh, int n) {
   }
 }
 
-__global__ __launch_bounds__(256) void sort_scatter_kernel(const uint32_t* kin, const int* vin, uint32_t* kout, int* vout, int shift,
+inline __global__ __launch_bounds__(256) void sort_scatter_kernel(const uint32_t* kin, const int* vin, uint32_t* kout, int* vout, int shift,
                                                            int nblocks, const int* gh) {
   __shared__ int base[256];
   sort_scatter_block(kin, vin, kout, vout, shift, blockIdx.x, nblocks, gh, base);
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256) void sort_scatter_kernel(const uint32_t* kin, 
 
 // Up to kSortBlock tokens: keys and all passes in one workgroup (buffers 0 / 1 alternate; `passes` is even or
 // odd, the caller reads the result from buffer passes % 2).
-__global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int passes,
+inline __global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm lt, const int* rows, const int* n_rows, int64_t T, int passes,
                                                                 uint32_t* keys0, int* vals0, uint32_t* keys1, int* vals1) {
   __shared__ int tab[256];
   __shared__ int gh[256];

@@ -250,7 +250,7 @@ __global__ void lce_fwd_shard_merge_kernel(const f32x4_t* parts, const float* xl
 
 // merges the partials of R vocabulary shards (shard-major [R][T]) in the fixed order r = 0, 1, ... and
 // emits the five per-token outputs
-__global__ void lce_merge_shards_kernel(const f32x4_t* partials, int R, int64_t T, float* logprobs, float* entropy,
+inline __global__ void lce_merge_shards_kernel(const f32x4_t* partials, int R, int64_t T, float* logprobs, float* entropy,
                                         float* maximum, float* accumulate, float* entropy_b) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
@@ -270,7 +270,7 @@ __global__ void lce_merge_shards_kernel(const f32x4_t* partials, int R, int64_t 
 }
 
 // deterministic single-workgroup sum of x[0..n) * scale -> out[0]
-__global__ void lce_reduce_sum_kernel(const float* x, int64_t n, float scale, float* out) {
+inline __global__ void lce_reduce_sum_kernel(const float* x, int64_t n, float scale, float* out) {
   __shared__ double sh[1024];
   double acc = 0.0;
   for (int64_t i = threadIdx.x; i < n; i += blockDim.x) acc += (double)x[i];
@@ -866,7 +866,7 @@ LCE_DEV bool token_is_active(const float* g_lp, int64_t g_lp_stride, const float
   return (g_lp[t * g_lp_stride] != 0.f) || (g_ent && g_ent[t] != 0.f);
 }
 
-__global__ __launch_bounds__(256) void active_count_kernel(const float* g_lp, int64_t g_lp_stride, const float* g_ent, int64_t T,
+inline __global__ __launch_bounds__(256) void active_count_kernel(const float* g_lp, int64_t g_lp_stride, const float* g_ent, int64_t T,
                                                            int* block_counts) {
   __shared__ int part[4];
   const int64_t base = (int64_t)blockIdx.x * kActiveBlock;
@@ -881,7 +881,7 @@ __global__ __launch_bounds__(256) void active_count_kernel(const float* g_lp, in
   if (threadIdx.x == 0) block_counts[blockIdx.x] = part[0] + part[1] + part[2] + part[3];
 }
 
-__global__ __launch_bounds__(256) void active_rows_kernel(const float* g_lp, int64_t g_lp_stride, const float* g_ent, int64_t T,
+inline __global__ __launch_bounds__(256) void active_rows_kernel(const float* g_lp, int64_t g_lp_stride, const float* g_ent, int64_t T,
                                                           const int* block_counts, int* rows, int* inv, int* n_rows) {
   __shared__ int part[4];
   __shared__ int before;
@@ -915,7 +915,7 @@ __global__ __launch_bounds__(256) void active_rows_kernel(const float* g_lp, int
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *n_rows = pos0;
 }
 
-__global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
+inline __global__ void fill_zero_kernel(uint32_t* p, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0u;
 }
 
@@ -1252,7 +1252,7 @@ LCE_DEV int64_t ppo_out_index(const PpoArgs& p, int64_t row, int64_t c) {
 
 // Per-token terms and unscaled gradients; workgroup (row, seg) reduces its segment of one row to
 // partials[row * segs + seg][0..6] = sums of (loss, entropy, clipped, -log ratio, dual-clipped, 1, kl) x mask.
-__global__ void ppo_terms_kernel(PpoArgs p) {
+inline __global__ void ppo_terms_kernel(PpoArgs p) {
   __shared__ float sh[8][256];
   float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int64_t row = (int64_t)blockIdx.x / p.segs;
@@ -1367,7 +1367,7 @@ __device__ inline void ppo_block_sum(double (&v)[NV], double (*sh)[256]) {
 // out: [0] loss = pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss, [1] pg_loss, [2] entropy_loss,
 //      [3] pg_clipfrac, [4] ppo_kl, [5] pg_clipfrac_lower, [6] sum(mask),
 //      [7] dp_size / denominator of the mode (1 / tokens or 1 / sequences included), [8] kl_loss
-__global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs, int64_t row_len, PpoAgg g,
+inline __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs, int64_t row_len, PpoAgg g,
                                   double* row_tot, float* row_weight, float* out) {
   __shared__ double sh[5][256];
   double a[5] = {0.0, 0.0, 0.0, 0.0, 0.0};  // clipped, -log ratio, dual-clipped, sum(mask), rows with tokens
@@ -1424,7 +1424,7 @@ __global__ void ppo_finish_kernel(const float* partials, int64_t rows, int segs,
   }
 }
 
-__global__ void ppo_scale_kernel(PpoArgs p, const float* row_weight) {
+inline __global__ void ppo_scale_kernel(PpoArgs p, const float* row_weight) {
   const int64_t row = (int64_t)blockIdx.x / p.segs;
   const int64_t c0 = ((int64_t)blockIdx.x % p.segs) * p.seg_len;
   const int64_t c1 = c0 + p.seg_len < p.row_len ? c0 + p.seg_len : p.row_len;

@@ -159,7 +159,7 @@ LCE_DEV void fwd16_body(const FwdArgs<typename Cfg::TIN>& p, char* lds) {
 // backward: d_logits tiles
 // ------------------------------------------------------------------------------------------------
 // per-position constants of the d_logits tiles (see DsArgs::tokc)
-__global__ void ds_token_consts_kernel(const int* rows, const int* n_rows, int64_t T, int64_t tpad, const float* g_lp, int64_t g_lp_stride,
+inline __global__ void ds_token_consts_kernel(const int* rows, const int* n_rows, int64_t T, int64_t tpad, const float* g_lp, int64_t g_lp_stride,
                                        float g_lp_scale, const float* g_ent, const float* maximum, const float* accumulate,
                                        const float* entropy_b, const int64_t* labels, int64_t vocab_offset, int64_t V, float rcp_tau,
                                        f32x4_t* tokc, int* tokl) {
