@@ -235,3 +235,16 @@ def test_metric_aggregation_kinds_of_ppo_loss():
     assert d["b"].aggregate() == 2.0 and d["a"].aggregation == AggregationType.MEAN
     with pytest.raises(ValueError, match="Unsupported loss mode: gpg"):
         C.get_policy_loss_fn("gpg")
+
+
+def test_tile_map_covers_every_tile_once_and_balances_the_xcds(tmp_path):
+    """The workgroup -> tile map of all tiled kernels, checked exhaustively on the host (tests/tile_map_check.cpp):
+    a hole or a duplicate would be a wrong result on the GPU, an uneven split over the 8 XCDs a slow one (a forward with
+    12 token tiles x 20 splits used to leave one XCD with 40 of the 240 workgroups and take two rounds)."""
+    import subprocess
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = str(tmp_path / "tile_map_check")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-o", exe, os.path.join(here, "tile_map_check.cpp")], check=True, timeout=300)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.startswith("ok"), r.stdout + r.stderr

@@ -17,8 +17,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-namespace lce {
+#include "tile_map.hpp"
 
+namespace lce {
 
 typedef __bf16 bf16_t;
 typedef bf16_t bf16x8_t __attribute__((ext_vector_type(8)));
@@ -508,60 +509,6 @@ struct GemmCore {
     // gfx9 s_waitcnt simm16: vmcnt[3:0] bits 3:0, expcnt bits 6:4, lgkmcnt bits 11:8, vmcnt[5:4] bits 15:14
     static_assert(N < 64, "vmcnt range");
     __builtin_amdgcn_s_waitcnt(((N & 0xF) | ((N >> 4) << 14)) | 0x0F70);
-  }
-};
-
-// XCD-aware decode of a flat workgroup id into a (row-tile, col-tile) pair.
-// Hardware deals workgroup ids round-robin over the 8 XCDs (each with its own L2), so ids with the
-// same (id % 8) share an L2.  We hand each XCD a contiguous range of "virtual" ids and cut the
-// virtual id space into blocks of 32 tiles shaped BR x (32/BR): the 32 workgroups resident on one
-// XCD then touch only BR row-tiles and 32/BR col-tiles of the operands.
-struct TileMap {
-  int nrow_tiles, ncol_tiles;  // tiles along the "row" operand (blocks of BR) and "col" operand
-  int br, bc;                  // block shape, br * bc == 32
-  int nrb, ncb;                // blocks along rows / cols
-  int rows_fastest;            // 1: consecutive blocks walk the row dimension first
-  int total;                   // launched workgroups (multiple of 8)
-
-  // shape of the 32-tile blocks that one XCD works on: up to 8 tiles along the row side
-  __host__ __device__ __forceinline__ static int block_rows(int nrow_tiles) {
-    int br = 1;
-    while (br < 8 && br < nrow_tiles) br <<= 1;
-    return br;
-  }
-  // the same map over fewer row tiles (a count that only the device knows): its workgroups are the
-  // first `total` ids of the grid that was sized for the full map, the others have nothing to do
-  __device__ __forceinline__ TileMap with_rows(int rows) const { return make(rows, ncol_tiles, rows >= br ? br : block_rows(rows), rows_fastest); }
-
-  __host__ __device__ __forceinline__ static TileMap make(int nrow_tiles, int ncol_tiles, int br, int rows_fastest) {
-    TileMap t;
-    t.nrow_tiles = nrow_tiles;
-    t.ncol_tiles = ncol_tiles;
-    t.br = br;
-    t.bc = 32 / br;
-    t.nrb = (nrow_tiles + t.br - 1) / t.br;
-    t.ncb = (ncol_tiles + t.bc - 1) / t.bc;
-    t.rows_fastest = rows_fastest;
-    t.total = t.nrb * t.ncb * 32;
-    return t;
-  }
-  // returns false when the slot is padding (no tile)
-  __device__ __forceinline__ bool decode(int bid, int& rt, int& ct) const {
-    if (bid >= total) return false;
-    const int per_xcd = total >> 3;
-    const int vid = (bid & 7) * per_xcd + (bid >> 3);
-    const int blk = vid >> 5, within = vid & 31;
-    int rb, cb;
-    if (rows_fastest) {
-      rb = blk % nrb;
-      cb = blk / nrb;
-    } else {
-      cb = blk % ncb;
-      rb = blk / ncb;
-    }
-    rt = rb * br + within / bc;
-    ct = cb * bc + within % bc;
-    return rt < nrow_tiles && ct < ncol_tiles;
   }
 };
 

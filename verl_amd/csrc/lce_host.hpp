@@ -191,21 +191,23 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
 }
 
 // Vocabulary splits of the forward with 256-token tiles.  A workgroup owns one (token tile, split) pair and walks the
-// split's vocabulary tiles itself, so the launch takes ceil(workgroups / CUs) rounds of ceil(tiles / splits) tiles
-// each: pick the split count with the fewest tile-times (ties: fewer splits, fewer partials to merge), among the
-// multiples of the XCD block's width `bc`: the 32 workgroups that share an L2 then cover 32 / bc token tiles x bc
-// splits and fetch each operand slab once for several of them.  (One split per token tile, which ties on tile-times
-// from 256 token tiles on, leaves every workgroup of an XCD with its own 256 rows of hidden: measured 440 instead of
-// 1300 TFLOP/s at 65536 and at 262144 tokens.)  With 48 token tiles (12288 tokens) eight splits are 384 workgroups =
-// two rounds of 75 tiles; sixteen splits give three rounds of 38.
+// split's vocabulary tiles itself, and the tile map gives every XCD the same number of workgroups, so the launch takes
+// ceil(workgroups / CUs) rounds of ceil(tiles / splits) tiles each: pick the split count with the fewest tile-times,
+// counting a quarter of a tile per workgroup for its ramp-up and its partial results (so ties go to fewer splits), from
+// the XCD block's width `bc` on: the 32 workgroups that share an L2 then cover 32 / bc token tiles x bc splits and fetch
+// each operand slab once for several of them.  (One split per token tile, which ties on tile-times from 256 token tiles
+// on, leaves every workgroup of an XCD with its own 256 rows of hidden: measured 440 instead of 1300 TFLOP/s at 65536
+// and at 262144 tokens.)  With 48 token tiles (12288 tokens) eight splits are 384 workgroups = two rounds of 75 tiles;
+// sixteen splits give three rounds of 38.
 constexpr int kNumCUs = 256;
 int forward_splits_256(int ntt, int nvt) {
   const int bc = 32 / block_rows(ntt);
   int best = bc;
   int64_t best_cost = -1;
-  for (int S = bc; S <= 256 && (S <= nvt || S == bc); S += bc) {
-    const int64_t rounds = ((int64_t)ntt * S + kNumCUs - 1) / kNumCUs;
-    const int64_t cost = rounds * ((nvt + S - 1) / S);
+  for (int S = bc; S <= 256 && (S <= nvt || S == bc); ++S) {
+    const int64_t per_xcd = ((int64_t)ntt * S + 7) / 8;
+    const int64_t rounds = (per_xcd + kNumCUs / 8 - 1) / (kNumCUs / 8);
+    const int64_t cost = rounds * (4 * ((nvt + S - 1) / S) + 1);
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = S; }
   }
   return best;
