@@ -20,7 +20,7 @@ def _case(seed):
     T = rnd.choice([1, 2, 31, 64, 255, 256, 257, 300, 511, 777, 1024, 1500, 2049])
     H = 128 * rnd.choice([1, 2, 3, 5, 8])
     V = rnd.choice([2, 17, 255, 256, 257, 1000, 4099, 8192, 12345, 20011])
-    if seed >= 1000:  # many tokens: the backward's 16x16x32 tiles (from 4096 tokens), ragged against their 256 x 256 tiles
+    if seed >= 1000:  # many tokens, ragged against the 256 x 256 tiles of the backward's 16x16x32 loop (the default beyond 1280 tokens)
         T = rnd.choice([4096, 4097, 4500, 5000, 8191, 9001])
         H = 128 * rnd.choice([1, 2, 3])
         V = rnd.choice([255, 257, 1000, 4099, 12345])

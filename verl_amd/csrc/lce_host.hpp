@@ -35,9 +35,8 @@ extern std::vector<hipEvent_t> prof_pool;
 // four-wave 16x16x32 loop (variant 5) above the token counts below.
 constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2, kVariantCore16 = 5;
 // variant 5 is the default above these token counts (measured at H=3584, V=152064: the forward gains 2-6% from 1024
-// tokens on; forward + backward breaks even at 4096 tokens, where the 32x32x16 path still saves the transpose of W, and
-// gains 4.5% at 8192)
-constexpr int64_t kCore16MinTokensFwd = 512, kCore16MinTokensBwd = 4096;
+// tokens on; forward + backward is 2% slower with it at 1024 tokens, 2% faster at 1536 and 2048, 4% at 3072)
+constexpr int64_t kCore16MinTokensFwd = 512, kCore16MinTokensBwd = 1280;
 struct Tuning {
   int variant_fwd = kDefaultVariantFwd, variant_bwd = kDefaultVariantBwd;
   bool variant_forced = false;   // lce_set_variant was called: no size-based choice of the tile
