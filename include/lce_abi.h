@@ -53,8 +53,9 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
 /* The same forward for callers that cannot allocate device memory and have no workspace to hand over (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
  * partial statistics go to a buffer of LCE_STATIC_SCRATCH_BYTES that is part of the library's own device image (one
- * copy per GPU, held until the process ends); the call allocates nothing and returns LCE_E_WORKSPACE when
- * lce_forward_workspace_bytes(T, H, V, dtype) exceeds that size (beyond about 116000 tokens).  All calls on one GPU share the
+ * copy per GPU, held until the process ends); the call allocates nothing, uses at most as many vocabulary splits as the
+ * buffer has room for (so its results may differ from lce_forward's in the last bits of the fp32 sums) and returns
+ * LCE_E_WORKSPACE when there is no room for four (beyond about 116000 tokens).  All calls on one GPU share the
  * buffer: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  The first call on
  * a device looks the buffer's address up, so make one call outside a graph capture before capturing. */
 #define LCE_STATIC_SCRATCH_BYTES (8u << 20)

@@ -52,6 +52,23 @@ def test_static_scratch_forward_matches_workspace_forward_twice_in_a_row():
         assert torch.isfinite(got[0]).all() and torch.isfinite(got[1]).all()
 
 
+def test_static_scratch_forward_where_the_buffer_limits_the_split_count():
+    """13312 tokens against 152064 vocabulary rows: the workspace forward cuts the vocabulary into 54 splits (11.5 MB of
+    partial statistics), the 8 MiB buffer has room for 39.  Another partition of the same fp32 sums: equal to 1e-5
+    (relative to the largest value), not bit for bit."""
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V = 13312, 128, 152064
+    assert lib.lce_forward_workspace_bytes(T, H, V, _abi.DTYPE_BF16) > (8 << 20)
+    h, w, y = _inputs(T, H, V, 3)
+    got = _forward(lib, _abi, h, w, y, 0.9, static=True)
+    want = _forward(lib, _abi, h, w, y, 0.9, static=False)
+    for a, b in zip(got, want):
+        assert torch.isfinite(a).all()
+        assert (a - b).abs().max().item() <= 1e-5 * max(1.0, b.abs().max().item())
+
+
 def test_static_scratch_forward_rejects_sizes_beyond_its_buffer():
     from verl_amd import _abi
 

@@ -154,17 +154,23 @@ int lce_profile_read(double* total_ms, int64_t* launches, int reset) {
   return LCE_OK;
 }
 
+// bytes of forward workspace when at most max_splits vocabulary splits are used: their partial statistics [S][T][4] fp32,
+// the label logits [T] and (for the reductions) the per-token log-probs [T]
+static size_t forward_workspace_need(int64_t T, int64_t V, int max_splits) {
+  if (T <= 0) return 256;
+  return align256((size_t)forward_splits_upper_bound(T, V > 0 ? V : 1, max_splits) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
+}
+
 size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
   (void)H; (void)dtype;
-  if (T <= 0) return 256;
-  return align256((size_t)forward_splits_upper_bound(T, V > 0 ? V : 1) * (size_t)T * 16) + 2 * align256((size_t)T * 4);
+  return forward_workspace_need(T, V, kMaxSplits);
 }
 
 // shared body of lce_forward and lce_forward_shard
 static int forward_entry(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
                          int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
                          float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
-                         void* stream, int64_t label_offset, float* shard_out) {
+                         void* stream, int64_t label_offset, float* shard_out, int max_splits = kMaxSplits) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -176,8 +182,8 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     return LCE_OK;
   }
   if (!shard_out && (!logprobs || !entropy || !maximum || !accumulate || !entropy_b)) return fail(LCE_E_ARG, "null output pointer");
-  if (!workspace || workspace_bytes < lce_forward_workspace_bytes(T, H, V, dtype))
-    return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, lce_forward_workspace_bytes(T, H, V, dtype));
+  if (!workspace || workspace_bytes < forward_workspace_need(T, V, max_splits))
+    return fail(LCE_E_WORKSPACE, "forward workspace too small: %zu < %zu", workspace_bytes, forward_workspace_need(T, V, max_splits));
   char* ws = static_cast<char*>(workspace);
   const Tuning tu = tuning_snapshot();
   int sel = tu.variant_fwd;
@@ -191,7 +197,7 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 2;
   }
   return kForward[dtype](sel, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum,
-                         accumulate, entropy_b, ws, st, label_offset, shard_out);
+                         accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits);
 }
 
 int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
@@ -206,17 +212,24 @@ int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int6
                        int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy, float* maximum,
                        float* accumulate, float* entropy_b, void* stream) {
   if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
-  const size_t need = lce_forward_workspace_bytes(T, H, V, dtype);
-  if (need > (size_t)LCE_STATIC_SCRATCH_BYTES)
-    return fail(LCE_E_WORKSPACE, "lce_forward_static: T=%lld needs %zu bytes of scratch, the built-in buffer holds %zu; use lce_forward with a workspace",
-                (long long)T, need, (size_t)LCE_STATIC_SCRATCH_BYTES);
+  // as many vocabulary splits as the buffer has room for (16 bytes per token and split, 8 more per token); the forward
+  // wants at least the four that fill an XCD's tile block
+  int max_splits = kMaxSplits;
+  if (T > 0) {
+    const size_t fixed = 2 * align256((size_t)T * 4) + 256;
+    const size_t room = (size_t)LCE_STATIC_SCRATCH_BYTES > fixed ? ((size_t)LCE_STATIC_SCRATCH_BYTES - fixed) / ((size_t)T * 16) : 0;
+    if (room < 4)
+      return fail(LCE_E_WORKSPACE, "lce_forward_static: T=%lld needs %zu bytes of scratch, the built-in buffer holds %zu; use lce_forward with a workspace",
+                  (long long)T, fixed + (size_t)T * 64, (size_t)LCE_STATIC_SCRATCH_BYTES);
+    if (room < (size_t)kMaxSplits) max_splits = (int)room;
+  }
   void* ws = nullptr;
   const int rc = static_scratch(&ws);
   if (rc) return rc;
   // (what must start at zero, the label logits, is cleared by a fill kernel inside the forward: nothing of the previous
   // call's contents is read)
   return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
-                       accumulate, entropy_b, ws, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr);
+                       accumulate, entropy_b, ws, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr, max_splits);
 }
 
 int lce_forward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,

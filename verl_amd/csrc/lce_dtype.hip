@@ -28,7 +28,7 @@ namespace lce_shared {
 int TU_FN(forward)(int sel, LCE_FWD_PARAMS) {
 #define LCE_RUN(Vt)                                                                                                          \
   return forward_impl<typename Vt<TuT>::Cfg>((const TuT*)h, ldh, (const TuT*)W, ldw, labels, T, H, V, temperature, reduction, \
-                                             lp, ent, mx, ac, eb, ws, st, label_offset, shard_out)
+                                             lp, ent, mx, ac, eb, ws, st, label_offset, shard_out, max_splits)
   switch (sel) {
     case 0: LCE_RUN(Variant0);
     case 1: LCE_RUN(Variant1);

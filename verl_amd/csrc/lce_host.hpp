@@ -60,7 +60,7 @@ enum { kSelT64 = 6, kSelT128 = 7 };
 #define LCE_FWD_PARAMS                                                                                                      \
   const void *h, int64_t ldh, const void *W, int64_t ldw, const int64_t *labels, int64_t T, int64_t H, int64_t V,          \
       float temperature, int reduction, float *lp, float *ent, float *mx, float *ac, float *eb, char *ws, hipStream_t st,   \
-      int64_t label_offset, float *shard_out
+      int64_t label_offset, float *shard_out, int max_splits
 #define LCE_BWD_PARAMS                                                                                                      \
   const void *h, int64_t ldh, const void *W, int64_t ldw, const int64_t *labels, int64_t T, int64_t H, int64_t V,          \
       float temperature, int reduction, const float *mx, const float *ac, const float *eb, const float *glp,               \
@@ -199,11 +199,13 @@ int launch_gemm(const typename Cfg::TIN* A, int64_t lda, const typename Cfg::TIN
 // and at 262144 tokens.)  With 48 token tiles (12288 tokens) eight splits are 384 workgroups = two rounds of 75 tiles;
 // sixteen splits give three rounds of 38.
 constexpr int kNumCUs = 256;
-int forward_splits_256(int ntt, int nvt) {
+constexpr int kMaxSplits = 256;
+int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
   const int bc = 32 / block_rows(ntt);
+  if (max_splits < bc) return max_splits > 1 ? max_splits : 1;  // (a caller with very little room for partial results)
   int best = bc;
   int64_t best_cost = -1;
-  for (int S = bc; S <= 256 && (S <= nvt || S == bc); ++S) {
+  for (int S = bc; S <= max_splits && (S <= nvt || S == bc); ++S) {
     const int64_t per_xcd = ((int64_t)ntt * S + 7) / 8;
     const int64_t rounds = (per_xcd + kNumCUs / 8 - 1) / (kNumCUs / 8);
     const int64_t cost = rounds * (4 * ((nvt + S - 1) / S) + 1);
@@ -216,7 +218,7 @@ template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                  int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* logprobs, float* entropy,
                  float* maximum, float* accumulate, float* entropy_b, char* ws, hipStream_t st, int64_t label_offset = 0,
-                 float* shard_out = nullptr) {
+                 float* shard_out = nullptr, int max_splits = kMaxSplits) {
   // shard_out: W is one shard of a larger vocabulary starting at row label_offset; instead of the five
   // outputs the per-token partial (max, sum exp, sum logit*exp, label logit) goes to shard_out [T][4]
   typedef typename Cfg::TIN TIN;
@@ -225,8 +227,10 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   // splits: enough workgroups to fill 256 CUs, in multiples of the XCD block width
   const int br = block_rows(ntt), bc = 32 / br;
   const int nrb = (ntt + br - 1) / br;
-  int S = Cfg::BN == 256 ? forward_splits_256(ntt, nvt) : bc * ((8 + nrb - 1) / nrb);
+  // max_splits: the caller's workspace holds partial results of at most that many splits
+  int S = Cfg::BN == 256 ? forward_splits_256(ntt, nvt, max_splits) : bc * ((8 + nrb - 1) / nrb);
   if (S > nvt) S = nvt;
+  if (S > max_splits) S = max_splits;
   // The narrow token tiles serve the HBM-bound case (up to 128 tokens: one streaming read of W).  There each
   // split takes one contiguous range of rows, the same length for all, instead of whole tiles dealt round robin
   // (594 tiles over 256 splits would be 3 against 2, and a split's tiles would lie 256 tiles apart).  Measured
@@ -301,15 +305,15 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
 }
 
 // upper bound of the number of vocabulary splits forward_impl picks, over the token-tile widths in use
-int forward_splits_upper_bound(int64_t T, int64_t V) {
-  int best = forward_splits_256((int)((T + 255) / 256), (int)((V + 255) / 256));
+int forward_splits_upper_bound(int64_t T, int64_t V, int max_splits = kMaxSplits) {
+  int best = forward_splits_256((int)((T + 255) / 256), (int)((V + 255) / 256), max_splits);
   for (int bn = 64; bn <= 128; bn <<= 1) {
     const int ntt = (int)((T + bn - 1) / bn);
     const int br = block_rows(ntt), bc = 32 / br, nrb = (ntt + br - 1) / br;
     const int S = bc * ((8 + nrb - 1) / nrb);
     if (S > best) best = S;
   }
-  return best;
+  return best < max_splits ? best : max_splits;
 }
 
 struct BwdLayout {
