@@ -27,7 +27,7 @@ typedef short i16x4_lds_t __attribute__((ext_vector_type(4)));
 // column (i % 4) of the run that lane (i / 4) pointed at in each row.
 LCE_DEV u32x2_t tr_read_b64(const char* lds_addr) {
   const i16x4_lds_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (i16x4_lds_t __attribute__((address_space(3)))*)(uint32_t)(uintptr_t)lds_addr);
+      (i16x4_lds_t __attribute__((address_space(3)))*)(uintptr_t)(uint32_t)(uintptr_t)lds_addr);
   u32x2_t r;
   __builtin_memcpy(&r, &v, 8);
   return r;
