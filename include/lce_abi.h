@@ -66,7 +66,9 @@ int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int6
 /* Backward.  Replaces efficient_entropy_backward (verl/utils/kernel/kernels.py:1518-1729): its
  * d_logits kernel (:1380-1515) and the two vendor GEMMs per vocab split (:1714-1724).
  *   dlogprobs [T] fp32 (reduction none) or [1] fp32 (sum / mean); dentropy [T] fp32 or NULL (treated as zero)
- *   d_hidden [T, H] and d_weight [V, H], contiguous, in the input dtype.
+ *   d_hidden [T, H] and d_weight [V, H], contiguous, in the input dtype.  One of the two may be NULL (the reference
+ *   always computes both): that gradient is not wanted, e.g. d_weight for a frozen lm-head, and its GEMM, a third
+ *   of the backward's work, is left out; the other gradient is bit for bit what the full call gives.
  * The vocabulary is processed in chunks of `vchunk` columns (0 = library default, else a multiple
  * of 256); per chunk the gradient of the logits exists only as a [T, vchunk] tile pair in the
  * workspace.  Sums over the vocabulary (d_hidden) and over tokens (d_weight) are carried in fp32

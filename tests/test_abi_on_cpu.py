@@ -97,10 +97,14 @@ def test_signature_matches_reference():
     fsig = inspect.signature(kernels.efficient_entropy_forward)
     assert list(fsig.parameters) == ["hidden", "weight", "labels", "reduction", "temperature", "dist_process_group"]
     bsig = inspect.signature(kernels.efficient_entropy_backward)
-    assert list(bsig.parameters) == [
+    positional = [n for n, p in bsig.parameters.items() if p.kind is not inspect.Parameter.KEYWORD_ONLY]
+    assert positional == [
         "dlogprobs", "dentropy", "hidden", "weight", "labels", "maximum", "acc", "entropy_b", "reduction",
         "should_return_fp32_grad", "temperature", "dist_process_group",
     ]  # fmt: skip
+    # beyond the reference's: two keyword-only switches that default to the reference's behaviour (both gradients)
+    extras = {n: p.default for n, p in bsig.parameters.items() if p.kind is inspect.Parameter.KEYWORD_ONLY}
+    assert extras == {"need_d_hidden": True, "need_d_weight": True}
     assert kernels.get_entropy_reduction_enum_number("none") == 0
     assert kernels.get_entropy_reduction_enum_number("sum") == 1
     assert kernels.get_entropy_reduction_enum_number("mean") == 2

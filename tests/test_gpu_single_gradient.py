@@ -1,0 +1,94 @@
+"""Backward with only one gradient wanted (d_weight NULL for a frozen lm-head, d_hidden NULL for inputs without
+gradient): the remaining gradient is bit for bit what the full call returns, on every backward path (streaming kernels
+for few tokens, the 32x32 loop, the 16x16x32 loop, fp32 inputs, fp32 gradients, masked tokens, several chunks), and the
+autograd node asks only for what autograd needs."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+CASES = [
+    # T, H, V, dtype, vocab chunk, mask
+    (48, 256, 5003, torch.bfloat16, 0, "dense"),        # streaming kernels, 64-token shape
+    (100, 128, 9001, torch.float16, 4096, "random"),    # streaming kernels, 128-token shape, three chunks
+    (700, 256, 5003, torch.bfloat16, 0, "dense"),       # 32x32x16 loop
+    (700, 128, 4099, torch.float32, 1024, "prefix"),    # fp32 inputs, several chunks
+    (3000, 256, 5003, torch.bfloat16, 2048, "random"),  # 16x16x32 loop, W read in place, several chunks
+    (9001, 128, 1000, torch.float16, 0, "dense"),       # 16x16x32 loop, ragged token tiles
+]
+
+
+def _inputs(T, H, V, dtype, mask, seed=7):
+    g = torch.Generator().manual_seed(seed)
+    h = (torch.rand(T, H, generator=g) - 0.5).to(dtype).to(DEV)
+    w = ((torch.rand(V, H, generator=g) - 0.5) * (4.0 / H ** 0.5)).to(dtype).to(DEV)
+    y = torch.randint(0, V, (T,), generator=g).to(DEV)
+    g_lp = (torch.rand(T, generator=g) * 2 - 1).to(DEV)
+    g_ent = (torch.rand(T, generator=g) - 0.5).to(DEV)
+    if mask == "prefix":
+        g_lp[: T // 3] = 0
+        g_ent[: T // 3] = 0
+    elif mask == "random":
+        keep = (torch.rand(T, generator=g) < 0.6).to(DEV)
+        g_lp, g_ent = g_lp * keep, g_ent * keep
+    return h, w, y, g_lp, g_ent
+
+
+@pytest.mark.parametrize("fp32_grads", [False, True])
+@pytest.mark.parametrize("T,H,V,dtype,vchunk,mask", CASES)
+def test_one_gradient_equals_the_full_call(T, H, V, dtype, vchunk, mask, fp32_grads):
+    from verl_amd.utils.kernel import kernels
+
+    h, w, y, g_lp, g_ent = _inputs(T, H, V, dtype, mask)
+    kernels.set_vocab_chunk(vchunk)
+    try:
+        lp, ent, mx, acc, eb = kernels.efficient_entropy_forward(h, w, y, 0, 0.8)
+        args = (g_lp, g_ent, h, w, y, mx, acc, eb, 0, fp32_grads, 0.8, None)
+        dh, dw = kernels.efficient_entropy_backward(*args)
+        dh_only, none_w = kernels.efficient_entropy_backward(*args, need_d_weight=False)
+        none_h, dw_only = kernels.efficient_entropy_backward(*args, need_d_hidden=False)
+    finally:
+        kernels.set_vocab_chunk(0)
+    assert none_w is None and none_h is None
+    assert dh_only.dtype == dh.dtype and dw_only.dtype == dw.dtype
+    assert torch.equal(dh_only, dh), (dh_only.float() - dh.float()).abs().max().item()
+    assert torch.equal(dw_only, dw), (dw_only.float() - dw.float()).abs().max().item()
+    assert dh.float().abs().max() > 0 and dw.float().abs().max() > 0
+    assert kernels.efficient_entropy_backward(*args, need_d_hidden=False, need_d_weight=False) == (None, None)
+
+
+def test_autograd_asks_only_for_the_gradients_it_needs():
+    from verl_amd import linear_cross_entropy
+
+    T, H, V = 1500, 256, 5003
+    h, w, y, g_lp, g_ent = _inputs(T, H, V, torch.bfloat16, "dense", seed=11)
+
+    def grads(h_req, w_req):
+        hh = h.clone().requires_grad_(h_req)
+        ww = w.clone().requires_grad_(w_req)
+        lp, ent = linear_cross_entropy(hh, ww, y, 1.3, "none")
+        torch.autograd.backward((lp, ent), (g_lp, g_ent))
+        return hh.grad, ww.grad
+
+    dh, dw = grads(True, True)
+    dh_only, no_w = grads(True, False)   # a frozen lm-head
+    no_h, dw_only = grads(False, True)   # detached hidden states
+    assert no_w is None and no_h is None
+    assert torch.equal(dh_only, dh) and torch.equal(dw_only, dw)
+
+
+def test_both_gradients_null_is_an_error_through_the_abi():
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    T, H, V = 64, 128, 512
+    z = torch.zeros(V * H, device=DEV, dtype=torch.bfloat16)
+    f = torch.zeros(T, device=DEV)
+    y = torch.zeros(T, device=DEV, dtype=torch.int64)
+    n = lib.lce_backward_workspace_bytes(T, H, V, _abi.DTYPE_BF16, 0)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    rc = lib.lce_backward(z.data_ptr(), H, z.data_ptr(), H, y.data_ptr(), T, H, V, _abi.DTYPE_BF16, 1.0, 0, f.data_ptr(), f.data_ptr(),
+                          f.data_ptr(), f.data_ptr(), None, None, None, ws.data_ptr(), n, 0, None)
+    assert rc != 0 and b"nothing to compute" in lib.lce_last_error()

@@ -286,13 +286,14 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const size_t esz = esize(dtype);
-  if (!d_weight) return fail(LCE_E_ARG, "null d_weight");
+  if (!d_weight && !d_hidden) return fail(LCE_E_ARG, "null d_hidden and d_weight: nothing to compute");
   if (T == 0) {
+    if (!d_weight) return LCE_OK;
     const int64_t words = (int64_t)((size_t)V * H * (grads_f32 ? 4 : esz) / 4);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, st, reinterpret_cast<uint32_t*>(d_weight), words);
     return check_launch("fill_zero_kernel");
   }
-  if (!d_hidden || !maximum || !accumulate || !entropy_b || !dlogprobs) return fail(LCE_E_ARG, "null pointer");
+  if (!maximum || !accumulate || !entropy_b || !dlogprobs) return fail(LCE_E_ARG, "null pointer");
   if (!aligned16(d_hidden) || !aligned16(d_weight)) return fail(LCE_E_ARG, "gradients must be 16-byte aligned");
   if (vchunk < 0) return fail(LCE_E_ARG, "vchunk must be >= 0");
   const Tuning tu = tuning_snapshot();

@@ -468,13 +468,14 @@ int launch_ds_few_tokens(DsArgs<typename Cfg::TIN> d, int64_t T, int nvt, hipStr
 // Both gradient GEMMs of one vocabulary chunk of a backward with at most 128 tokens, as one launch of the streaming
 // kernels (few_tokens.hpp): d_weight rows of the chunk in the output dtype, d_hidden as L.ksplit fp32 partials.
 template <typename Cfg, typename TOUT, int KT>
-int launch_few_gemms(const FewArgs<typename Cfg::TIN>& q, hipStream_t st) {
+int launch_few_gemms(const FewArgs<typename Cfg::TIN>& q, bool with_dh, hipStream_t st) {
   typedef typename Cfg::TIN TIN;
   typedef FewShape<KT> S;
   const int n_ht = (int)((q.H + S::HW - 1) / S::HW);
   auto kern = lce_bwd_few_kernel<TIN, TOUT, KPerm<Cfg>, KT>;
   allow_lds(kern, S::LDS_BYTES);
-  hipLaunchKernelGGL(kern, dim3((unsigned)(q.n_dw + n_ht * q.ksplit)), dim3(256), S::LDS_BYTES, st, q);
+  // (q.n_dw = 0: no d_weight workgroups; without d_hidden the grid ends after them)
+  hipLaunchKernelGGL(kern, dim3((unsigned)(q.n_dw + (with_dh ? n_ht * q.ksplit : 0))), dim3(256), S::LDS_BYTES, st, q);
   return check_launch("lce_bwd_few_kernel");
 }
 
@@ -485,7 +486,10 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                   void* d_hidden, void* d_weight, bool grads_f32, char* ws, int64_t vchunk, hipStream_t st,
                   int64_t vocab_offset, const Tuning& tu) {
   // vocab_offset: W is the shard [vocab_offset, vocab_offset + V) of a larger vocabulary (labels are global ids)
+  // d_hidden or d_weight may be null (not both): that gradient is not wanted (a frozen lm-head, an input without
+  // gradient) and its GEMM, a third of the backward's work, is left out
   typedef typename Cfg::TIN TIN;
+  const bool need_dh = d_hidden != nullptr, need_dw = d_weight != nullptr;
   const BwdLayout L = bwd_layout(tu, T, H, V, sizeof(TIN), vchunk, KPerm<Cfg>::GT, KPerm<Cfg>::GV);
   TIN* dS[2] = {reinterpret_cast<TIN*>(ws + L.off_dS[0]), reinterpret_cast<TIN*>(ws + L.off_dS[1])};
   TIN* dST[2] = {reinterpret_cast<TIN*>(ws + L.off_dST[0]), reinterpret_cast<TIN*>(ws + L.off_dST[1])};
@@ -530,7 +534,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       lt.g_lp = coef; lt.g_stride = 1; lt.scale = 1.0f;
     }
     const int nblocks = L.sort_items / kSortBlock;
-    if (nblocks == 1) {
+    if (!need_dw) {
+      // (the tokens grouped by label serve the one-hot rows of d_weight only)
+    } else if (nblocks == 1) {
       hipLaunchKernelGGL(label_sort_single_kernel, dim3(1), dim3(256), 0, st, lt, rows, n_rows, T, L.sort_passes, skeys[0], svals[0],
                          skeys[1], svals[1]);
       if ((rc = check_launch("label_sort_single_kernel"))) return rc;
@@ -630,20 +636,23 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
           q.dS = dS[cc & 1]; q.ldS = L.ldS; q.Ht = Ht; q.ldHt = L.ldHt; q.W = W + v0 * ldw; q.ldw = ldw;
           q.vrows = vrows; q.ucols = kc; q.H = H;
           q.kt = T <= 64 ? 64 : 128; q.nt = (int)T; q.n_rows = n_rows;
-          q.dW = grads_f32 ? static_cast<void*>(static_cast<float*>(d_weight) + v0 * H) : static_cast<void*>(static_cast<TIN*>(d_weight) + v0 * H);
+          q.dW = !need_dw ? nullptr
+                 : grads_f32 ? static_cast<void*>(static_cast<float*>(d_weight) + v0 * H) : static_cast<void*>(static_cast<TIN*>(d_weight) + v0 * H);
           q.dHp = dHacc; q.part_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
           q.ksplit = L.ksplit; q.kslice = round_up((q.ucols + L.ksplit - 1) / L.ksplit, 64);
           q.accumulate = cc == 0 ? 0 : 1;
-          q.n_dw = (int)(q.ucols / 64);
+          q.n_dw = need_dw ? (int)(q.ucols / 64) : 0;
           ProfScope prof(PC_BWD_CHUNK, st);
-          if (T <= 64) rc = grads_f32 ? launch_few_gemms<Cfg, float, 64>(q, st) : launch_few_gemms<Cfg, TIN, 64>(q, st);
-          else rc = grads_f32 ? launch_few_gemms<Cfg, float, 128>(q, st) : launch_few_gemms<Cfg, TIN, 128>(q, st);
+          if (T <= 64) rc = grads_f32 ? launch_few_gemms<Cfg, float, 64>(q, need_dh, st) : launch_few_gemms<Cfg, TIN, 64>(q, need_dh, st);
+          else rc = grads_f32 ? launch_few_gemms<Cfg, float, 128>(q, need_dh, st) : launch_few_gemms<Cfg, TIN, 128>(q, need_dh, st);
           if (rc) return rc;
           few_done = true;
         }
       }
       if (!few_done) {
-        if (L.tn_dh) {
+        if (!need_dh) {
+          // (no d_hidden GEMM)
+        } else if (L.tn_dh) {
           // W as it lies in memory (K-major for this product), fetched with transposing LDS reads
           p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, W + v0 * ldw, ldw, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
           p.gh.tn = 2;
@@ -657,16 +666,18 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
           if ((rc = check_launch("transpose W"))) return rc;
           p.gh = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Wt, L.ldWt, T, H, kc, dHacc, H, nullptr, 0, cc == 0 ? 0 : 1);
         }
-        p.gh.m_dev = n_rows;
-        if (L.ksplit > 1) {
+        if (need_dh) p.gh.m_dev = n_rows;
+        if (need_dh && L.ksplit > 1) {
           p.gh.ksplit = L.ksplit;
           p.gh.kslice = round_up((kc + L.ksplit - 1) / L.ksplit, Cfg::BK);
           p.gh.cf_split_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
         }
         // d_weight[v0 : v0 + vrows][H] = dST[vrows][Tpad] . Ht[H][Tpad]^T   (written in the input dtype, or as fp32)
-        float* dw_f32 = grads_f32 ? static_cast<float*>(d_weight) + v0 * H : nullptr;
-        TIN* dw_t = grads_f32 ? nullptr : static_cast<TIN*>(d_weight) + v0 * H;
-        if (L.tn) {
+        float* dw_f32 = need_dw && grads_f32 ? static_cast<float*>(d_weight) + v0 * H : nullptr;
+        TIN* dw_t = need_dw && !grads_f32 ? static_cast<TIN*>(d_weight) + v0 * H : nullptr;
+        if (!need_dw) {
+          // (no d_weight GEMM)
+        } else if (L.tn) {
           // d_weight[v0 : v0 + vrows][H] = dS[tokens][vrows]^T . hidden[tokens][H], both operands K-major
           p.gw = make_gemm_args<Cfg>(dS[cc & 1], L.ldS, Ht, L.ldHt, vrows, H, round_up(T, 64), dw_f32, H, dw_t, H, grads_f32 ? 0 : 2);
           p.gw.tn = 1;
@@ -676,11 +687,16 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
           p.gw = make_gemm_args<Cfg>(dST[cc & 1], L.ldST, Ht, L.ldHt, vrows, H, L.tpad, dw_f32, H, dw_t, H, grads_f32 ? 0 : 2);
           p.gw.k_dev = n_rows; p.gw.k_gran = KPerm<Cfg>::GT;
         }
-        p.n_gh = p.gh.map.total * L.ksplit;
-        p.n_gw = p.gw.map.total;
-        if (p.gh.kslice > p.gw.K) {  // longer tiles go first
+        p.n_gh = need_dh ? p.gh.map.total * L.ksplit : 0;
+        p.n_gw = need_dw ? p.gw.map.total : 0;
+        if (need_dh && need_dw && p.gh.kslice > p.gw.K) {  // longer tiles go first
           std::swap(p.gh, p.gw);
           std::swap(p.n_gh, p.n_gw);
+          swapped = true;
+        } else if (!need_dw) {  // an only GEMM sits in the first slot
+          p.gw = p.gh;
+          p.n_gw = p.n_gh;
+          p.n_gh = 0;
           swapped = true;
         }
       }
@@ -713,7 +729,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     launch_chunk(p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
   }
-  {
+  if (need_dh) {
     // d_hidden = ordered sum of the fp32 partials, rounded once; zero rows for tokens without gradient
     ProfScope prof(PC_DH_FINISH, st);
     int64_t blocks = (T * (H / 4) + 255) / 256;
@@ -727,7 +743,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                          static_cast<TIN*>(d_hidden), lt, W, ldw);
     if ((rc = check_launch("dh_finish_kernel"))) return rc;
   }
-  if (L.sort_items) {
+  if (L.sort_items && need_dw) {
     // one-hot part of d_weight: every chunk's rows hold their softmax terms by now
     ProfScope prof(PC_LABEL_ROWS, st);
     const int res = L.sort_passes & 1;

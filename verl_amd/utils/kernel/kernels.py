@@ -171,8 +171,17 @@ def efficient_entropy_backward(
     should_return_fp32_grad: bool = False,
     temperature: typing.Optional[float] = 1.0,
     dist_process_group=None,
+    *,
+    need_d_hidden: bool = True,
+    need_d_weight: bool = True,
 ) -> list[torch.Tensor]:
-    """Returns (d_hidden, d_weight) in ``hidden.dtype`` (fp32 when ``should_return_fp32_grad``)."""
+    """Returns (d_hidden, d_weight) in ``hidden.dtype`` (fp32 when ``should_return_fp32_grad``).
+
+    ``need_d_hidden`` / ``need_d_weight`` (not in the reference, which always computes both): ``False`` leaves that
+    gradient's GEMM out, a third of the backward's work, and returns ``None`` in its place, e.g. for a frozen lm-head
+    under LoRA."""
+    if not (need_d_hidden or need_d_weight):
+        return None, None
     _require_single_rank(dist_process_group)
     if _config._backward == BackwardEnum._Split_Dlogits_M:
         raise NotImplementedError("BackwardEnum._Split_Dlogits_M is not implemented yet")
@@ -196,10 +205,11 @@ def efficient_entropy_backward(
     # should_return_fp32_grad: both gradients straight from the fp32 accumulators, without the rounding to the input dtype
     # (verl/utils/kernel/kernels.py:1562-1567)
     grad_dtype = torch.float32 if should_return_fp32_grad else hidden.dtype
-    d_hidden = torch.empty((T, H), device=dev, dtype=grad_dtype)
-    d_weight = torch.empty((V, H), device=dev, dtype=grad_dtype)
+    d_hidden = torch.empty((T, H), device=dev, dtype=grad_dtype) if need_d_hidden else None
+    d_weight = torch.empty((V, H), device=dev, dtype=grad_dtype) if need_d_weight else None
     if T == 0:
-        d_weight.zero_()
+        if d_weight is not None:
+            d_weight.zero_()
     else:
         lib = _abi.load()
         with torch.cuda.device(dev):
@@ -210,7 +220,7 @@ def efficient_entropy_backward(
             rc = entry(
                 hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
                 code, float(temperature), reduction, maximum.data_ptr(), acc.data_ptr(), entropy_b.data_ptr(),
-                g_lp.data_ptr(), _abi.ptr(g_ent), d_hidden.data_ptr(), d_weight.data_ptr(), ws.data_ptr(), ws_bytes,
+                g_lp.data_ptr(), _abi.ptr(g_ent), _abi.ptr(d_hidden), _abi.ptr(d_weight), ws.data_ptr(), ws_bytes,
                 vchunk, _abi.current_stream(dev),
             )  # fmt: skip
             _abi.check(rc, "lce_backward")

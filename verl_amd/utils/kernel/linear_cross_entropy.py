@@ -57,12 +57,14 @@ class LinearCrossEntropy(torch.autograd.Function):
         shape, mode, temperature, group = ctx.call
         if dlogprobs is None:  # only the entropy was used downstream
             dlogprobs = torch.zeros((rows.shape[0],) if mode == 0 else (), device=rows.device, dtype=torch.float32)
+        # a gradient that autograd does not ask for (a frozen lm-head under LoRA, detached hidden states) is not computed
+        need_hidden, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         d_rows, d_weight = kernels.efficient_entropy_backward(
             dlogprobs, dentropy, rows, weight, flat_labels, maximum, accumulate, entropy_b, mode,
             False,  # should_return_fp32_grad: autograd wants the inputs' dtype
-            temperature, group,
+            temperature, group, need_d_hidden=need_hidden, need_d_weight=need_weight,
         )  # fmt: skip
-        return d_rows.view(shape), d_weight, None, None, None, None
+        return (d_rows.view(shape) if d_rows is not None else None), d_weight, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply
