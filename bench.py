@@ -228,6 +228,8 @@ def main():
     ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
     ap.add_argument("--no-transposed-reads", action="store_true", help="diagnostic: d_weight GEMM from a vocab-major copy of the d_logits")
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE", help="diagnostic: lce_set_option(KEY, VALUE)")
+    ap.add_argument("--frozen-head", action="store_true",
+                    help="the weight takes no gradient (LoRA that leaves lm_head alone): the backward leaves the d_weight GEMM out")
     ap.add_argument("--print-state", action="store_true", help="print the library state that keys profiles/traffic.json and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -262,6 +264,8 @@ def main():
     T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload][:8]
     flags = {"variant": args.variant, "vchunk": args.vchunk, "split_backward": bool(args.split_backward),
              "options": sorted(args.option + (["3=0"] if args.no_transposed_reads else []) + (["2=1"] if args.dlogits_tokens_first else []))}
+    if args.frozen_head:
+        flags["frozen_head"] = True
     state = library_state(lib, T, H, V, flags)
     if args.print_state:
         print(json.dumps({"workload": args.workload, "state": state}), flush=True)
@@ -269,7 +273,7 @@ def main():
     fwd_only = len(WORKLOADS[args.workload]) > 8 and WORKLOADS[args.workload][8]
     g = torch.Generator(device=dev).manual_seed(1234 + 2)
     h = torch.randn(T, H, device=dev, generator=g).bfloat16().requires_grad_(True)
-    w = (torch.randn(V, H, device=dev, generator=g) * wstd).bfloat16().requires_grad_(True)
+    w = (torch.randn(V, H, device=dev, generator=g) * wstd).bfloat16().requires_grad_(not args.frozen_head)
     y = torch.randint(0, V, (T,), device=dev, generator=g)
     g_lp = torch.randn(T, device=dev, generator=g)
     g_ent = torch.randn(T, device=dev, generator=g)
@@ -365,10 +369,12 @@ def main():
     # algorithmic FLOPs per step of each MFMA kernel class (the recompute of the logits in the
     # backward is executed but not counted): forward 2*T*V*H; backward d_hidden + d_weight 4*Ta*V*H,
     # Ta = tokens with a non-zero upstream gradient (the others add exactly zero and are skipped)
-    algo = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": 4.0 * t_active}
+    # (--frozen-head: one gradient GEMM instead of two)
+    n_grads = 1.0 if args.frozen_head else 2.0
+    algo = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": 2.0 * n_grads * t_active}
     if args.split_backward:
         algo.update({"gemm_nt_kernel(d_hidden)": 2.0 * t_active, "gemm_nt_kernel(d_weight)": 2.0 * t_active})
-    executed = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": 6.0 * t_active, "gemm_nt_kernel(d_hidden)": 2.0 * t_active,
+    executed = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": (2.0 + 2.0 * n_grads) * t_active, "gemm_nt_kernel(d_hidden)": 2.0 * t_active,
                 "gemm_nt_kernel(d_weight)": 2.0 * t_active, "lce_bwd_ds_kernel": 2.0 * t_active}
     mfma = {k: v for k, v in kernels.items() if k in algo}
     dom = max(mfma, key=lambda k: mfma[k]["ms_per_step"])
@@ -429,18 +435,18 @@ def main():
     }
     # Algorithmic FLOPs of the step: forward 2*T*V*H, backward 4*Ta*V*H over the Ta tokens that carry an upstream gradient
     # (the mandated recompute of the logits is executed but not counted).  With Ta = T this is the reference's 6*T*V*H.
-    algorithmic = (2.0 * T + 4.0 * t_active) * V * H / (elapsed / args.steps)
+    algorithmic = (2.0 * T + 2.0 * n_grads * t_active) * V * H / (elapsed / args.steps)
     if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM:
         # few tokens: the step is four streaming passes over [V, H] in the input dtype (W read by the forward, by the
         # d_logits tiles and by the d_hidden GEMM; d_weight written), and HBM bounds it.  The backward's two launches
         # (d_logits tiles; both gradient GEMMs) account for three of the four.
         k = kernels["lce_bwd_chunk_kernel"]
-        nbytes = 3.0 * V * H * 2.0 / k["launches_per_step"]
+        nbytes = (1.0 + n_grads) * V * H * 2.0 / k["launches_per_step"]  # (W read twice, d_weight written; --frozen-head: W read twice)
         roofline = {"bound": "hbm", "kernel": "lce_bwd_chunk_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                     "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
                     "traffic": measured_traffic(args.workload, "lce_bwd_chunk_kernel", state),
                     "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes,
-                    "step_bytes": 4.0 * V * H * 2.0, "step_GBps": 4.0 * V * H * 2.0 / (elapsed / args.steps) / 1e9}
+                    "step_bytes": (2.0 + n_grads) * V * H * 2.0, "step_GBps": (2.0 + n_grads) * V * H * 2.0 / (elapsed / args.steps) / 1e9}
     out = {
         "metric": "fwd+bwd tokens/s, 7B lm-head logprob+entropy; % of bf16 MFMA peak",
         "value": tokens_per_s,
@@ -456,7 +462,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau,
-                   "pass": "fwd+ppo_loss+bwd" if ppo else "fwd+bwd", "tokens_with_gradient": t_active},
+                   "pass": ("fwd+ppo_loss+bwd" if ppo else "fwd+bwd") + (" (d_hidden only: frozen head)" if args.frozen_head else ""),
+                   "tokens_with_gradient": t_active},
         "memory": memory,
         "algorithmic_tflops": algorithmic / 1e12,
         "frac_of_bf16_peak": algorithmic / PEAK_BF16,
@@ -465,7 +472,7 @@ def main():
         "row_skip": t_active < T,
         "per_token_accounting_tflops": 6.0 * T * V * H / (elapsed / args.steps) / 1e12,
         # what the kernels execute: forward on T tokens, recompute + two GEMMs on the tokens with gradient
-        "executed_tflops": (2.0 * T + 6.0 * t_active) * V * H / (elapsed / args.steps) / 1e12,
+        "executed_tflops": (2.0 * T + (2.0 + 2.0 * n_grads) * t_active) * V * H / (elapsed / args.steps) / 1e12,
         "roofline": roofline,
         "kernels": kernels,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
