@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 7
+#define LCE_ABI_VERSION 8
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1, LCE_DTYPE_F16 = 2 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */

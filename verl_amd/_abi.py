@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LCE_LIBRARY_PATH") or os.path.join(_HERE, "lib", "liblce_gfx950.so")
 
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 # every symbol include/lce_abi.h declares: name -> (restype, argtypes)
 _c = ctypes
