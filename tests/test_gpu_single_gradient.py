@@ -59,6 +59,29 @@ def test_one_gradient_equals_the_full_call(T, H, V, dtype, vchunk, mask, fp32_gr
     assert kernels.efficient_entropy_backward(*args, need_d_hidden=False, need_d_weight=False) == (None, None)
 
 
+@pytest.mark.parametrize("seed", list(range(200, 216)) + list(range(1100, 1108)))
+def test_one_gradient_on_random_shapes(seed):
+    """The shapes of tests/test_gpu_random_shapes.py (ragged tokens and vocabularies, reductions, masks, chunk widths)."""
+    from tests.test_gpu_random_shapes import _case
+    from verl_amd.utils.kernel import kernels
+
+    dtype, T, H, V, tau, reduction, mask, vchunk = _case(seed)
+    h, w, y, g_lp, g_ent = _inputs(T, H, V, dtype, "random" if mask != "dense" else "dense", seed=seed)
+    mode = kernels.get_entropy_reduction_enum_number(reduction)
+    if mode != 0:
+        g_lp = torch.tensor(0.7, device=DEV)
+    kernels.set_vocab_chunk(vchunk)
+    try:
+        lp, ent, mx, acc, eb = kernels.efficient_entropy_forward(h, w, y, mode, tau)
+        args = (g_lp, g_ent, h, w, y, mx, acc, eb, mode, False, tau, None)
+        dh, dw = kernels.efficient_entropy_backward(*args)
+        dh_only, _ = kernels.efficient_entropy_backward(*args, need_d_weight=False)
+        _, dw_only = kernels.efficient_entropy_backward(*args, need_d_hidden=False)
+    finally:
+        kernels.set_vocab_chunk(0)
+    assert torch.equal(dh_only, dh) and torch.equal(dw_only, dw), (dtype, T, H, V, reduction, mask, vchunk)
+
+
 def test_autograd_asks_only_for_the_gradients_it_needs():
     from verl_amd import linear_cross_entropy
 
