@@ -67,6 +67,10 @@ def test_default_chunk_rule_and_workspace_budget():
         # few tokens: the whole vocabulary in one chunk (one single-buffered d_logits tile)
         few = lib.lce_backward_workspace_bytes(64, H, V, 0, 0)
         assert few == lib.lce_backward_workspace_bytes(64, H, V, 0, 152064)
+        # very many tokens: narrower chunks, so that the two d_logits buffers stay within 4 GiB
+        assert lib.lce_backward_workspace_bytes(65536, 5120, V, 0, 0) == lib.lce_backward_workspace_bytes(65536, 5120, V, 0, 8192)
+        assert lib.lce_backward_workspace_bytes(262144, 4096, 128256, 0, 0) == lib.lce_backward_workspace_bytes(262144, 4096, 128256, 0, 4096)
+        assert lib.lce_backward_workspace_bytes(1 << 21, 4096, 128256, 0, 0) == lib.lce_backward_workspace_bytes(1 << 21, 4096, 128256, 0, 2048)
         sizes = []
         for budget in (600 << 20, 1 << 30, 2 << 30, 1 << 40):
             kernels.set_workspace_budget(budget)

@@ -430,8 +430,8 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
 BwdLayout bwd_layout(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
     // Upper bound of the whole workspace: a quarter of one [T, V] tile plus one fp32 [V, H].  Below it the default is
-    // a chunk of 8192 columns, or wider while one d_logits buffer stays within 256 MiB (few tokens: the whole vocabulary
-    // in one chunk, which saves a pass over W per chunk).  Measured at config 2 on the 16x16x32 loop: 8192 columns cost
+    // a chunk of 8192 columns, wider while one d_logits buffer stays within 256 MiB (few tokens: the whole vocabulary
+    // in one chunk, which saves a pass over W per chunk), narrower once two such buffers would pass 4 GiB.  Measured at config 2 on the 16x16x32 loop: 8192 columns cost
     // 0.4% against the widest chunk the bound allows (56.2 against 56.0 ms per step) with 0.9 instead of 2.9 GiB of
     // workspace; 4096 columns cost 6%.  A byte budget (LCE_OPT_WORKSPACE_BUDGET) replaces the default rule: the widest
     // chunk whose workspace fits it, but never fewer than 2048 columns.
@@ -442,6 +442,11 @@ BwdLayout bwd_layout(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t e
     } else {
       int64_t cols = (((int64_t)256 << 20) / (T * (int64_t)esz)) / 256 * 256;
       if (cols < 8192) cols = 8192;
+      // very many tokens: the two d_logits buffers stay within 4 GiB (at 262144 tokens chunks of 4096 columns take as
+      // long as chunks of 8192, 567.1 against 567.2 ms per actor step, with 10.1 instead of 14.1 GiB of workspace: a
+      // launch is long enough there for its fixed costs not to show)
+      const int64_t cap = (((int64_t)2 << 30) / (T * (int64_t)esz)) / 256 * 256;
+      if (cols > cap) cols = cap < 2048 ? 2048 : cap;
       if (cols < vchunk) vchunk = cols;
     }
     while (vchunk > 2048 && (double)bwd_layout_for(tu, T, H, V, esz, vchunk, 256, 256).total + 512.0 > gate) vchunk -= 1024;
