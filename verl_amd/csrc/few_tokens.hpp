@@ -78,11 +78,13 @@ struct FewArgs {
 
 // ------------------------------------------------------------------------------------------------------------------
 // d_weight, few tokens.  Workgroup = 256 threads = 4 waves; it owns dS columns [u0, u0 + 64) and walks H in tiles of
-// 256; wave w multiplies columns 64w .. 64w+63 of the tile:  C[m = h][n = u] = sum_t Ht[t][h] * dS[t][u].
+// HW = 256 or 128 columns; a wave multiplies 64 columns of the tile with all 64 dS columns (HW = 256) or with 32 of
+// them (HW = 128: two waves side by side along each):  C[m = h][n = u] = sum_t Ht[t][h] * dS[t][u].
 // MFMA rows are assigned to h in pairs of blocks: block 2i'+b, row 4g+r  <->  h = 32i' + 8g + 4b + r, so a lane ends
-// up with 8 consecutive h for one u and a store instruction covers 16 rows x 64 bytes; with 256-column tiles and 16-bit
-// output a wave's 64 x 64 results pass through a tile of its own in LDS and leave it as whole 128-byte lines
-// (measured on the d_weight workgroups alone, 64 tokens, H=3584, V=152064: 243 -> 228 us, 4.48 -> 4.78 TB/s).
+// up with 8 consecutive h for one u.  With 16-bit output a wave's results pass through a tile of its own in LDS and
+// leave it as whole 128-byte lines, eight lanes per row (measured on the d_weight workgroups alone, H=3584, V=152064:
+// 64 tokens 243 -> 228 us, 4.48 -> 4.78 TB/s; 96 tokens 306 -> 296 us); fp32 output is stored from the registers,
+// 16 rows x 128 bytes per instruction.
 // ------------------------------------------------------------------------------------------------------------------
 template <typename TIN, typename TOUT, typename Perm, int KT, int HW>
 LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
@@ -90,12 +92,15 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
   static_assert(HW == 256 || HW == 128, "columns of a hidden tile");
   constexpr int KS = KT / 32;
   constexpr int RB = HW * 2, CPR = HW / 8;  // bytes and 16-byte chunks of a hidden tile's row
-  constexpr int WH = HW / 4, MI = WH / 16;  // columns and 16-row MFMA blocks of a wave
-  constexpr bool STAGE = sizeof(TOUT) == 2 && WH == 64;  // a wave's row piece is a whole 128-byte line: stores go through LDS
+  // waves: WAVES_H along the tile's columns x WAVES_U along the 64 dS columns; a wave owns 64 columns of the hidden tile
+  // (MI = 4 MFMA row blocks) and NJ blocks of 16 dS columns
+  constexpr int WH = 64, MI = 4, WAVES_H = HW / WH, WAVES_U = 4 / WAVES_H, NJ = 4 / WAVES_U;
+  constexpr bool STAGE = sizeof(TOUT) == 2;  // 16-bit output: a wave's row piece is one 128-byte line, stored through LDS
   char* sB = lds;                    // dS tile: KT rows x 128 bytes (64 columns), chunk c of row r at c ^ (r & 7)
   char* sA = lds + KT * 128;         // hidden tile: KT rows x RB bytes, chunk c of row r at c ^ fw_swz(r)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int g = lane >> 4, l16 = lane & 15, e = l16 >> 2, q = l16 & 3;
+  const int wh = wave % WAVES_H, wu = wave / WAVES_H;  // this wave's place along the hidden tile and along the dS columns
   const int64_t u0 = (int64_t)bid * 64;
 
   // dS tile -> LDS (KT * 8 chunks of 16 bytes)
@@ -124,11 +129,11 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
     }
   };
   fetch(0);
-  // output rows of this lane: dS column u0 + 16 j + l16
-  int64_t vrow[4];
+  // output rows of this lane: dS column u0 + 16 NJ wu + 16 j + l16
+  int64_t vrow[NJ];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t v = Perm::vocab_at(u0 + 16 * j + l16);
+  for (int j = 0; j < NJ; ++j) {
+    const int64_t v = Perm::vocab_at(u0 + 16 * NJ * wu + 16 * j + l16);
     vrow[j] = v < p.vrows ? v : -1;
   }
   // token positions that take part (a device-side count may cut the host's): rows beyond them are not read
@@ -140,12 +145,12 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
   // B fragments (dS) are the same for every h tile: they stay in registers (read once the tile has landed) unless 128
   // token positions meet 256-column tiles (registers)
   constexpr bool KEEP_B = KT <= 64 || HW <= 128;
-  u32x4_t bf[KEEP_B ? KS : 1][4];
-  auto read_b = [&](int ks, u32x4_t (&out)[4]) {
+  u32x4_t bf[KEEP_B ? KS : 1][NJ];
+  auto read_b = [&](int ks, u32x4_t (&out)[NJ]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // lanes (e, q) of group g address row 32 ks + 8 g + e (+4), columns 16 j + 4 q ..
-      const int r0 = 32 * ks + 8 * g + e, r1 = r0 + 4, col = 16 * j + 4 * q;
+    for (int j = 0; j < NJ; ++j) {
+      // lanes (e, q) of group g address row 32 ks + 8 g + e (+4), columns 16 NJ wu + 16 j + 4 q ..
+      const int r0 = 32 * ks + 8 * g + e, r1 = r0 + 4, col = 16 * NJ * wu + 16 * j + 4 * q;
       const u32x2_t lo = tr_read_b64(sB + r0 * 128 + (((col >> 3) ^ (r0 & 7)) * 16) + (col & 7) * 2);
       const u32x2_t hi = tr_read_b64(sB + r1 * 128 + (((col >> 3) ^ (r1 & 7)) * 16) + (col & 7) * 2);
       out[j] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
@@ -161,19 +166,19 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
       for (int ks = 0; ks < KS; ++ks) read_b(ks, bf[KEEP_B ? ks : 0]);
     }
     if (ht + 1 < n_ht) fetch((int64_t)(ht + 1) * HW);
-    f32x4_t acc[MI][4];
+    f32x4_t acc[MI][NJ];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks >= ks_n) break;
       u32x4_t af[MI];
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        // block i = 2i' + b: the run of lane q starts at column WH wave + 32 i' + 8 q + 4 b
-        const int col = WH * wave + 32 * (i >> 1) + 8 * q + 4 * (i & 1);
+        // block i = 2i' + b: the run of lane q starts at column WH wh + 32 i' + 8 q + 4 b
+        const int col = WH * wh + 32 * (i >> 1) + 8 * q + 4 * (i & 1);
         const int r0 = 32 * ks + 8 * g + e, r1 = r0 + 4;
         const u32x2_t lo = tr_read_b64(sA + r0 * RB + (((col >> 3) ^ fw_swz(r0)) * 16) + (col & 7) * 2);
         const u32x2_t hi = tr_read_b64(sA + r1 * RB + (((col >> 3) ^ fw_swz(r1)) * 16) + (col & 7) * 2);
@@ -183,15 +188,15 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) mma16<TIN>(acc[i][j], af[i], bf[KEEP_B ? ks : 0][j]);
+        for (int j = 0; j < NJ; ++j) mma16<TIN>(acc[i][j], af[i], bf[KEEP_B ? ks : 0][j]);
     }
     if constexpr (STAGE) {
-      // Whole 128-byte lines per store: the wave's 64 rows x 64 columns go through a tile of its own in LDS (16-byte
+      // Whole 128-byte lines per store: the wave's 16 NJ rows x 64 columns go through a tile of its own in LDS (16-byte
       // chunk c of row r at c ^ ((r / 2) % 8), so that the 16 rows x 4 chunks of one write fall into different banks)
       // and leave it eight rows at a time, eight lanes per row.  No barrier: LDS operations of one wave complete in order.
-      char* sC = lds + KT * 128 + KT * RB + wave * 8192;
+      char* sC = lds + KT * 128 + KT * RB + wave * (NJ * 2048);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int ip = 0; ip < MI / 2; ++ip) {
           float d[8];
@@ -200,20 +205,20 @@ LCE_DEV void dw_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
           const int row = 16 * j + l16, c = 4 * ip + g;
           store_run<TOUT, 8>(reinterpret_cast<TOUT*>(sC + row * 128 + ((c ^ ((row >> 1) & 7)) * 16)), d);
         }
-      const int64_t hw0 = (int64_t)ht * HW + WH * wave;
+      const int64_t hw0 = (int64_t)ht * HW + WH * wh;
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
+      for (int it = 0; it < NJ * 2; ++it) {
         const int row = it * 8 + (lane >> 3), pc = lane & 7, c = pc ^ ((row >> 1) & 7);
         const u32x4_t v = *reinterpret_cast<const u32x4_t*>(sC + row * 128 + pc * 16);
-        const int64_t vr = Perm::vocab_at(u0 + row), h = hw0 + c * 8;
+        const int64_t vr = Perm::vocab_at(u0 + 16 * NJ * wu + row), h = hw0 + c * 8;
         if (vr < p.vrows && h < p.H) *reinterpret_cast<u32x4_t*>(static_cast<TOUT*>(p.dW) + vr * p.H + h) = v;
       }
       continue;
     }
-    // lane (g, l16): rows h = h0 + WH wave + 32 i' + 8 g + (0..7) of output row vrow[j]
-    const int64_t hb = (int64_t)ht * HW + WH * wave + 8 * g;
+    // lane (g, l16): rows h = h0 + WH wh + 32 i' + 8 g + (0..7) of output row vrow[j]
+    const int64_t hb = (int64_t)ht * HW + WH * wh + 8 * g;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       if (vrow[j] < 0) continue;
 #pragma unroll
       for (int ip = 0; ip < MI / 2; ++ip) {
@@ -342,7 +347,7 @@ LCE_DEV void dh_few_tile(const FewArgs<TIN>& p, int bid, char* lds) {
 template <int KT>
 struct FewShape {
   static constexpr int NT = KT, HW = KT <= 64 ? 256 : 128, HW_DW = HW;
-  static constexpr int DW = KT * 128 + KT * HW_DW * 2 + (HW_DW == 256 ? 4 * 8192 : 0);  // (+ the waves' store tiles)
+  static constexpr int DW = KT * 128 + KT * HW_DW * 2 + HW_DW * 128;  // dS tile, hidden tile, the four waves' store tiles
   static constexpr int DH = 64 * HW * 2 + NT * 128;
   static constexpr int LDS_BYTES = DW > DH ? DW : DH;
 };
