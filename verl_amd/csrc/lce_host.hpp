@@ -465,8 +465,16 @@ int launch_ds_few_tokens(DsArgs<typename Cfg::TIN> d, int64_t T, int nvt, hipStr
   static_assert(SmallCfg::WM == Cfg::WM && SmallCfg::FM == Cfg::FM && SmallCfg::BM == Cfg::BM, "same vocabulary order in dS");
   const int ntt = (int)((T + SmallCfg::BN - 1) / SmallCfg::BN);
   d.map = TileMap::make(ntt, nvt, block_rows(ntt), 0);
+  unsigned grid = (unsigned)d.map.total;
+  if (ntt == 1) {
+    // one contiguous range of rows per workgroup, the same length for all and at most one workgroup per CU (measured
+    // on the kernel, 64 tokens, H=3584, V=152064: 594 tiles on 256 CUs, 3 against 2, took 215 us)
+    const int64_t pad_end = round_up(d.vrows, SmallCfg::WM);
+    d.range_rows = round_up((pad_end + kNumCUs - 1) / kNumCUs, SmallCfg::WM);
+    grid = (unsigned)((pad_end + d.range_rows - 1) / d.range_rows);
+  }
   allow_lds(lce_bwd_ds_kernel<SmallCfg>, SmallCfg::LDS_BYTES);
-  hipLaunchKernelGGL(lce_bwd_ds_kernel<SmallCfg>, dim3(d.map.total), dim3(SmallCfg::NTHREADS), SmallCfg::LDS_BYTES, st, d);
+  hipLaunchKernelGGL(lce_bwd_ds_kernel<SmallCfg>, dim3(grid), dim3(SmallCfg::NTHREADS), SmallCfg::LDS_BYTES, st, d);
   return check_launch("lce_bwd_ds_kernel");
 }
 
@@ -615,6 +623,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.label_outside = lt.labels != nullptr ? tu.label_outside : 0;
       d.tokc = tokc; d.tokl = tokl; d.lab0 = v0;
       d.strip = Cfg::CORE16 ? tu.ds_strip : 1;
+      d.range_rows = 0;
       if (Cfg::CORE16 && L.tn) {
         // the compact copy of hidden built for the d_weight GEMM: the tiles read it without a row gather
         d.h = Ht; d.ldh = L.ldHt; d.rows = nullptr;

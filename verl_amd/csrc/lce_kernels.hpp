@@ -327,6 +327,7 @@ struct DsArgs {
   const int* tokl;
   int64_t lab0;
   int strip;  // vocabulary tiles that one workgroup walks (the map's columns are strips)
+  int64_t range_rows;  // few tokens: > 0 = every workgroup of lce_bwd_ds_kernel takes that many vocabulary rows (a multiple of the wave tile's)
 };
 
 // The two gradient GEMMs sum over the vocabulary (d_hidden) and over the tokens (d_weight); any
@@ -491,18 +492,14 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
   }
 }
 
+// One 256-row vocabulary tile of the d_logits pass for the token tile at n0: rows m0 .. of the chunk, of which the
+// workgroup owns those below own_end (a multiple of the wave tile's rows; the rest belongs to a neighbour and is
+// neither read beyond the clamp nor written).
 template <typename Cfg>
-LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
-  const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;  // tokens that take part
-  int tt, vt;
-  // with a device-side token count the XCD-aware map is rebuilt over the token tiles that exist, so
-  // that they spread evenly over the XCDs (the host's map would leave whole XCDs without work)
-  const TileMap map = p.n_rows ? p.map.with_rows((int)((Tc + Cfg::BN - 1) / Cfg::BN)) : p.map;
-  if (!map.decode(bid, tt, vt)) return;
-  const int64_t n0 = (int64_t)tt * Cfg::BN, m0 = (int64_t)vt * Cfg::BM;
+LCE_DEV void ds_tile_at(const DsArgs<typename Cfg::TIN>& p, int64_t n0, int64_t m0, int64_t own_end, int64_t Tc, char* lds) {
   const int lane = threadIdx.x & 63, hh = lane >> 5, ln = lane & 31;
   GemmCore<Cfg> g;
-  g.init(p.W, p.ldw, m0, p.vrows, p.h, p.ldh, n0, Tc, p.rows);
+  g.init(p.W, p.ldw, m0, own_end < p.vrows ? own_end : p.vrows, p.h, p.ldh, n0, Tc, p.rows);
   f32x16_t acc[Cfg::FM][Cfg::FN];
   g.run(lds, p.H, acc);
 
@@ -520,9 +517,36 @@ LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   }
   const bool interior = vloc0 + Cfg::WM <= p.vrows && tok0 + Cfg::WN <= Tc;
   __syncthreads();  // every wave's slab loads have landed and its operand reads are done: LDS is free
+  if (vloc0 >= own_end) return;  // (a whole wave tile of the neighbour's rows; the caller's barriers are outside)
   char* stage_lds = lds + g.wave * DsStage<Cfg>::WAVE_BYTES;
   if (interior && __builtin_amdgcn_ballot_w64(has_label) == 0) ds_epilogue<Cfg, false>(p, acc, tok0, Tc, vloc0, hh, ln, stage_lds);
   else ds_epilogue<Cfg, true>(p, acc, tok0, Tc, vloc0, hh, ln, stage_lds);
+}
+
+template <typename Cfg>
+LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
+  const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;  // tokens that take part
+  if (p.range_rows > 0) {
+    // Few tokens (one token tile, HBM-bound): every workgroup takes one contiguous range of range_rows vocabulary rows,
+    // the same length for all, instead of whole 256-row tiles (594 tiles over 256 CUs would be 3 against 2).  The last
+    // tile of a range is clamped at the range's end: its surplus rows are repeats of one row in the loads, and the
+    // waves that hold only such rows store nothing.
+    if (Tc <= 0) return;  // no token takes part: nothing to read (the operand loads clamp to the last token) or to write
+    const int64_t pad_end = (p.vrows + Cfg::WM - 1) / Cfg::WM * Cfg::WM;  // (rows up to the wave tile are written as zeros)
+    const int64_t r0 = (int64_t)bid * p.range_rows;
+    const int64_t r1 = r0 + p.range_rows < pad_end ? r0 + p.range_rows : pad_end;
+    for (int64_t m0 = r0; m0 < r1; m0 += Cfg::BM) {
+      if (m0 > r0) __syncthreads();  // the staging tiles of the previous tile's epilogue are read out
+      ds_tile_at<Cfg>(p, 0, m0, r1, Tc, lds);
+    }
+    return;
+  }
+  int tt, vt;
+  // with a device-side token count the XCD-aware map is rebuilt over the token tiles that exist, so
+  // that they spread evenly over the XCDs (the host's map would leave whole XCDs without work)
+  const TileMap map = p.n_rows ? p.map.with_rows((int)((Tc + Cfg::BN - 1) / Cfg::BN)) : p.map;
+  if (!map.decode(bid, tt, vt)) return;
+  ds_tile_at<Cfg>(p, (int64_t)tt * Cfg::BN, (int64_t)vt * Cfg::BM, (int64_t)1 << 40, Tc, lds);
 }
 
 // ------------------------------------------------------------------------------------------------
