@@ -124,6 +124,35 @@ def cpu_baseline(seconds_budget: float = 20.0):
     }
 
 
+def unfused_context(h, w, y, tau, g_lp, g_ent):
+    """Forward + backward of the oracle's autograd restatement (`oracle.lce_oracle.lce_unfused_autograd`: one fp32
+    [T, V] logits tensor) on the GPU: milliseconds and peak extra device memory.  Any failure (memory) is reported, not raised."""
+    import torch
+
+    from oracle import lce_oracle as O
+
+    dev = h.device
+    try:
+        out = None
+        for _ in range(2):  # warm-up (hipBLASLt heuristics, allocator), then the timed run
+            del out
+            torch.cuda.synchronize()
+            base = torch.cuda.memory_allocated(dev)
+            torch.cuda.reset_peak_memory_stats(dev)
+            t0 = time.perf_counter()
+            out = O.lce_unfused_autograd(h, w, y, tau, g_lp, g_ent, torch.float32)
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3
+            peak = torch.cuda.max_memory_allocated(dev) - base
+        del out
+        torch.cuda.empty_cache()
+        return {"what": "reference test's torch path: fp32 [T, V] logits materialised, softmax + logsumexp + cross_entropy, autograd",
+                "fwd_bwd_ms": ms, "peak_extra_bytes": peak}
+    except Exception as e:  # noqa: BLE001
+        torch.cuda.empty_cache()
+        return {"error": f"{type(e).__name__}: {str(e)[:200]}"}
+
+
 PEAK_HBM = 8e12  # MI355X HBM3E peak, bytes/s
 
 LOGITS_WORKLOADS = {
@@ -215,19 +244,162 @@ def run_logits_workload(args, name):
     print(json.dumps(out), flush=True)
 
 
+CEILING_WORKLOAD = "mfma-ceiling"
+
+
+class _PowerSampler:
+    """Socket power (W) and shader clock (MHz) of GPU 0 sampled every 50 ms through amdsmi on a host thread; every
+    reading is None where the module or a field is missing."""
+
+    def __init__(self):
+        import threading
+
+        self.samples = []
+        self._stop = False
+        self.error = None
+        self._thread = threading.Thread(target=self._run, daemon=True)
+        self._thread.start()
+
+    def _run(self):
+        try:
+            try:
+                import amdsmi
+            except ImportError:
+                sys.path.insert(0, "/opt/rocm/share/amd_smi")
+                import amdsmi
+            amdsmi.amdsmi_init()
+            handle = amdsmi.amdsmi_get_processor_handles()[0]
+            try:
+                self.cap_watts = amdsmi.amdsmi_get_power_cap_info(handle).get("power_cap", 0) / 1e6
+            except Exception:
+                self.cap_watts = None
+            while not self._stop:
+                p = amdsmi.amdsmi_get_power_info(handle)
+                c = amdsmi.amdsmi_get_clock_info(handle, amdsmi.AmdSmiClkType.GFX)
+                watts = p.get("current_socket_power", p.get("average_socket_power"))
+                mhz = c.get("clk", c.get("cur_clk"))
+                self.samples.append((time.time(), watts if isinstance(watts, (int, float)) else None, mhz if isinstance(mhz, (int, float)) else None))
+                time.sleep(0.05)
+        except Exception as e:  # no amdsmi, no permission: the rates are still measured
+            self.error = f"{type(e).__name__}: {e}"
+
+    def window(self, t0, t1):
+        """Mean power and clock over the last 60 % of [t0, t1] (the governor has settled by then)."""
+        ta = t0 + 0.4 * (t1 - t0)
+        sel = [(w, c) for (t, w, c) in self.samples if ta <= t <= t1]
+        ws = [w for w, _ in sel if w is not None]
+        cs = [c for _, c in sel if c is not None]
+        return (sum(ws) / len(ws) if ws else None, sum(cs) / len(cs) if cs else None, len(sel))
+
+    def stop(self):
+        self._stop = True
+
+
+def run_mfma_ceiling(args):
+    """What plain bf16 GEMMs of this path's shapes sustain on THIS box: the library's 16x16x32 mainloop (`lce_gemm_nt`,
+    fp32 C; `lce_gemm_tn` for the K-major d_weight layout) next to torch.matmul (hipBLASLt, bf16 C), on all-zero operands
+    and on the benchmark's distributions (N(0,1) x N(0,0.02)), with socket power and shader clock sampled meanwhile.
+    The fused kernels cannot beat what the matrix pipes sustain on such data; this is the yardstick for them."""
+    import torch
+
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    sampler = _PowerSampler()
+    time.sleep(0.3)
+    T, H, V, vc = 16384, 3584, 152064, 8192
+    shapes = [
+        # name, M, N, K  (C[M, N] = A[M, K] . B[N, K]^T)
+        ("forward-like 16384 x 16384 x 3584", 16384, 16384, 3584),
+        ("d_logits tiles of one 8192-column chunk", T, vc, H),
+        ("d_hidden GEMM of one chunk", T, H, vc),
+        ("d_weight GEMM of one chunk", vc, H, T),
+    ]
+    g = torch.Generator(device=dev).manual_seed(99)
+    cases = []
+    seconds = 0.6
+
+    def timed(fn, flops):
+        fn(); fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); fn(); e1.record()
+        torch.cuda.synchronize()
+        reps = max(5, int(seconds * 1e3 / max(e0.elapsed_time(e1), 1e-3)))
+        t0 = time.time()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.time()
+        ms = e0.elapsed_time(e1) / reps
+        watts, mhz, n = sampler.window(t0, t1)
+        time.sleep(0.3)  # let the board cool between cases
+        return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "socket_watts": watts, "shader_mhz": mhz, "samples": n, "reps": reps}
+
+    for data in ("zeros", "randn x 0.02 randn"):
+        for name, M, N, K in shapes:
+            if data == "zeros":
+                A = torch.zeros(M, K, device=dev, dtype=torch.bfloat16)
+                B = torch.zeros(N, K, device=dev, dtype=torch.bfloat16)
+            else:
+                A = torch.randn(M, K, device=dev, generator=g).bfloat16()
+                B = (torch.randn(N, K, device=dev, generator=g) * 0.02).bfloat16()
+            flops = 2.0 * M * N * K
+            Cf = torch.empty(M, N, device=dev, dtype=torch.float32)
+            r = timed(lambda: _abi.check(lib.lce_gemm_nt(A.data_ptr(), K, B.data_ptr(), K, Cf.data_ptr(), N, M, N, K, 0, 3, st), "lce_gemm_nt"), flops)
+            cases.append({"shape": name, "M": M, "N": N, "K": K, "data": data, "engine": "lce_gemm_nt (16x16x32 loop, fp32 C)", **r})
+            del Cf
+            Cb = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+            Bt = B.t()
+            r = timed(lambda: torch.matmul(A, Bt, out=Cb), flops)
+            cases.append({"shape": name, "M": M, "N": N, "K": K, "data": data, "engine": "torch.matmul (hipBLASLt, bf16 C)", **r})
+            del Cb
+            if name.startswith("d_weight"):
+                # the layout the backward really uses: both operands K-major, A[K, M], B[K, N] (row strides in whole 256-column tiles)
+                At, Bk = A.t().contiguous(), B.t().contiguous()
+                Cf = torch.empty(M, N, device=dev, dtype=torch.float32)
+                r = timed(lambda: _abi.check(lib.lce_gemm_tn(At.data_ptr(), M, Bk.data_ptr(), N, Cf.data_ptr(), N, M, N, K, 3, st), "lce_gemm_tn"), flops)
+                cases.append({"shape": name, "M": M, "N": N, "K": K, "data": data, "engine": "lce_gemm_tn (16x16x32 loop, K-major operands, fp32 C)", **r})
+                del At, Bk, Cf
+            del A, B
+    sampler.stop()
+    rand = [c for c in cases if c["data"] != "zeros"]
+    best_lib = max(c["tflops"] for c in rand if c["engine"].startswith("lce_"))
+    best_blas = max(c["tflops"] for c in rand if c["engine"].startswith("torch"))
+    # time of one fwd+bwd step of the headline workload if its four GEMM-shaped passes (8*T*V*H executed FLOP) ran at these rates
+    step_flops = 8.0 * T * V * H
+    out = {
+        "metric": "plain bf16 GEMM rate on this box (yardstick for the fused kernels), random operands",
+        "value": max(best_lib, best_blas), "unit": "TFLOP/s", "n_gpus": 1, "steps": None, "warmup": None, "ms_per_step": None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": CEILING_WORKLOAD, "seconds_per_case": seconds},
+        "best_library_mainloop_tflops": best_lib, "best_hipblaslt_tflops": best_blas,
+        "headline_step_ms_at_best_rate": step_flops / (max(best_lib, best_blas) * 1e12) * 1e3,
+        "power_cap_watts": getattr(sampler, "cap_watts", None), "power_sampler_error": sampler.error,
+        "cases": cases,
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS) + sorted(LOGITS_WORKLOADS))
+    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS) + sorted(LOGITS_WORKLOADS) + [CEILING_WORKLOAD])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
     ap.add_argument("--split-backward", action="store_true", help="diagnostic: time the backward's three phases as separate launches")
     ap.add_argument("--dlogits-tokens-first", action="store_true", help="diagnostic: tile order of the d_logits pass")
-    ap.add_argument("--no-transposed-reads", action="store_true", help="diagnostic: d_weight GEMM from a vocab-major copy of the d_logits")
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE", help="diagnostic: lce_set_option(KEY, VALUE)")
+    ap.add_argument("--no-unfused-context", action="store_true",
+                    help="skip the context figure: the reference test's unfused torch path (fp32 [T, V] logits, autograd) timed on the same GPU")
     ap.add_argument("--frozen-head", action="store_true",
                     help="the weight takes no gradient (LoRA that leaves lm_head alone): the backward leaves the d_weight GEMM out")
     ap.add_argument("--print-state", action="store_true", help="print the library state that keys profiles/traffic.json and exit")
@@ -240,6 +412,9 @@ def main():
     if args.workload in LOGITS_WORKLOADS:
         run_logits_workload(args, args.workload)
         return
+    if args.workload == CEILING_WORKLOAD:
+        run_mfma_ceiling(args)
+        return
 
     import torch
 
@@ -251,8 +426,6 @@ def main():
         _abi.check(lib.lce_set_variant(args.variant), "lce_set_variant")
     if args.split_backward:
         _abi.check(lib.lce_set_option(1, 1), "lce_set_option")
-    if args.no_transposed_reads:
-        _abi.check(lib.lce_set_option(3, 0), "lce_set_option")
     if args.dlogits_tokens_first:
         _abi.check(lib.lce_set_option(2, 1), "lce_set_option")
     for kv in args.option:
@@ -263,7 +436,7 @@ def main():
     dev = torch.device("cuda:0")
     T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload][:8]
     flags = {"variant": args.variant, "vchunk": args.vchunk, "split_backward": bool(args.split_backward),
-             "options": sorted(args.option + (["3=0"] if args.no_transposed_reads else []) + (["2=1"] if args.dlogits_tokens_first else []))}
+             "options": sorted(args.option + (["2=1"] if args.dlogits_tokens_first else []))}
     if args.frozen_head:
         flags["frozen_head"] = True
     state = library_state(lib, T, H, V, flags)
@@ -365,6 +538,13 @@ def main():
     prof = _abi.profile_read(reset=True)
     lib.lce_profile_enable(0)
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
+    # Context only, never the target: the unfused torch path of the reference's own test (materialised fp32 [T, V] logits,
+    # softmax, logsumexp, cross_entropy, autograd; tests/utils/test_linear_cross_entropy.py:49-62,290-349 prints the same
+    # pair of figures) on the same GPU and inputs, after everything that is timed: one warm-up, then one timed forward + backward.
+    unfused = None
+    if not args.no_unfused_context and not fwd_only and not ppo and not args.frozen_head and T * V <= 16384 * 152064:
+        unfused = unfused_context(h, w, y, tau, g_lp, g_ent)
+
     # the dominant kernel (largest share of the step) and its algorithmic FLOPs per launch:
     # algorithmic FLOPs per step of each MFMA kernel class (the recompute of the logits in the
     # backward is executed but not counted): forward 2*T*V*H; backward d_hidden + d_weight 4*Ta*V*H,
@@ -475,6 +655,7 @@ def main():
         "executed_tflops": (2.0 * T + (2.0 + 2.0 * n_grads) * t_active) * V * H / (elapsed / args.steps) / 1e12,
         "roofline": roofline,
         "kernels": kernels,
+        "unfused_torch_same_gpu": unfused,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
     }
     print(json.dumps(out), flush=True)

@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 8
+#define LCE_ABI_VERSION 9
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1, LCE_DTYPE_F16 = 2 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -27,7 +27,8 @@ enum {
   LCE_OK = 0,
   LCE_E_ARG = -1,       /* bad shape, dtype, alignment or null pointer */
   LCE_E_WORKSPACE = -2, /* workspace too small */
-  LCE_E_LAUNCH = -3     /* HIP reported an error at launch */
+  LCE_E_LAUNCH = -3,    /* HIP reported an error at launch */
+  LCE_E_BUSY = -4       /* lce_forward_static: the built-in scratch buffer is still in use by a call on another stream */
 };
 
 int lce_abi_version(void);
@@ -56,8 +57,12 @@ int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw
  * copy per GPU, held until the process ends); the call allocates nothing, uses at most as many vocabulary splits as the
  * buffer has room for (so its results may differ from lce_forward's in the last bits of the fp32 sums) and returns
  * LCE_E_WORKSPACE when there is no room for four (beyond about 116000 tokens).  All calls on one GPU share the
- * buffer: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  The first call on
- * a device looks the buffer's address up, so make one call outside a graph capture before capturing. */
+ * buffer, so calls that overlap on one GPU would race for it; calls on one stream do not overlap.  The library keeps, per
+ * GPU, the stream of the last call and an event behind its last kernel: a call on another stream while that one has not
+ * finished returns LCE_E_BUSY and launches nothing (host-side check, no device work).  Calls recorded into a HIP graph
+ * are neither checked nor remembered: the order of a graph's nodes is the caller's.  The first call on a device looks
+ * the buffer's address up and creates that event, so make one call outside a graph capture before capturing; with
+ * lce_profile_enable(1) every call also creates timing events. */
 #define LCE_STATIC_SCRATCH_BYTES (8u << 20)
 int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T, int64_t H,
                        int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy, float* maximum,
@@ -131,8 +136,14 @@ int lce_logits_backward(const void* logits, int64_t ldl, const int64_t* labels, 
 /* Replaces calculate_sum_pi_squared_from_logits (verl/utils/torch_functional.py:687-703; called on the actor's
  * logits at verl/workers/engine/fsdp/transformer_impl.py:1413,1513): out[r] = sum_v softmax(logits[r])_v ^ 2
  * = exp(logsumexp(2 z) - 2 logsumexp(z)), one pass over the row, fp32 arithmetic.  logits [R, V] row stride ldl;
- * out [R] fp32. */
-int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream);
+ * out [R] fp32; lse_out [R] fp32 or NULL: the rows' logsumexp, which lets the backward skip its own reduction pass. */
+int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, float* lse_out,
+                              void* stream);
+/* Its autograd twin (the reference's function is plain torch, hence differentiable): d_logits [R, V] (row stride ldd, dtype
+ * of the logits) = g[r] * 2 p (p - S_r), p = softmax(logits[r]), S_r = sum_v p_v^2.  g [R] fp32; lse / sum_pi2 [R] fp32 as
+ * the forward wrote them, or NULL (then both are recomputed from the row).  One read and one write of the rows. */
+int lce_logits_sum_pi_squared_backward(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, const float* lse,
+                                       const float* sum_pi2, const float* g, void* d_logits, int64_t ldd, void* stream);
 
 /* Consumer of the path's outputs: the clipped PPO policy loss with dual clip, any of agg_loss's aggregation
  * modes, the entropy bonus and the KL penalty against a reference policy.  Replaces, for the vanilla loss,
@@ -185,71 +196,66 @@ int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packe
                         float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
                         float* g_log_prob_packed, float* g_entropy_packed, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Diagnostic: C[M, N] (fp32, row stride ldc) = A[M, K] . B[N, K]^T with the library's MFMA
- * mainloop (the same code that the entry points above use).  K a multiple of 64 (bf16) / 32 (fp32).
- * No counterpart in the reference; exists so the mainloop can be tested and timed on its own. */
-int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
-                int64_t K, int dtype, int variant, void* stream);
-
-/* Diagnostic twin for K-major operands (bf16 only): C[M, N] = A[K, M]^T . B[K, N], the layout of the d_weight GEMM
- * (A = d_logits [tokens, vocab], B = hidden [tokens, H]).  K a multiple of 64; lda >= M and ldb >= N rounded up to 256. */
-int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
-                void* stream);
-
-/* Tuning hook: selects the tile / LDS-ring configuration used by the mainloops of forward and backward,
- * 0 <= variant < lce_num_variants(); -1 restores the defaults (which differ between the two).  Process-wide. */
-int lce_set_variant(int variant);
-int lce_num_variants(void);
-/* Diagnostic options (process-wide).  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and
- * the two gradient GEMMs of a backward chunk as three kernels instead of one (for per-phase timing).
- * LCE_OPT_DLOGITS_TOKENS_FIRST: order in which an XCD's consecutive blocks of d_logits tiles walk the
- * chunk: -1 = chosen by size (default), 0 = along the vocabulary, 1 = along the tokens.
- * LCE_OPT_DW_TRANSPOSED_READS (default 1, bf16 only): the d_weight GEMM reads the token-major d_logits with
- * transposing LDS reads; 0 builds a second, vocab-major copy of the d_logits for it (changes the workspace size:
- * set it before querying lce_backward_workspace_bytes).
- * LCE_OPT_DLOGITS_FEW_TOKEN_TILES (default 1, 16-bit inputs): with at most 128 tokens the d_logits tiles of the backward
- * use the narrow token tiles and deep LDS ring of the few-token forward; 0 = the backward's own 256 x 256 tiles.
- * LCE_OPT_LABEL_TERM_OUTSIDE (default 2, 16-bit inputs only): 1 = the one-hot part g_logprob / temperature * 1[v == label]
- * of the gradient of the logits is added to d_hidden and to the label rows of d_weight in fp32 instead of being rounded
- * to 16 bits with the rest of the d_logits tile; 2 = the label's whole entry of d_logits (one-hot and softmax part,
- * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32; 0 keeps everything inside
- * the tile, which is the reference's data format (verl/utils/kernel/kernels.py:1666-1724).  Changes the workspace size
- * like the option above.
- * LCE_OPT_DLOGITS_STRIP (default 1, 16-bit inputs on the 16x16x32 loop): vocabulary tiles that one workgroup of the
- * d_logits pass walks before it ends (1..64).
- * LCE_OPT_DHIDDEN_KSPLIT (default 0 = by shape): K slices of the d_hidden GEMM, each with its own fp32 partial that
- * is summed in a fixed order afterwards (0..16; changes the workspace size).
+/* One product-level option (process-wide; every entry point works from one snapshot of the settings taken when it starts).
  * LCE_OPT_WORKSPACE_BUDGET (default 0 = the built-in rule, chunks of 8192 vocabulary columns or wider while one
  * d_logits buffer stays within 256 MiB): a byte count; lce_backward_workspace_bytes with vocab_chunk <= 0 then
  * returns the workspace of the widest chunk that fits it (never below 2048 columns, never above the bound
  * 0.25 * T * V * esz + 4 * V * H), and lce_backward with vocab_chunk <= 0 uses that chunk.  An explicit vocab_chunk
  * is not touched.  Takes the role of the reference's fixed vocab_per_split = 9504 (verl/utils/kernel/kernels.py:1666-1670).
- * LCE_OPT_FEW_TOKEN_GEMMS (default 1, 16-bit inputs): with at most 128 tokens both gradient GEMMs of the backward run
- * as one launch of streaming kernels (d_weight written once in 64-byte runs, d_hidden from fp32 K-slice partials with
- * the weight read in place); 0 = the 256 x 256 tile kernels.  Changes the workspace size.
- * LCE_OPT_DHIDDEN_IN_PLACE (default 1, 16-bit inputs on the 16x16x32 loop): the d_hidden GEMM reads the weight as it
- * lies in memory (K-major operand through transposing LDS reads); 0 = a transposed copy of every vocabulary chunk is
- * built first (one more launch and H x chunk elements of workspace per chunk; same speed at T=16384).  Changes the
- * workspace size. */
+ * LCE_OPT_LABEL_TERM_OUTSIDE (default 2, 16-bit inputs only) chooses the data format of the gradient of the logits:
+ * 0 = the label's entry is rounded to 16 bits with the rest of the d_logits tile, which is the reference's format
+ * (verl/utils/kernel/kernels.py:1666-1724); 1 = its one-hot part g_logprob / temperature * 1[v == label] is added to
+ * d_hidden and to the label rows of d_weight in fp32 instead; 2 = the label's whole entry (one-hot and softmax part,
+ * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32.  Changes the workspace size:
+ * set it before querying lce_backward_workspace_bytes. */
 enum {
-  LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
-  LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
-  LCE_OPT_DW_TRANSPOSED_READS = 3,
   LCE_OPT_LABEL_TERM_OUTSIDE = 4,
-  LCE_OPT_DLOGITS_FEW_TOKEN_TILES = 5,
-  LCE_OPT_DLOGITS_STRIP = 6,
-  LCE_OPT_DHIDDEN_KSPLIT = 7,
-  LCE_OPT_WORKSPACE_BUDGET = 8,
-  LCE_OPT_FEW_TOKEN_GEMMS = 9,
-  LCE_OPT_DHIDDEN_IN_PLACE = 10
+  LCE_OPT_WORKSPACE_BUDGET = 8
 };
 int lce_set_option(int key, int64_t value);
 
-/* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every kernel
- * launch of the library is bracketed by HIP events on the caller's stream; lce_profile_read waits
- * for them and returns, per kernel class c < lce_profile_num_classes(), the summed duration in
- * milliseconds and the number of launches (arrays sized by the caller).  Creating events allocates
- * host-side driver objects, so keep it disabled under graph capture. */
+/* ---------------------------------------------------------------------------------------------------------------------
+ * DIAGNOSTIC BLOCK (block version 2).  Nothing below is needed to use the path; none of it has a counterpart in the
+ * reference.  It exists so that the benchmark and the tests can time the pieces of a call separately and run the
+ * mainloops on their own.  A caller that integrates the library binds the entry points above and ignores these.
+ * ------------------------------------------------------------------------------------------------------------------- */
+
+/* C[M, N] (fp32, row stride ldc) = A[M, K] . B[N, K]^T with one of the library's MFMA mainloops (the same code that the
+ * entry points above run).  K a multiple of 64 (16-bit) / 32 (fp32).  variant: see lce_set_variant. */
+int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N,
+                int64_t K, int dtype, int variant, void* stream);
+/* Twin for K-major operands (bf16 only): C[M, N] = A[K, M]^T . B[K, N], the layout of the d_weight GEMM
+ * (A = d_logits [tokens, vocab], B = hidden [tokens, H]).  K a multiple of 64; lda >= M and ldb >= N rounded up to 256.
+ * variant 3 runs the four-wave 16x16x32 loop, any other the eight-wave split ring. */
+int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                int variant, void* stream);
+
+/* Forces one mainloop for forward and backward instead of the choice by size, 0 <= variant < lce_num_variants();
+ * -1 restores the defaults.  0, 1: eight waves of 64 x 128 on v_mfma_f32_32x32x16, LDS ring of five half slabs with the
+ * A resp. B operand fetched early; 2: the same tile with a ring of two whole slabs; 3: four waves of 128 x 128 on
+ * v_mfma_f32_16x16x32 (16-bit inputs; fp32 inputs run variant 1's loop on v_mfma_f32_32x32x2).  The backward is built on
+ * variants 1 and 3: forcing 0 or 2 leaves it on 1. */
+int lce_set_variant(int variant);
+int lce_num_variants(void);
+/* Diagnostic keys of lce_set_option.  LCE_OPT_SPLIT_BACKWARD_LAUNCHES: launch the d_logits tiles and the two gradient
+ * GEMMs of a backward chunk as three kernels instead of one (per-phase timing).  LCE_OPT_DLOGITS_TOKENS_FIRST: order in
+ * which an XCD's consecutive blocks of d_logits tiles walk the chunk: -1 = chosen by size (default), 0 = along the
+ * vocabulary, 1 = along the tokens.  LCE_OPT_DHIDDEN_KSPLIT (default 0 = by shape): K slices of the d_hidden GEMM, each
+ * with its own fp32 partial that is summed in a fixed order afterwards (0..16; changes the workspace size).
+ * LCE_OPT_FEW_TOKEN_GEMMS (default 1, 16-bit inputs): with at most 128 tokens both gradient GEMMs of the backward run
+ * as one launch of streaming kernels; 0 = the 256 x 256 tile kernels, which the tests compare them with (changes the
+ * workspace size). */
+enum {
+  LCE_OPT_SPLIT_BACKWARD_LAUNCHES = 1,
+  LCE_OPT_DLOGITS_TOKENS_FIRST = 2,
+  LCE_OPT_DHIDDEN_KSPLIT = 7,
+  LCE_OPT_FEW_TOKEN_GEMMS = 9
+};
+
+/* Per-kernel timing for benchmarks.  While enabled, every kernel launch of the library is bracketed by HIP events on the
+ * caller's stream; lce_profile_read waits for them and returns, per kernel class c < lce_profile_num_classes(), the
+ * summed duration in milliseconds and the number of launches (arrays sized by the caller).  Creating events allocates
+ * host-side driver objects (also inside lce_forward_static), so keep it disabled under graph capture. */
 int lce_profile_enable(int on);
 int lce_profile_num_classes(void);
 const char* lce_profile_class_name(int cls);

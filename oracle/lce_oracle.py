@@ -13,6 +13,9 @@ What each function follows in the reference tree (paths relative to the referenc
 * ``lce_backward``           verl/utils/kernel/kernels.py:1443-1507 (closed-form ``d_logits``),
                              :1714-1724 (``d_hidden = dz @ W``, ``d_weight = dz.T @ h``),
                              verl/utils/experimental/torch_functional.py:61-93 (same math)
+* ``lce_unfused_autograd``   tests/utils/test_linear_cross_entropy.py:49-62 with ``torch.autograd.grad`` (:254-262): the
+                             same values once more through autograd on materialised logits (pinned by equality
+                             with ``lce_forward`` / ``lce_backward``)
 * ``logprobs_from_logits``   verl/utils/torch_functional.py:155-207
 * ``entropy_from_logits``    verl/utils/torch_functional.py:231-245
 * ``sum_pi_squared_from_logits`` verl/utils/torch_functional.py:687-703
@@ -144,6 +147,24 @@ def lce_backward(
         d_hidden[s:e] = dz @ w
         d_weight += dz.t() @ hc
     return d_hidden.reshape(hidden.shape), d_weight
+
+
+def lce_unfused_autograd(hidden, weight, labels, temperature, g_logprobs, g_entropy, compute_dtype=torch.float32):
+    """The unfused path exactly as the reference's test states it (tests/utils/test_linear_cross_entropy.py:49-62,
+    ``run_torch_entropy``): one materialised ``[T, V]`` logits tensor in ``compute_dtype``, ``softmax``,
+    ``logsumexp``, ``cross_entropy``, gradients by ``torch.autograd.grad``.  Returns
+    ``(logprobs, entropy, d_hidden, d_weight)``; checked against ``lce_forward`` / ``lce_backward`` (the chunked closed
+    form) in tests/test_oracle_lce.py.  The benchmark times it on the GPU as the context figure the reference's test
+    prints next to its fused kernel (:290-349); it is never the product path."""
+    h = hidden.detach().reshape(-1, hidden.shape[-1]).requires_grad_(True)
+    w = weight.detach().requires_grad_(True)
+    logits = torch.matmul(h.to(compute_dtype), w.to(compute_dtype).transpose(0, 1))
+    logits = logits / temperature
+    pd = torch.nn.functional.softmax(logits, dim=-1)
+    entropy = torch.logsumexp(logits, dim=-1) - torch.sum(pd * logits, dim=-1)
+    logprobs = torch.neg(torch.nn.functional.cross_entropy(logits, labels.reshape(-1), reduction="none"))
+    d_hidden, d_weight = torch.autograd.grad((entropy, logprobs), (h, w), (g_entropy.to(compute_dtype), g_logprobs.to(compute_dtype)))
+    return logprobs.detach(), entropy.detach(), d_hidden.reshape(hidden.shape), d_weight
 
 
 def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, compute_dtype=torch.float32):

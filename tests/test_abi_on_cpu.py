@@ -245,6 +245,37 @@ def test_metric_aggregation_kinds_of_ppo_loss():
         C.get_policy_loss_fn("gpg")
 
 
+def test_metric_values_are_plain_numbers_for_every_consumer():
+    """verl/utils/metric/utils.py:103-113 turns an appended tensor into a float at once; here the read-back is deferred
+    until somebody looks, and from then on `values`, a pickle, `repr`, `init_list` and `reduce_metrics` (:25-58, :162-163)
+    see what the reference's consumers see: floats, never tensors."""
+    import pickle
+
+    from verl_amd.utils.metric import AggregationType, Metric, reduce_metrics
+
+    m = Metric("mean", torch.tensor(1.5))
+    m.append(torch.tensor([2.5]))
+    m.append(4)
+    assert any(isinstance(v, torch.Tensor) for v in m._items)  # nothing has been read back yet
+    twin = pickle.loads(pickle.dumps(m))
+    assert twin.values == [1.5, 2.5, 4] and all(not isinstance(v, torch.Tensor) for v in twin.values)
+    assert twin.aggregation == AggregationType.MEAN and twin.aggregate() == pytest.approx(8.0 / 3)
+    assert m.values == [1.5, 2.5, 4] and all(isinstance(v, (int, float)) for v in m.values)
+    assert not any(isinstance(v, torch.Tensor) for v in m._items)  # read back once, kept as floats
+    assert "tensor" not in repr(m)
+    e = m.init_list()
+    assert e.values == [] and e.aggregation == AggregationType.MEAN
+    # extending from a metric with pending scalars keeps them pending, and folds the same
+    a = Metric("sum", torch.tensor(2.0))
+    b = Metric("sum", [1.0])
+    b.extend(a)
+    assert b.aggregate() == 3.0
+    out = reduce_metrics({"actor/pg_loss": Metric("sum", [1.0, 2.0]), "x_max": [1.0, 5.0], "x_min": [1.0, 5.0], "y": [1.0, 5.0]})
+    assert out == {"actor/pg_loss": 3.0, "x_max": 5.0, "x_min": 1.0, "y": 3.0}
+    m.values = [7.0, torch.tensor(9.0)]
+    assert m.values == [7.0, 9.0]
+
+
 def test_tile_map_covers_every_tile_once_and_balances_the_xcds(tmp_path):
     """The workgroup -> tile map of all tiled kernels, checked exhaustively on the host (tests/tile_map_check.cpp):
     a hole or a duplicate would be a wrong result on the GPU, an uneven split over the 8 XCDs a slow one (a forward with

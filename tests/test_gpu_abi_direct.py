@@ -130,3 +130,64 @@ def test_error_codes_leave_the_device_untouched():
     assert lib.lce_forward(*args()) == 0
     torch.cuda.synchronize()
     assert not (out == 7.0).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_sum_pi_squared_backward_with_and_without_the_saved_row_statistics(dtype):
+    """lce_logits_sum_pi_squared_backward takes the rows' logsumexp and sum p^2 from the forward, or recomputes both when
+    they are NULL; both ways must give autograd's gradient of the reference expression
+    (verl/utils/torch_functional.py:687-703) on a padded row stride."""
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    R, V, ld = 9, 5003, 5016
+    g = torch.Generator().manual_seed(3)
+    buf = (torch.randn(R, ld, generator=g) * 2).to(dtype).to(DEV)
+    z = buf[:, :V]
+    up = torch.randn(R, generator=g).to(DEV)
+    code = _abi.dtype_code(dtype)
+    st = torch.cuda.current_stream().cuda_stream
+    s = torch.empty(R, device=DEV)
+    lse = torch.empty(R, device=DEV)
+    _abi.check(lib.lce_logits_sum_pi_squared(buf.data_ptr(), ld, R, V, code, s.data_ptr(), lse.data_ptr(), st), "forward")
+    torch.testing.assert_close(lse.double(), torch.logsumexp(z.double(), -1), atol=1e-5, rtol=1e-6)
+    zz = z.double().requires_grad_(True)
+    (want,) = torch.autograd.grad(O.sum_pi_squared_from_logits(zz, torch.float64), zz, up.double())
+    for with_stats in (True, False):
+        d = torch.full((R, ld), 7.0, device=DEV, dtype=dtype)
+        rc = lib.lce_logits_sum_pi_squared_backward(buf.data_ptr(), ld, R, V, code, lse.data_ptr() if with_stats else None,
+                                                    s.data_ptr() if with_stats else None, up.data_ptr(), d.data_ptr(), ld, st)
+        _abi.check(rc, "backward")
+        got = d[:, :V].double()
+        if dtype == torch.float32:
+            assert ((got - want).abs().max() / want.abs().max()).item() < 1e-5
+        else:
+            assert ((got - want).abs() <= 2e-2 + want.abs() * 2.0**-7).all()
+        assert (d[:, V:] == 7.0).all()  # the padding of the rows is not written
+    assert lib.lce_logits_sum_pi_squared_backward(buf.data_ptr(), ld, R, V, code, None, None, None, d.data_ptr(), ld, st) != 0
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+def test_diagnostic_gemms_match_torch(variant):
+    """lce_gemm_nt / lce_gemm_tn (the mainloops on their own, which the benchmark's yardstick workload times) against
+    torch.matmul in fp32 on bf16 operands, ragged M and N."""
+    from verl_amd import _abi
+
+    lib = _abi.load()
+    M, N, K = 300, 520, 192
+    g = torch.Generator().manual_seed(variant)
+    A = (torch.randn(M, K, generator=g)).bfloat16().to(DEV)
+    B = (torch.randn(N, K, generator=g)).bfloat16().to(DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    C = torch.zeros(M, N, device=DEV)
+    _abi.check(lib.lce_gemm_nt(A.data_ptr(), K, B.data_ptr(), K, C.data_ptr(), N, M, N, K, 0, variant, st), "lce_gemm_nt")
+    want = A.float() @ B.float().t()
+    torch.testing.assert_close(C, want, atol=1e-3, rtol=1e-4)
+    # K-major operands, rows allocated in whole 256-column tiles
+    At = torch.zeros(K, 512, device=DEV, dtype=torch.bfloat16)
+    Bt = torch.zeros(K, 768, device=DEV, dtype=torch.bfloat16)
+    At[:, :M] = A.t()
+    Bt[:, :N] = B.t()
+    C2 = torch.zeros(M, N, device=DEV)
+    _abi.check(lib.lce_gemm_tn(At.data_ptr(), 512, Bt.data_ptr(), 768, C2.data_ptr(), N, M, N, K, variant, st), "lce_gemm_tn")
+    torch.testing.assert_close(C2, want, atol=1e-3, rtol=1e-4)

@@ -133,10 +133,39 @@ def test_sum_pi_squared_closed_forms_strides_and_errors():
         view = buf[:, off:off + 1000]
         torch.testing.assert_close(F.calculate_sum_pi_squared_from_logits(view).float(),
                                    O.sum_pi_squared_from_logits(view), atol=2e-2, rtol=2e-2)
-    with pytest.raises(NotImplementedError):
-        F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))
     with torch.no_grad():
         F.calculate_sum_pi_squared_from_logits(z.clone().requires_grad_(True))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(5, 40), (3, 7, 1031), (16, 152064), (1, 1)])
+def test_sum_pi_squared_backward_matches_autograd_of_the_reference_formula(dtype, shape):
+    """The reference's expression is plain torch (verl/utils/torch_functional.py:687-703), so it is differentiable; the
+    kernel's gradient g * 2 p (p - sum p^2) must equal autograd through exp(logsumexp(2 z) - 2 logsumexp(z)) in fp64."""
+    from verl_amd.utils import torch_functional as F
+
+    g = torch.Generator().manual_seed(shape[-1] + 7)
+    z = (torch.randn(*shape, generator=g) * 2).to(dtype).to(DEV)
+    up = torch.randn(*shape[:-1], generator=g).to(dtype).to(DEV)
+    z1 = z.clone().requires_grad_(True)
+    out = F.calculate_sum_pi_squared_from_logits(z1)
+    (got,) = torch.autograd.grad(out, z1, up)
+    assert got.shape == z.shape and got.dtype == dtype
+    z2 = z.double().requires_grad_(True)
+    (want,) = torch.autograd.grad(O.sum_pi_squared_from_logits(z2, torch.float64), z2, up.double())
+    # fp32: 1e-5 relative to the largest entry of the row's gradient; bf16: 2e-2 absolute plus one ulp of the value
+    if dtype == torch.float32:
+        scale = want.abs().amax(-1, keepdim=True).clamp_min(1e-30)
+        assert ((got.double() - want).abs() / scale).max().item() < 1e-5
+    else:
+        assert ((got.double() - want).abs() <= 2e-2 + want.abs() * 2.0**-7).all()
+    # rows whose alignment differs from the output's take the kernel's element-wise path
+    if len(shape) == 2 and shape[-1] > 8:
+        buf = torch.zeros(shape[0], shape[1] + 3, device=DEV, dtype=dtype)
+        buf[:, 1:1 + shape[1]] = z
+        v = buf[:, 1:1 + shape[1]].detach().requires_grad_(True)
+        (got2,) = torch.autograd.grad(F.calculate_sum_pi_squared_from_logits(v), v, up)
+        torch.testing.assert_close(got2.double(), got.double(), atol=1e-6 if dtype == torch.float32 else 2e-2, rtol=1e-5 if dtype == torch.float32 else 2e-2)
 
 
 @pytest.mark.parametrize("shape", [(8, 17), (3, 5, 32), (1, 1024)])

@@ -383,6 +383,52 @@ def test_ppo_loss_entry_with_the_reference_signature(nested, globals_set):
     assert metrics["kl_coef"] == 0.01
 
 
+@pytest.mark.parametrize("fields", ["jagged", "padded-wider", "padded-narrower"])
+def test_ppo_loss_honours_max_response_len(fields):
+    """verl/workers/utils/padding.py:112-118: on a nested batch the padded width of the response slice is the non-tensor
+    entry max_response_len when it is given, else the longest response.  Every field of the batch is brought to exactly
+    that width, whatever width it arrives in (jagged, padded wider, padded to the longest row only); a width shorter
+    than the longest response is an error."""
+    from verl_amd.workers.utils.losses import ppo_loss
+
+    prompt, resp = [3, 1, 7, 2, 5], [5, 1, 12, 9, 2]
+    R = 15  # max_response_len, larger than the longest response (12)
+    lp, ent, old, adv, ref, mask = _packed_case(prompt, resp, R, seed=21)
+    cols = torch.arange(R, device=DEV)[None, :] < torch.tensor(resp, device=DEV)[:, None]
+
+    def field(t):
+        if fields == "jagged":
+            return _jagged(t[cols], resp)
+        if fields == "padded-wider":
+            return torch.nn.functional.pad(t, (0, 4), value=7.0)  # garbage beyond the width must never be read
+        return t[:, :12].contiguous()
+
+    data = {"prompts": _jagged(torch.arange(sum(prompt), device=DEV), prompt), "responses": _jagged(torch.arange(sum(resp), device=DEV), resp),
+            "response_mask": field(mask), "old_log_probs": field(old), "advantages": field(adv), "ref_log_prob": field(ref),
+            "max_response_len": R, "dp_size": 1, "batch_num_tokens": None, "global_batch_size": None}
+    cfg = _ActorConfig(use_kl_loss=True, loss_agg_mode="seq-mean-token-sum-norm", loss_scale_factor=None)
+    lp1, ent1 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    lens = [p + r for p, r in zip(prompt, resp)]
+    loss, metrics = ppo_loss(cfg, {"log_probs": _jagged(lp1, lens), "entropy": _jagged(ent1, lens)}, data)
+    loss.backward()
+    lp2, ent2 = lp.clone().requires_grad_(True), ent.clone().requires_grad_(True)
+    pad = lambda t: t * cols  # noqa: E731  (what the reference's to_padded_tensor leaves beyond a row's end: zeros)
+    rloss, rmet = O.ppo_actor_loss(O.no_padding_2_padding(lp2, prompt, resp, R), O.no_padding_2_padding(ent2, prompt, resp, R), pad(old),
+                                   pad(adv), pad(mask), clip_ratio=0.2, entropy_coeff=1e-3, loss_agg_mode="seq-mean-token-sum-norm",
+                                   ref_log_prob=pad(ref), kl_loss_type="low_var_kl", kl_loss_coef=0.01, dp_size=1, batch_num_tokens=None,
+                                   global_batch_size=None, loss_scale_factor=None)
+    rloss.backward()
+    # (seq-mean-token-sum-norm divides by the padded width: the result depends on max_response_len, which is the point)
+    torch.testing.assert_close(loss, rloss, atol=1e-6, rtol=1e-5)
+    torch.testing.assert_close(lp1.grad, lp2.grad, atol=1e-8, rtol=1e-5)
+    torch.testing.assert_close(ent1.grad, ent2.grad, atol=1e-9, rtol=1e-5)
+    for k in ("actor/pg_loss", "actor/entropy_loss", "kl_loss", "actor/ppo_kl"):
+        assert metrics[k].aggregate() == pytest.approx(rmet[k], rel=1e-5, abs=1e-6), k
+    data["max_response_len"] = 11
+    with pytest.raises(ValueError, match="shorter than the longest response"):
+        ppo_loss(cfg, {"log_probs": _jagged(lp1, lens), "entropy": _jagged(ent1, lens)}, data)
+
+
 def test_ppo_loss_entry_refuses_what_has_no_fused_kernel():
     from verl_amd.workers.utils.losses import ppo_loss
 

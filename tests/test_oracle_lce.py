@@ -152,6 +152,23 @@ def test_backward_matches_autograd(reduction, with_entropy):
     torch.testing.assert_close(dw, w.grad, rtol=1e-10, atol=1e-12)
 
 
+def test_unfused_autograd_restatement_equals_the_closed_form():
+    """`lce_unfused_autograd` (the reference test's torch path through autograd, which the benchmark times on the GPU as
+    context) gives the same four results as the chunked closed form."""
+    h, w, y = _rand(7, 6, 19, seed=23)
+    tau = 1.3
+    g = torch.Generator().manual_seed(5)
+    g_lp = torch.randn(7, generator=g, dtype=torch.float64)
+    g_ent = torch.randn(7, generator=g, dtype=torch.float64)
+    lp, ent, dh, dw = O.lce_unfused_autograd(h, w, y, tau, g_lp, g_ent, torch.float64)
+    rlp, rent = O.lce_forward(h, w, y, tau, compute_dtype=torch.float64)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, tau, compute_dtype=torch.float64)
+    torch.testing.assert_close(lp, rlp, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(ent, rent, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(dh, rdh, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(dw, rdw, rtol=1e-10, atol=1e-12)
+
+
 def test_backward_finite_differences():
     h, w, y = _rand(3, 4, 9, seed=13)
     tau, eps = 1.5, 1e-6

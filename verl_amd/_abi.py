@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LCE_LIBRARY_PATH") or os.path.join(_HERE, "lib", "liblce_gfx950.so")
 
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 # every symbol include/lce_abi.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -38,12 +38,13 @@ SYMBOLS = {
     ),
     "lce_logits_forward": (_i, [_p, _i64, _p, _i64, _i64, _i, _p, _p, _p, _p]),
     "lce_logits_backward": (_i, [_p, _i64, _p, _i64, _i64, _i, _p, _p, _p, _p, _i64, _p]),
-    "lce_logits_sum_pi_squared": (_i, [_p, _i64, _i64, _i64, _i, _p, _p]),
+    "lce_logits_sum_pi_squared": (_i, [_p, _i64, _i64, _i64, _i, _p, _p, _p]),
+    "lce_logits_sum_pi_squared_backward": (_i, [_p, _i64, _i64, _i64, _i, _p, _p, _p, _p, _i64, _p]),
     "lce_ppo_loss_workspace_bytes": (_sz, [_i64, _i64]),
     "lce_ppo_loss": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _f, _i64, _i64, _i, _f, _f, _f, _f, _f, _f, _f, _f, _p, _p, _p, _p, _sz, _p]),
     "lce_ppo_loss_packed": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i, _f, _i64, _i64, _i, _f, _f, _f, _f, _f, _f, _f, _f, _p, _p, _p, _p, _sz, _p]),
     "lce_gemm_nt": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _i, _p]),
-    "lce_gemm_tn": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _p]),
+    "lce_gemm_tn": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _p]),
     "lce_set_variant": (_i, [_i]),
     "lce_num_variants": (_i, []),
     "lce_set_option": (_i, [_i, _i64]),

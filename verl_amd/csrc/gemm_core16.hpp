@@ -114,20 +114,6 @@ struct GemmCore16 {
     b_rd = (uint32_t)(wave_n * Cfg::WN * 128) + off;
   }
 
-  // the same tile position along B, another 256 rows of A (row-major operands)
-  LCE_DEV void init_a(const TIN* A, int64_t lda, int64_t m0, int64_t M) {
-    a_base = reinterpret_cast<const char*>(A + m0 * lda);
-    const int rows_a = (int)((M - m0) < (int64_t)Cfg::BM ? (M - m0) : (int64_t)Cfg::BM);
-    const int lr = lane >> 3, pc = lane & 7;
-#pragma unroll
-    for (int j = 0; j < HL; ++j) {
-      const int row = (j * Cfg::NW + wave) * 8 + lr;
-      const int c = pc ^ ((row >> 1) & 7);
-      const int ra = row < rows_a ? row : rows_a - 1;
-      va[j] = (uint32_t)((int64_t)ra * lda * 2) + (uint32_t)(c * 16);
-    }
-  }
-
   // K-major operands: A[k][m0 + 0..256), B[k][n0 + 0..256) with row strides lda / ldb (elements); both must be
   // allocated in whole 256-column tiles.  A ring slot holds 64 k-rows of 512 bytes; chunk c of row r sits at
   // position c ^ swz(r), swz(r) = 4 (r % 4) ^ 2 ((r / 8) % 2), so that the eight k-rows that half a wave touches

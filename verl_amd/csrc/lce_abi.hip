@@ -62,21 +62,31 @@ static __device__ __align__(256) unsigned char scratch[LCE_STATIC_SCRATCH_BYTES]
 namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
-void* g_scratch_ptr[kMaxDevices] = {nullptr};
-// device address of `scratch` on the current device
-int static_scratch(void** out) {
+// per device: the address of `scratch`, and who used it last (the stream, and an event recorded behind that call's last
+// kernel) so that a call on ANOTHER stream while that one is still running is refused instead of racing for the buffer
+struct StaticUse {
+  void* ptr = nullptr;
+  hipEvent_t done = nullptr;
+  hipStream_t last_stream = nullptr;
+  bool recorded = false;
+};
+StaticUse g_static[kMaxDevices];
+// set-up of the current device's entry (once per device; the caller holds g_scratch_mu)
+int static_scratch(StaticUse** out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(LCE_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
   if (dev < 0 || dev >= kMaxDevices) return fail(LCE_E_ARG, "device index %d out of range", dev);
-  std::lock_guard<std::mutex> l(g_scratch_mu);
-  if (!g_scratch_ptr[dev]) {
+  StaticUse& u = g_static[dev];
+  if (!u.ptr) {
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr) return fail(LCE_E_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
-    g_scratch_ptr[dev] = ptr;
+    e = hipEventCreateWithFlags(&u.done, hipEventDisableTiming);
+    if (e != hipSuccess) return fail(LCE_E_LAUNCH, "hipEventCreateWithFlags: %s", hipGetErrorString(e));
+    u.ptr = ptr;
   }
-  *out = g_scratch_ptr[dev];
+  *out = &u;
   return LCE_OK;
 }
 }  // namespace
@@ -100,23 +110,16 @@ int lce_set_option(int key, int64_t value) {
   Tuning& t = g_tuning;
   switch (key) {
     case LCE_OPT_SPLIT_BACKWARD_LAUNCHES: t.split_bwd = value != 0; return LCE_OK;
-    case LCE_OPT_DW_TRANSPOSED_READS: t.dw_transposed_reads = value != 0; return LCE_OK;
     case LCE_OPT_LABEL_TERM_OUTSIDE:
       if (value < 0 || value > 2) return fail(LCE_E_ARG, "LCE_OPT_LABEL_TERM_OUTSIDE takes 0, 1 or 2");
       t.label_outside = (int)value;
       return LCE_OK;
-    case LCE_OPT_DLOGITS_FEW_TOKEN_TILES: t.ds_few_tokens = value != 0; return LCE_OK;
     case LCE_OPT_DLOGITS_TOKENS_FIRST: t.ds_tokens_first = value < 0 ? -1 : (value != 0); return LCE_OK;
     case LCE_OPT_DHIDDEN_KSPLIT:
       if (value < 0 || value > 16) return fail(LCE_E_ARG, "LCE_OPT_DHIDDEN_KSPLIT takes 0..16");
       t.dh_ksplit = (int)value;
       return LCE_OK;
-    case LCE_OPT_DLOGITS_STRIP:
-      if (value < 1 || value > 64) return fail(LCE_E_ARG, "LCE_OPT_DLOGITS_STRIP takes 1..64");
-      t.ds_strip = (int)value;
-      return LCE_OK;
     case LCE_OPT_FEW_TOKEN_GEMMS: t.few_token_gemms = value != 0; return LCE_OK;
-    case LCE_OPT_DHIDDEN_IN_PLACE: t.dh_in_place16 = value != 0; return LCE_OK;
     case LCE_OPT_WORKSPACE_BUDGET:
       if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_WORKSPACE_BUDGET takes a byte count (0 = the built-in default)");
       t.ws_budget = value;
@@ -190,11 +193,11 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
   if (!tu.variant_forced) {
     if (T <= 64) sel = kSelT64;
     else if (T <= 128) sel = kSelT128;
-    else if (T <= 512) sel = 1;  // W (the A operand) streams from HBM: give it the early slot
+    else if (T <= 512) sel = 0;  // W (the A operand) streams from HBM: give it the early slot
     else if (esize(dtype) == 2 && T > kCore16MinTokensFwd) sel = kVariantCore16;
     // the split ring: measured 4-7% faster than the 2-stage ring up to 8192 tokens, equal (+-1%) beyond, and
     // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
-    else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 2;
+    else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 1;
   }
   return kForward[dtype](sel, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum,
                          accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits);
@@ -223,13 +226,28 @@ int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int6
                   (long long)T, fixed + (size_t)T * 64, (size_t)LCE_STATIC_SCRATCH_BYTES);
     if (room < (size_t)kMaxSplits) max_splits = (int)room;
   }
-  void* ws = nullptr;
-  const int rc = static_scratch(&ws);
+  // One call at a time per device on the host side: the check below, the launches and the record behind them are one step.
+  std::lock_guard<std::mutex> l(g_scratch_mu);
+  StaticUse* use = nullptr;
+  int rc = static_scratch(&use);
   if (rc) return rc;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  // (a capturing stream records nothing here and is not checked: inside a graph the order of the nodes is the caller's)
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  const bool capturing = hipStreamIsCapturing(st, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+  if (!capturing && use->recorded && use->last_stream != st && hipEventQuery(use->done) == hipErrorNotReady)
+    return fail(LCE_E_BUSY, "lce_forward_static: the previous call on this GPU, on another stream, is still running and owns the "
+                            "built-in scratch buffer; order the two streams, or use lce_forward with a workspace of your own");
   // (what must start at zero, the label logits, is cleared by a fill kernel inside the forward: nothing of the previous
   // call's contents is read)
-  return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
-                       accumulate, entropy_b, ws, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr, max_splits);
+  rc = forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
+                     accumulate, entropy_b, use->ptr, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr, max_splits);
+  if (rc == LCE_OK && !capturing && T > 0) {
+    if (hipEventRecord(use->done, st) != hipSuccess) return fail(LCE_E_LAUNCH, "lce_forward_static: hipEventRecord failed");
+    use->last_stream = st;
+    use->recorded = true;
+  }
+  return rc;
 }
 
 int lce_forward_shard(const void* hidden, int64_t ldh, const void* weight_shard, int64_t ldw, const int64_t* labels, int64_t T,
@@ -343,11 +361,11 @@ int lce_gemm_nt(const void* A, int64_t lda, const void* B, int64_t ldb, float* C
 }
 
 int lce_gemm_tn(const void* A, int64_t lda, const void* B, int64_t ldb, float* C, int64_t ldc, int64_t M, int64_t N, int64_t K,
-                void* stream) {
+                int variant, void* stream) {
   if (!A || !B || !C || !aligned16(A) || !aligned16(B)) return fail(LCE_E_ARG, "bad pointer");
   if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0 || lda % 8 != 0 || ldb % 8 != 0) return fail(LCE_E_ARG, "gemm_tn: bad shape");
   if (lda < round_up(M, 256) || ldb < round_up(N, 256)) return fail(LCE_E_ARG, "gemm_tn: rows must be allocated in whole 256-column tiles");
-  const bool core16 = tuning_snapshot().variant_bwd == kVariantCore16;  // the same product on the four-wave 16x16x32 loop
+  const bool core16 = variant == kVariantCore16;  // the same product on the four-wave 16x16x32 loop
   if (core16 && N % 4 != 0) return fail(LCE_E_ARG, "gemm_tn: N must be a multiple of 4");
   return gemm_tn_bf16(core16, A, lda, B, ldb, C, ldc, M, N, K, reinterpret_cast<hipStream_t>(stream));
 }
@@ -370,7 +388,7 @@ int lce_logits_forward(const void* logits, int64_t ldl, const int64_t* labels, i
   return check_launch("logits_fwd_kernel");
 }
 
-int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, void* stream) {
+int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, float* out, float* lse_out, void* stream) {
   if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
   if (R < 0 || V <= 0 || ldl < V) return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld", (long long)R, (long long)V, (long long)ldl);
   if (R == 0) return LCE_OK;
@@ -379,12 +397,34 @@ int lce_logits_sum_pi_squared(const void* logits, int64_t ldl, int64_t R, int64_
   constexpr int NT = 512;
   ProfScope prof(PC_LOGITS_FWD, st);
   if (dtype == LCE_DTYPE_BF16)
-    hipLaunchKernelGGL((logits_pi2_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, V, out);
+    hipLaunchKernelGGL((logits_pi2_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, V, out, lse_out);
   else if (dtype == LCE_DTYPE_F16)
-    hipLaunchKernelGGL((logits_pi2_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, V, out);
+    hipLaunchKernelGGL((logits_pi2_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, V, out, lse_out);
   else
-    hipLaunchKernelGGL((logits_pi2_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, V, out);
+    hipLaunchKernelGGL((logits_pi2_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, V, out, lse_out);
   return check_launch("logits_pi2_kernel");
+}
+
+int lce_logits_sum_pi_squared_backward(const void* logits, int64_t ldl, int64_t R, int64_t V, int dtype, const float* lse, const float* sum_pi2,
+                                       const float* g, void* d_logits, int64_t ldd, void* stream) {
+  if (!known_dtype(dtype)) return fail(LCE_E_ARG, "unsupported dtype %d", dtype);
+  if (R < 0 || V <= 0 || ldl < V || ldd < V)
+    return fail(LCE_E_ARG, "bad shape R=%lld V=%lld ldl=%lld ldd=%lld", (long long)R, (long long)V, (long long)ldl, (long long)ldd);
+  if (R == 0) return LCE_OK;
+  if (!logits || !g || !d_logits) return fail(LCE_E_ARG, "null pointer");
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  constexpr int NT = 512;
+  ProfScope prof(PC_LOGITS_BWD, st);
+  if (dtype == LCE_DTYPE_BF16)
+    hipLaunchKernelGGL((logits_pi2_bwd_kernel<bf16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const bf16_t*)logits, ldl, V, lse, sum_pi2, g,
+                       (bf16_t*)d_logits, ldd);
+  else if (dtype == LCE_DTYPE_F16)
+    hipLaunchKernelGGL((logits_pi2_bwd_kernel<f16_t, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const f16_t*)logits, ldl, V, lse, sum_pi2, g,
+                       (f16_t*)d_logits, ldd);
+  else
+    hipLaunchKernelGGL((logits_pi2_bwd_kernel<float, NT>), dim3((unsigned)R), dim3(NT), 0, st, (const float*)logits, ldl, V, lse, sum_pi2, g,
+                       (float*)d_logits, ldd);
+  return check_launch("logits_pi2_bwd_kernel");
 }
 
 // geometry of the PPO loss launches: workgroups per row and elements per workgroup

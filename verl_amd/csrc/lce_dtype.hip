@@ -34,8 +34,6 @@ int TU_FN(forward)(int sel, LCE_FWD_PARAMS) {
     case 1: LCE_RUN(Variant1);
     case 2: LCE_RUN(Variant2);
     case 3: LCE_RUN(Variant3);
-    case 4: LCE_RUN(Variant4);
-    case 5: LCE_RUN(Variant5);
     case kSelT64: LCE_RUN(VariantT64);
     case kSelT128: LCE_RUN(VariantT128);
   }
@@ -51,8 +49,6 @@ int TU_FN(gemm_nt)(int sel, LCE_GEMM_PARAMS) {
     case 1: LCE_RUN(Variant1);
     case 2: LCE_RUN(Variant2);
     case 3: LCE_RUN(Variant3);
-    case 4: LCE_RUN(Variant4);
-    case 5: LCE_RUN(Variant5);
   }
 #undef LCE_RUN
   return fail(LCE_E_ARG, "variant %d out of range", sel);
@@ -64,13 +60,10 @@ int TU_FN(backward)(int sel, LCE_BWD_PARAMS) {
 #define LCE_RUN(Vt)                                                                                                           \
   return backward_impl<typename Vt<TuT>::Cfg>((const TuT*)h, ldh, (const TuT*)W, ldw, labels, T, H, V, temperature, reduction, \
                                               mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st, vocab_offset, tu)
+  // (bwd_variant() hands over one of the two mainloops the backward is built on)
   switch (sel) {
-    case 0: LCE_RUN(Variant0);
-    case 1: LCE_RUN(Variant1);
-    case 2: LCE_RUN(Variant2);
-    case 3: LCE_RUN(Variant3);
-    case 4: LCE_RUN(Variant4);
-    case 5: LCE_RUN(Variant5);
+    case kDefaultVariantBwd: LCE_RUN(Variant1);
+    case kVariantCore16: LCE_RUN(Variant3);
   }
 #undef LCE_RUN
   return fail(LCE_E_ARG, "variant %d out of range", sel);

@@ -32,9 +32,9 @@ extern std::vector<hipEvent_t> prof_pool;
 // Defaults of the 32x32x16 loops: the backward's long-K GEMMs gain 3% from the split ring; the forward gains from it
 // only up to 8192 tokens and beyond that fetches twice as much through the fabric with it at the same speed (the XCD's
 // workgroups drift apart and lose L2 sharing), so large fp32 forwards keep the 2-stage ring.  16-bit inputs run the
-// four-wave 16x16x32 loop (variant 5) above the token counts below.
-constexpr int kDefaultVariantFwd = 3, kDefaultVariantBwd = 2, kVariantCore16 = 5;
-// variant 5 is the default above these token counts (measured at H=3584, V=152064: the forward gains 2-6% from 1024
+// four-wave 16x16x32 loop (variant 3) above the token counts below.
+constexpr int kDefaultVariantFwd = 2, kDefaultVariantBwd = 1, kVariantCore16 = 3;
+// variant 3 is the default above these token counts (measured at H=3584, V=152064: the forward gains 2-6% from 1024
 // tokens on; forward + backward is 2% slower with it at 1024 tokens, 2% faster at 1536 and 2048, 4% at 3072)
 constexpr int64_t kCore16MinTokensFwd = 512, kCore16MinTokensBwd = 1280;
 struct Tuning {
@@ -42,18 +42,14 @@ struct Tuning {
   bool variant_forced = false;   // lce_set_variant was called: no size-based choice of the tile
   int split_bwd = 0;             // diagnostic: launch the three sub-problems of a backward chunk separately
   int ds_tokens_first = -1;      // tile order of the d_logits pass; -1: by size
-  int ds_few_tokens = 1;         // d_logits tiles of a backward with at most 128 tokens: narrow token tiles, deeper ring
   int label_outside = 2;         // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
   int dh_ksplit = 0;             // K slices of the d_hidden GEMM; 0: chosen by shape
-  int ds_strip = 1;              // vocabulary tiles per workgroup of the d_logits pass on the 16x16x32 loop
-  int dw_transposed_reads = 1;   // d_weight GEMM straight from the token-major d_logits (bf16); 0: from a second, vocab-major copy
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
   int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
-  int dh_in_place16 = 1;         // 16x16x32 backward: the d_hidden GEMM reads W in place (mixed mode) instead of a transposed chunk
 };
 
-// tile selectors of the per-type launchers: 0..5 are the variants of lce_set_variant, then the two few-token forward tiles
-enum { kSelT64 = 6, kSelT128 = 7 };
+// tile selectors of the per-type launchers: 0..3 are the variants of lce_set_variant, then the two few-token forward tiles
+enum { kSelT64 = 4, kSelT128 = 5 };
 
 // The launchers of one element type each (lce_dtype.hip compiles them as separate objects).  `sel` is a tile selector;
 // the other arguments are those of forward_impl / backward_impl / launch_gemm below with untyped pointers.
@@ -88,9 +84,11 @@ namespace {
 bool known_dtype(int dtype) { return dtype == LCE_DTYPE_BF16 || dtype == LCE_DTYPE_F32 || dtype == LCE_DTYPE_F16; }
 size_t esize(int dtype) { return dtype == LCE_DTYPE_F32 ? 4 : 2; }
 
-// the mainloop variant a backward over T tokens of `esz`-byte elements runs with
+// the mainloop variant a backward over T tokens of `esz`-byte elements runs with.  The backward is built on two of the
+// mainloops: the four-wave 16x16x32 loop (variant 3) and the eight-wave split ring with the B operand early (variant 1,
+// which a forced variant 0 or 2 also selects: those two differ from it only in ways that matter to the forward).
 int bwd_variant(const Tuning& tu, int64_t T, size_t esz) {
-  if (tu.variant_forced) return tu.variant_bwd;
+  if (tu.variant_forced) return tu.variant_bwd == kVariantCore16 ? kVariantCore16 : kDefaultVariantBwd;
   return (esz == 2 && T > kCore16MinTokensBwd) ? kVariantCore16 : kDefaultVariantBwd;
 }
 
@@ -131,20 +129,18 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// tile configurations of the mainloop, selectable for tuning
-//            TIN     BM   BN   BKB NSTAGE WAVES_M WAVES_N
-template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 5, 2, 2, 2> Cfg; };  // 4 waves of 128x128, split ring
-template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 1> Cfg; };  // split ring of five half stages, A early
-template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 2> Cfg; };  // split ring of five half stages, B early
-template <typename TIN> struct Variant3 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };
+// tile configurations of the mainloop, selectable for tuning (lce_set_variant)
+//            TIN     BM   BN   BKB NSTAGE WAVES_M WAVES_N SPLIT
+template <typename TIN> struct Variant0 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 1> Cfg; };  // split ring of five half stages, A early
+template <typename TIN> struct Variant1 { typedef GemmCfg<TIN, 256, 256, 128, 5, 4, 2, 2> Cfg; };  // split ring of five half stages, B early
+template <typename TIN> struct Variant2 { typedef GemmCfg<TIN, 256, 256, 128, 2, 4, 2> Cfg; };     // two whole stages
+// four waves of 128x128 on v_mfma_f32_16x16x32 (16-bit inputs; fp32 inputs run the split-ring 32x32x2 loop instead)
+template <typename TIN> struct Variant3 { typedef GemmCfg16<TIN> Cfg; };
+template <> struct Variant3<float> { typedef GemmCfg<float, 256, 256, 128, 5, 4, 2, 2> Cfg; };
 // forward with few tokens (one pass over W, HBM-bound): narrow token tiles leave LDS for a deeper ring
 template <typename TIN> struct VariantT64 { typedef GemmCfg<TIN, 256, 64, 128, 4, 4, 2> Cfg; };
 template <typename TIN> struct VariantT128 { typedef GemmCfg<TIN, 256, 128, 128, 3, 4, 2> Cfg; };
-template <typename TIN> struct Variant4 { typedef GemmCfg<TIN, 256, 128, 128, 3, 2, 2> Cfg; };
-// four waves of 128x128 on v_mfma_f32_16x16x32 (16-bit inputs; fp32 inputs run the split-ring 32x32x2 loop instead)
-template <typename TIN> struct Variant5 { typedef GemmCfg16<TIN> Cfg; };
-template <> struct Variant5<float> { typedef GemmCfg<float, 256, 256, 128, 5, 4, 2, 2> Cfg; };
-constexpr int kNumVariants = 6;
+constexpr int kNumVariants = 4;
 
 template <typename K>
 void allow_lds(K kernel, int bytes) {
@@ -328,10 +324,9 @@ struct BwdLayout {
   bool few;    // at most 128 tokens, 16-bit inputs: both gradient GEMMs run as the streaming kernels of few_tokens.hpp
 };
 
-// The d_weight GEMM can take the token-major d_logits and hidden as they are (transposing LDS reads exist
-// for 16-bit elements and are wired for the 8-wave 256 x 256 tile variants 1-3); otherwise a vocab-major copy of the
-// d_logits and a transposed hidden are built for it.
-bool dw_transposed_reads(const Tuning& tu, int variant, size_t esz) { return esz == 2 && ((tu.dw_transposed_reads && variant >= 1 && variant <= 3) || variant == kVariantCore16); }
+// The d_weight GEMM takes the token-major d_logits and hidden as they are where transposing LDS reads exist (16-bit
+// elements); for fp32 a vocab-major copy of the d_logits and a transposed hidden are built for it.
+bool dw_transposed_reads(size_t esz) { return esz == 2; }
 
 // The d_hidden GEMM has only ceil(T/256) * ceil(H/256) output tiles, each with a K loop as long as the
 // vocabulary chunk.  With few tokens one such tile takes longer than a CU's share of the whole launch
@@ -351,13 +346,13 @@ int dh_ksplit(int64_t T, int64_t H, int64_t vchunk) {
 BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt, int64_t gv) {
   BwdLayout L;
   const int variant = bwd_variant(tu, T, esz);
-  L.tn = dw_transposed_reads(tu, variant, esz);
+  L.tn = dw_transposed_reads(esz);
   // Measured: reading W through the transposing LDS reads costs the d_hidden GEMM about 2% of its rate, and
   // saves one transpose of W per call.  The transpose is the larger cost up to some thousands of tokens
   // (T=64: 1.95 -> 1.43 ms per forward + backward, T=4096: 15.7 -> 14.7 ms at H=3584, V=152064), the GEMM
   // rate beyond that (T=16384: +0.5 ms).
   // (on the 16x16x32 loop the transposing reads of one operand cost under 1 %: W is always read in place there)
-  L.tn_dh = L.tn && (variant == kVariantCore16 ? tu.dh_in_place16 != 0 : T <= 8192);
+  L.tn_dh = L.tn && (variant == kVariantCore16 || T <= 8192);
   vchunk = round_up(vchunk, 256);
   if (vchunk > round_up(V, 256)) vchunk = round_up(V, 256);
   L.vchunk = vchunk;
@@ -622,13 +617,12 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       d.rows = rows; d.n_rows = n_rows;
       d.label_outside = lt.labels != nullptr ? tu.label_outside : 0;
       d.tokc = tokc; d.tokl = tokl; d.lab0 = v0;
-      d.strip = Cfg::CORE16 ? tu.ds_strip : 1;
       d.range_rows = 0;
       if (Cfg::CORE16 && L.tn) {
         // the compact copy of hidden built for the d_weight GEMM: the tiles read it without a row gather
         d.h = Ht; d.ldh = L.ldHt; d.rows = nullptr;
       }
-      const int nvt = ((int)((vrows + Cfg::BM - 1) / Cfg::BM) + d.strip - 1) / d.strip;  // columns of the map: strips of tiles
+      const int nvt = (int)((vrows + Cfg::BM - 1) / Cfg::BM);
       // Order in which an XCD's consecutive blocks walk the chunk.  Measured: along the vocabulary is 2-3%
       // faster on the launch while `hidden` is small enough to stay in the memory-side cache next to the
       // chunk's other operands (T=16384, H=3584: 117 MB), along the tokens is 2% faster beyond that
@@ -732,7 +726,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     }
     ProfScope prof(PC_BWD_CHUNK, st);
     if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
-      if (tu.ds_few_tokens && p.n_gw + p.n_gh == 0 && L.tn && T <= 128) {  // the first launch: d_logits tiles only
+      if (p.n_gw + p.n_gh == 0 && L.tn && T <= 128) {  // the first launch: d_logits tiles only
         const int nvt = (int)((p.ds.vrows + Cfg::BM - 1) / Cfg::BM);
         rc = T <= 64 ? launch_ds_few_tokens<typename VariantT64<TIN>::Cfg, Cfg>(p.ds, T, nvt, st)
                      : launch_ds_few_tokens<typename VariantT128<TIN>::Cfg, Cfg>(p.ds, T, nvt, st);

@@ -326,7 +326,6 @@ struct DsArgs {
   const f32x4_t* tokc;
   const int* tokl;
   int64_t lab0;
-  int strip;  // vocabulary tiles that one workgroup walks (the map's columns are strips)
   int64_t range_rows;  // few tokens: > 0 = every workgroup of lce_bwd_ds_kernel takes that many vocabulary rows (a multiple of the wave tile's)
 };
 
@@ -1156,13 +1155,71 @@ __global__ __launch_bounds__(NT) void logits_fwd_kernel(const TIN* logits, int64
 }
 
 // sum over the vocabulary of softmax(row)^2 = sum exp(z - m)^2 / (sum exp(z - m))^2, one pass
+// stats (optional, [R]): the row's logsumexp, kept for the backward
 template <typename TIN, int NT>
-__global__ __launch_bounds__(NT) void logits_pi2_kernel(const TIN* logits, int64_t ldl, int64_t V, float* out) {
+__global__ __launch_bounds__(NT) void logits_pi2_kernel(const TIN* logits, int64_t ldl, int64_t V, float* out, float* stats) {
   __shared__ float sh[3 * NT / 64];
   const int64_t r = blockIdx.x;
   float m, a, q;
   row_stats<TIN, NT, true>(logits + r * ldl, V, m, a, q, sh);
-  if (threadIdx.x == 0) out[r] = q / (a * a);
+  if (threadIdx.x == 0) {
+    out[r] = q / (a * a);
+    if (stats) stats[r] = m + logf(a);
+  }
+}
+
+// gradient of S = sum_v p_v^2 with respect to the logits: dS/dz_k = 2 p_k (p_k - S); d_logits = g * that.
+// lse / S: per-row logsumexp and sum of squares from the forward (either may be null: recomputed from the row).
+template <typename TIN, int NT>
+__global__ __launch_bounds__(NT) void logits_pi2_bwd_kernel(const TIN* logits, int64_t ldl, int64_t V, const float* lse_in, const float* s_in,
+                                                            const float* g, TIN* dl, int64_t ldd) {
+  typedef RowSplit<TIN> RS;
+  typedef typename RS::vec_t vec_t;
+  constexpr int N = RS::N;
+  __shared__ float sh[3 * NT / 64];
+  const int64_t r = blockIdx.x;
+  const TIN* row = logits + r * ldl;
+  float lse, S;
+  if (lse_in && s_in) {
+    lse = lse_in[r];
+    S = s_in[r];
+  } else {
+    float m, a, q;
+    row_stats<TIN, NT, true>(row, V, m, a, q, sh);
+    lse = m + logf(a);
+    S = q / (a * a);
+  }
+  const float lse2 = lse * kLog2e, g2 = 2.f * g[r];
+  TIN* out = dl + r * ldd;
+  auto value = [&](float z) {
+    const float pr = fast_exp2(__builtin_fmaf(z, kLog2e, -lse2));
+    return g2 * pr * (pr - S);
+  };
+  const RS rs(row, V);
+  const bool same = ((reinterpret_cast<uint64_t>(out) ^ reinterpret_cast<uint64_t>(row)) & 15) == 0;  // vector stores line up too
+  if (!same) {
+    for (int64_t v = threadIdx.x; v < V; v += NT) out[v] = (TIN)value(load_as_float(row, v));
+    return;
+  }
+  for (int64_t v = threadIdx.x; v < rs.head; v += NT) out[v] = (TIN)value(load_as_float(row, v));
+  const vec_t* vp = reinterpret_cast<const vec_t*>(row + rs.head);
+  vec_t* op = reinterpret_cast<vec_t*>(out + rs.head);
+  auto vec = [&](int64_t i, const vec_t& v) {
+    vec_t o;
+#pragma unroll
+    for (int e = 0; e < N; ++e) o[e] = (TIN)value((float)v[e]);
+    __builtin_nontemporal_store(o, &op[i]);  // written once, never re-read by this kernel
+  };
+  int64_t i = threadIdx.x;
+  for (; i + 3 * NT < rs.nvec; i += 4 * NT) {  // four loads in flight per lane
+    const vec_t a0 = vp[i], a1 = vp[i + NT], a2 = vp[i + 2 * NT], a3 = vp[i + 3 * NT];
+    vec(i, a0);
+    vec(i + NT, a1);
+    vec(i + 2 * NT, a2);
+    vec(i + 3 * NT, a3);
+  }
+  for (; i < rs.nvec; i += NT) vec(i, vp[i]);
+  for (int64_t v = rs.tail0 + threadIdx.x; v < V; v += NT) out[v] = (TIN)value(load_as_float(row, v));
 }
 
 template <typename TIN, int NT>

@@ -227,19 +227,16 @@ LCE_DEV void ds16_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x4_t (&a
   }
 }
 
-// A workgroup walks `strip` consecutive vocabulary tiles of one token tile, the first loads of the next tile in flight
-// while the finished one is written out.  (Measured: one tile per workgroup is the fastest, 3% ahead of strips of four;
-// the hardware dispatcher refills a CU quickly, the coarser grid quantises worse, and on this chip a wave cannot wait
-// for its loads without also waiting for its older stores.)
+// One workgroup per tile.  (Workgroups that walk strips of 2, 4 or 8 consecutive vocabulary tiles, with the first loads
+// of the next tile in flight while the finished one is written out, took the same time on the pass alone and more inside
+// the backward's combined launch, whose tail then is a strip long.)
 template <typename Cfg>
 LCE_DEV void ds16_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
   constexpr int NB = Cfg::NB;
   const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;  // tokens that take part
-  int tt, vs;
+  int tt, vt;
   const TileMap map = p.n_rows ? p.map.with_rows((int)((Tc + Cfg::BN - 1) / Cfg::BN)) : p.map;
-  if (!map.decode(bid, tt, vs)) return;
-  const int nvt = (int)((p.vrows + Cfg::BM - 1) / Cfg::BM);
-  const int vt0 = vs * p.strip, vt1 = vt0 + p.strip < nvt ? vt0 + p.strip : nvt;
+  if (!map.decode(bid, tt, vt)) return;
   const int64_t n0 = (int64_t)tt * Cfg::BN;
   const int lane = threadIdx.x & 63, g4 = lane >> 4, l16 = lane & 15;
   GemmCore16<Cfg> g;
@@ -257,45 +254,37 @@ LCE_DEV void ds16_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
       lab[j] = p.tokl[pos];
     }
   }
-  g.init(p.W, p.ldw, (int64_t)vt0 * Cfg::BM, p.vrows, p.h, p.ldh, n0, Tc, p.rows);
-  g.prologue(lds, p.H);
+  g.init(p.W, p.ldw, (int64_t)vt * Cfg::BM, p.vrows, p.h, p.ldh, n0, Tc, p.rows);
   f32x4_t acc[NB][NB];
-  for (int vt = vt0; vt < vt1; ++vt) {
-    g.main(lds, p.H, acc);
-    const int vloc0 = vt * Cfg::BM + g.wave_m * Cfg::WM;  // chunk-local vocabulary index of this wave's first row
-    __syncthreads();  // every wave's slab loads have landed and its operand reads are done: the ring is free
-    if (vt + 1 < vt1) {
-      g.init_a(p.W, p.ldw, (int64_t)(vt + 1) * Cfg::BM, p.vrows);
-      g.prologue(lds, p.H);
-    }
-    // fast path: no padded vocabulary rows and no label in the wave tile
-    bool has_label = false;
-    if (p.label_outside != 1) {
+  g.run(lds, p.H, acc);
+  const int vloc0 = vt * Cfg::BM + g.wave_m * Cfg::WM;  // chunk-local vocabulary index of this wave's first row
+  // fast path: no padded vocabulary rows and no label in the wave tile
+  bool has_label = false;
+  if (p.label_outside != 1) {
 #pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const int rel = lab[j] - (int)p.lab0 - vloc0;
-        has_label |= (rel >= 0 && rel < Cfg::WM);
-      }
+    for (int j = 0; j < NB; ++j) {
+      const int rel = lab[j] - (int)p.lab0 - vloc0;
+      has_label |= (rel >= 0 && rel < Cfg::WM);
     }
-    const bool labels_here = __builtin_amdgcn_ballot_w64(has_label) != 0;
-    // Labels kept out of the tiles altogether (label_outside == 2, the default): the tile is written by the common
-    // path, and the lane that stored a label's entry then overwrites it with a zero (same lane, same address, later
-    // store).  Measured on a 38144-column chunk of config 2, where one wave tile in nine holds a label: 3.71 -> 3.58 ms
-    // against patching inside the common arithmetic.  With the one-hot part inside the tile (0) the patch adds G there.
-    const bool in_tile = labels_here && p.label_outside == 0;
-    const bool edge = vloc0 + Cfg::WM > p.vrows;
-    if (edge && in_tile) ds16_epilogue<Cfg, true, true>(p, acc, tc, lab, tok0, vloc0, g4, l16);
-    else if (edge) ds16_epilogue<Cfg, false, true>(p, acc, tc, lab, tok0, vloc0, g4, l16);
-    else if (in_tile) ds16_epilogue<Cfg, true, false>(p, acc, tc, lab, tok0, vloc0, g4, l16);
-    else ds16_epilogue<Cfg, false, false>(p, acc, tc, lab, tok0, vloc0, g4, l16);
-    if (labels_here && p.label_outside == 2) {
+  }
+  const bool labels_here = __builtin_amdgcn_ballot_w64(has_label) != 0;
+  // Labels kept out of the tiles altogether (label_outside == 2, the default): the tile is written by the common
+  // path, and the lane that stored a label's entry then overwrites it with a zero (same lane, same address, later
+  // store).  Measured on a 38144-column chunk of config 2, where one wave tile in nine holds a label: 3.71 -> 3.58 ms
+  // against patching inside the common arithmetic.  With the one-hot part inside the tile (0) the patch adds G there.
+  const bool in_tile = labels_here && p.label_outside == 0;
+  const bool edge = vloc0 + Cfg::WM > p.vrows;
+  if (edge && in_tile) ds16_epilogue<Cfg, true, true>(p, acc, tc, lab, tok0, vloc0, g4, l16);
+  else if (edge) ds16_epilogue<Cfg, false, true>(p, acc, tc, lab, tok0, vloc0, g4, l16);
+  else if (in_tile) ds16_epilogue<Cfg, true, false>(p, acc, tc, lab, tok0, vloc0, g4, l16);
+  else ds16_epilogue<Cfg, false, false>(p, acc, tc, lab, tok0, vloc0, g4, l16);
+  if (labels_here && p.label_outside == 2) {
 #pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const int rel = lab[j] - (int)p.lab0 - vloc0;  // = 16 i + 4 g + r inside the wave tile
-        const int64_t tok = tok0 + j * 16 + l16;
-        if (rel >= 0 && rel < Cfg::WM && ((rel >> 2) & 3) == g4 && tok < p.tpad)
-          p.dS[tok * p.ldS + vloc0 + (rel >> 5) * 32 + g4 * 8 + ((rel >> 4) & 1) * 4 + (rel & 3)] = (typename Cfg::TIN)0.f;
-      }
+    for (int j = 0; j < NB; ++j) {
+      const int rel = lab[j] - (int)p.lab0 - vloc0;  // = 16 i + 4 g + r inside the wave tile
+      const int64_t tok = tok0 + j * 16 + l16;
+      if (rel >= 0 && rel < Cfg::WM && ((rel >> 2) & 3) == g4 && tok < p.tpad)
+        p.dS[tok * p.ldS + vloc0 + (rel >> 5) * 32 + g4 * 8 + ((rel >> 4) & 1) * 4 + (rel & 3)] = (typename Cfg::TIN)0.f;
     }
   }
 }

@@ -43,27 +43,36 @@ class LinearCrossEntropy(torch.autograd.Function):
         # the reference's two type checks (:64-65), messages included: callers' tests match on them
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
-        mode = kernels.get_entropy_reduction_enum_number(reduction.lower())
-        rows, flat_labels = _as_token_rows(hidden, labels)
-        logprobs, entropy, *stats = kernels.efficient_entropy_forward(rows, weight, flat_labels, mode, temperature, dist_process_group)
-        ctx.save_for_backward(rows, weight, flat_labels, *stats)  # stats = (maximum, accumulate, entropy_b), fp32 [T]
-        ctx.call = (hidden.shape, mode, temperature, dist_process_group)
-        ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
+        # the reference's profiler range (:66); on ROCm torch.cuda.nvtx is roctx, so `rocprofv3 --marker-trace` shows it
+        torch.cuda.nvtx.range_push("LinearCrossEntropy-forward")
+        try:
+            mode = kernels.get_entropy_reduction_enum_number(reduction.lower())
+            rows, flat_labels = _as_token_rows(hidden, labels)
+            logprobs, entropy, *stats = kernels.efficient_entropy_forward(rows, weight, flat_labels, mode, temperature, dist_process_group)
+            ctx.save_for_backward(rows, weight, flat_labels, *stats)  # stats = (maximum, accumulate, entropy_b), fp32 [T]
+            ctx.call = (hidden.shape, mode, temperature, dist_process_group)
+            ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
+        finally:
+            torch.cuda.nvtx.range_pop()
         return logprobs, entropy
 
     @staticmethod
     def backward(ctx, dlogprobs: typing.Optional[torch.Tensor], dentropy: typing.Optional[torch.Tensor]):
-        rows, weight, flat_labels, maximum, accumulate, entropy_b = ctx.saved_tensors
-        shape, mode, temperature, group = ctx.call
-        if dlogprobs is None:  # only the entropy was used downstream
-            dlogprobs = torch.zeros((rows.shape[0],) if mode == 0 else (), device=rows.device, dtype=torch.float32)
-        # a gradient that autograd does not ask for (a frozen lm-head under LoRA, detached hidden states) is not computed
-        need_hidden, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        d_rows, d_weight = kernels.efficient_entropy_backward(
-            dlogprobs, dentropy, rows, weight, flat_labels, maximum, accumulate, entropy_b, mode,
-            False,  # should_return_fp32_grad: autograd wants the inputs' dtype
-            temperature, group, need_d_hidden=need_hidden, need_d_weight=need_weight,
-        )  # fmt: skip
+        torch.cuda.nvtx.range_push("LinearCrossEntropy-backward")  # the reference's range (:93)
+        try:
+            rows, weight, flat_labels, maximum, accumulate, entropy_b = ctx.saved_tensors
+            shape, mode, temperature, group = ctx.call
+            if dlogprobs is None:  # only the entropy was used downstream
+                dlogprobs = torch.zeros((rows.shape[0],) if mode == 0 else (), device=rows.device, dtype=torch.float32)
+            # a gradient that autograd does not ask for (a frozen lm-head under LoRA, detached hidden states) is not computed
+            need_hidden, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+            d_rows, d_weight = kernels.efficient_entropy_backward(
+                dlogprobs, dentropy, rows, weight, flat_labels, maximum, accumulate, entropy_b, mode,
+                False,  # should_return_fp32_grad: autograd wants the inputs' dtype
+                temperature, group, need_d_hidden=need_hidden, need_d_weight=need_weight,
+            )  # fmt: skip
+        finally:
+            torch.cuda.nvtx.range_pop()
         return (d_rows.view(shape) if d_rows is not None else None), d_weight, None, None, None, None
 
 

@@ -164,24 +164,49 @@ def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 20
     return _EntropyFromLogits.apply(logits, torch.float32)
 
 
+class _SumPiSquaredFromLogits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits):
+        rows, V = _as_rows(logits)
+        R = rows.shape[0]
+        dev = logits.device
+        out = torch.empty((R,), device=dev, dtype=torch.float32)
+        keep = ctx.needs_input_grad[0]
+        lse = torch.empty((R,), device=dev, dtype=torch.float32) if keep else None
+        if R > 0:
+            with torch.cuda.device(dev):
+                rc = _abi.load().lce_logits_sum_pi_squared(
+                    rows.data_ptr(), rows.stride(0), R, V, _abi.dtype_code(logits.dtype), out.data_ptr(), _abi.ptr(lse), _abi.current_stream(dev)
+                )
+                _abi.check(rc, "lce_logits_sum_pi_squared")
+        if keep:
+            ctx.save_for_backward(rows, lse, out)
+            ctx.shape, ctx.dtype = logits.shape, logits.dtype
+        return out.reshape(logits.shape[:-1]).to(logits.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        rows, lse, s = ctx.saved_tensors
+        R, V = rows.shape
+        d = torch.empty((R, V), device=rows.device, dtype=rows.dtype)
+        g = g.reshape(-1).to(torch.float32).contiguous()
+        if R > 0:
+            with torch.cuda.device(rows.device):
+                rc = _abi.load().lce_logits_sum_pi_squared_backward(
+                    rows.data_ptr(), rows.stride(0), R, V, _abi.dtype_code(rows.dtype), lse.data_ptr(), s.data_ptr(), g.data_ptr(),
+                    d.data_ptr(), d.stride(0), _abi.current_stream(rows.device),
+                )  # fmt: skip
+                _abi.check(rc, "lce_logits_sum_pi_squared_backward")
+        return d.reshape(ctx.shape).to(ctx.dtype)
+
+
 def calculate_sum_pi_squared_from_logits(logits: torch.Tensor) -> torch.Tensor:
     """sum over the vocabulary of softmax(logits)**2 = exp(logsumexp(2*logits) - 2*logsumexp(logits));
-    shape ``logits.shape[:-1]``, dtype of ``logits``.  One pass over the logits.  The reference calls it on
-    the actor's logits while collecting log-probs (no graph); differentiating through it is not wired and
-    raises instead of returning a detached value."""
+    shape ``logits.shape[:-1]``, dtype of ``logits``.  One pass over the logits.  Differentiable like the reference's
+    plain-torch expression (``verl/utils/torch_functional.py:687-703``; the reference itself only calls it without a
+    graph): the backward is one more pass, ``d_logits = g * 2 p (p - sum p**2)``."""
     _require_gpu(logits)
-    if torch.is_grad_enabled() and logits.requires_grad:
-        raise NotImplementedError("calculate_sum_pi_squared_from_logits has no backward; call it under torch.no_grad()")
-    rows, V = _as_rows(logits)
-    R = rows.shape[0]
-    out = torch.empty((R,), device=logits.device, dtype=torch.float32)
-    if R > 0:
-        with torch.cuda.device(logits.device):
-            rc = _abi.load().lce_logits_sum_pi_squared(
-                rows.data_ptr(), rows.stride(0), R, V, _abi.dtype_code(logits.dtype), out.data_ptr(), _abi.current_stream(logits.device)
-            )
-            _abi.check(rc, "lce_logits_sum_pi_squared")
-    return out.reshape(logits.shape[:-1]).to(logits.dtype)
+    return _SumPiSquaredFromLogits.apply(logits)
 
 
 def masked_sum(values, mask, axis=None):

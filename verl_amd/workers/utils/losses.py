@@ -284,12 +284,30 @@ def batch_lens(data):
 
 
 def _padded(t: torch.Tensor, width: int) -> torch.Tensor:
-    """A batch field as ``[batch, width]``: nested (jagged) fields are padded with zeros like ``to_padded_tensor``."""
+    """A batch field as exactly ``[batch, width]``: nested (jagged) fields are padded with zeros like
+    ``to_padded_tensor``, then cut or zero-padded to ``width`` (a jagged tensor without a cached longest row can come
+    back wider than its longest row; columns beyond every row's length hold padding only)."""
     if t.is_nested:
         t = torch.nested.to_padded_tensor(t, 0.0)
-    if t.shape[1] < width:
+    if t.shape[1] > width:
+        t = t[:, :width]
+    elif t.shape[1] < width:
         t = torch.nn.functional.pad(t, (0, width - t.shape[1]))
-    return t
+    return t.contiguous()
+
+
+def response_width(data, response_lens) -> int:
+    """Padded width of the response slice as ``no_padding_2_padding`` picks it (``verl/workers/utils/padding.py:112-124``):
+    for nested batches the non-tensor entry ``max_response_len`` when it is there and not negative, else the longest
+    response; for padded batches the width of ``responses``."""
+    responses = data["responses"]
+    if not responses.is_nested:
+        return int(responses.shape[1])
+    given = _get(data, "max_response_len")
+    given = getattr(given, "data", given)  # (a tensordict NonTensorData wraps its payload)
+    if given is not None and int(given) >= 0:
+        return int(given)
+    return int(response_lens.max().item())
 
 
 def metric_aggregation_for(dp_size, batch_num_tokens, global_batch_size, loss_scale_factor):
@@ -342,9 +360,10 @@ def ppo_loss(config, model_output, data, dp_group=None):
     metric_aggregation = metric_aggregation_for(**info)
 
     prompt_lens, response_lens = batch_lens(data)
-    response_mask = data["response_mask"]
-    width = response_mask.shape[1] if not response_mask.is_nested else int(response_lens.max().item())
-    response_mask = _padded(response_mask, width).to(bool)
+    width = response_width(data, response_lens)
+    if int(response_lens.max().item()) > width:
+        raise ValueError(f"max_response_len = {width} is shorter than the longest response ({int(response_lens.max().item())})")
+    response_mask = _padded(data["response_mask"], width).to(bool)
     use_kl = bool(_cfg(config, "use_kl_loss", False))
     is_weights = _get(data, "rollout_is_weights")
     policy_loss, m = fused_ppo_loss_packed(
