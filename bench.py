@@ -319,7 +319,7 @@ def run_mfma_ceiling(args):
     ]
     g = torch.Generator(device=dev).manual_seed(99)
     cases = []
-    seconds = 0.6
+    seconds = 1.5
 
     def timed(fn, flops):
         fn(); fn()
@@ -386,12 +386,83 @@ def run_mfma_ceiling(args):
     print(json.dumps(out), flush=True)
 
 
+SWEEP_WORKLOAD = "token-sweep"
+
+
+def run_token_sweep(args):
+    """Forward and forward + backward of the Qwen2.5-7B head (H=3584, V=152064, bf16) at token counts from 128 to 2048 in
+    steps of 64 plus ragged counts: the band where the launchers switch code paths (at 64, 128, 512 and 1280 tokens) and
+    where the bound changes from HBM (one stream of W per pass: 4 passes of [V, H] forward + backward) to the matrix
+    pipes (ridge at 2.5e15 / 8e12 = 312 tokens forward, 417 forward + backward).  Each point: median of `--steps`
+    runs; `frac` is the larger of the two floors (algorithmic bytes / 8 TB/s, algorithmic FLOP / 2.5 PFLOP/s) over the
+    measured time.  Token tiles are 256 wide, so the matrix-pipe work is that of T rounded up to 256."""
+    import torch
+
+    from verl_amd import linear_cross_entropy
+
+    dev = torch.device("cuda:0")
+    H, V = 3584, 152064
+    g = torch.Generator(device=dev).manual_seed(1234)
+    w = (torch.randn(V, H, device=dev, generator=g) * 0.02).bfloat16()
+    counts = sorted(set(list(range(128, 2049, 64)) + [200, 333, 500, 777, 1000, 1300, 1500, 1999]))
+    n = max(3, args.steps)
+
+    def timed(step):
+        for _ in range(max(1, args.warmup)):
+            step()
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        ev[0].record()
+        for i in range(n):
+            step()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        return sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(n))[n // 2]
+
+    rows = []
+    for T in counts:
+        h = torch.randn(T, H, device=dev, generator=g).bfloat16()
+        y = torch.randint(0, V, (T,), device=dev, generator=g)
+        g_lp, g_ent = torch.randn(T, device=dev, generator=g), torch.randn(T, device=dev, generator=g)
+
+        def fwd():
+            with torch.no_grad():
+                linear_cross_entropy(h, w, y, 1.0, "none")
+
+        hg, wg = h.clone().requires_grad_(True), w.requires_grad_(True)
+
+        def fwd_bwd():
+            hg.grad = None
+            wg.grad = None
+            lp, ent = linear_cross_entropy(hg, wg, y, 1.0, "none")
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+
+        rec = {"T": T}
+        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 4.0, 6.0 * T * V * H)):
+            ms = timed(fn)
+            hbm_ms = passes * V * H * 2.0 / PEAK_HBM * 1e3
+            mfma_ms = flops / PEAK_BF16 * 1e3
+            rec[name] = {"ms": ms, "bound": "hbm" if hbm_ms >= mfma_ms else "mfma", "floor_ms": max(hbm_ms, mfma_ms),
+                         "frac": max(hbm_ms, mfma_ms) / ms, "tokens_per_s": T / (ms * 1e-3)}
+        w.requires_grad_(False)
+        rows.append(rec)
+    out = {
+        "metric": "fraction of the applicable roofline over token counts 128..2048 (forward; forward + backward)",
+        "value": min(r["fwd_bwd"]["frac"] for r in rows), "unit": "fraction (worst point, fwd+bwd)", "n_gpus": 1, "steps": n,
+        "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": {"workload": SWEEP_WORKLOAD, "H": H, "V": V},
+        "rows": rows, "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS) + sorted(LOGITS_WORKLOADS) + [CEILING_WORKLOAD])
+    ap.add_argument("--workload", default="qwen2.5-7b-head-T16384", choices=sorted(WORKLOADS) + sorted(LOGITS_WORKLOADS) + [CEILING_WORKLOAD, SWEEP_WORKLOAD])
+    ap.add_argument("--tokens", type=int, default=0, help="another token count T for the chosen head workload (its name gets the suffix @T<count>)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--vchunk", type=int, default=-1)
@@ -415,6 +486,9 @@ def main():
     if args.workload == CEILING_WORKLOAD:
         run_mfma_ceiling(args)
         return
+    if args.workload == SWEEP_WORKLOAD:
+        run_token_sweep(args)
+        return
 
     import torch
 
@@ -435,13 +509,19 @@ def main():
         K.set_vocab_chunk(args.vchunk)
     dev = torch.device("cuda:0")
     T, H, V, tau, wstd, nseq, shortest, ppo = WORKLOADS[args.workload][:8]
+    workload_name = args.workload
+    if args.tokens > 0:
+        if nseq:
+            raise SystemExit("--tokens: only for workloads without sequence structure")
+        T = args.tokens
+        workload_name = f"{args.workload}@T{T}"
     flags = {"variant": args.variant, "vchunk": args.vchunk, "split_backward": bool(args.split_backward),
              "options": sorted(args.option + (["2=1"] if args.dlogits_tokens_first else []))}
     if args.frozen_head:
         flags["frozen_head"] = True
     state = library_state(lib, T, H, V, flags)
     if args.print_state:
-        print(json.dumps({"workload": args.workload, "state": state}), flush=True)
+        print(json.dumps({"workload": workload_name, "state": state}), flush=True)
         return
     fwd_only = len(WORKLOADS[args.workload]) > 8 and WORKLOADS[args.workload][8]
     g = torch.Generator(device=dev).manual_seed(1234 + 2)
@@ -574,12 +654,12 @@ def main():
                 "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                 "ms_per_step": ms_per_step, "step_ms": step_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                 "dtype": "bf16", "data": "synthetic",
-                "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
+                "config": {"workload": workload_name, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
                 "algorithmic_tflops": flops / (elapsed / args.steps) / 1e12,
                 "frac_of_bf16_peak": flops / (elapsed / args.steps) / PEAK_BF16,
                 "roofline": {"bound": "mfma", "kernel": "lce_fwd_kernel", "achieved": flops / (k["avg_ms"] * 1e-3) / 1e12,
                              "peak": PEAK_BF16 / 1e12, "unit": "TFLOP/s", "frac": flops / (k["avg_ms"] * 1e-3) / PEAK_BF16,
-                             "traffic": measured_traffic(args.workload, "lce_fwd_kernel", state),
+                             "traffic": measured_traffic(workload_name, "lce_fwd_kernel", state),
                              "avg_launch_ms": k["avg_ms"], "flops_per_launch": flops},
                 "kernels": kernels,
                 "cpu_baseline": None,
@@ -592,10 +672,10 @@ def main():
             "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
             "data": "synthetic",
-            "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
+            "config": {"workload": workload_name, "T": T, "H": H, "V": V, "temperature": tau, "pass": "fwd"},
             "roofline": {"bound": "hbm", "kernel": "lce_fwd_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                          "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
-                         "traffic": measured_traffic(args.workload, "lce_fwd_kernel", state),
+                         "traffic": measured_traffic(workload_name, "lce_fwd_kernel", state),
                          "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes},
             "kernels": kernels,
             "cpu_baseline": None,
@@ -609,7 +689,7 @@ def main():
         "peak": PEAK_BF16 / 1e12,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16,
-        "traffic": measured_traffic(args.workload, dom, state),
+        "traffic": measured_traffic(workload_name, dom, state),
         "avg_launch_ms": mfma[dom]["avg_ms"],
         "flops_per_launch": flops_per_launch,
     }
@@ -624,7 +704,7 @@ def main():
         nbytes = (1.0 + n_grads) * V * H * 2.0 / k["launches_per_step"]  # (W read twice, d_weight written; --frozen-head: W read twice)
         roofline = {"bound": "hbm", "kernel": "lce_bwd_chunk_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                     "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
-                    "traffic": measured_traffic(args.workload, "lce_bwd_chunk_kernel", state),
+                    "traffic": measured_traffic(workload_name, "lce_bwd_chunk_kernel", state),
                     "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes,
                     "step_bytes": (2.0 + n_grads) * V * H * 2.0, "step_GBps": (2.0 + n_grads) * V * H * 2.0 / (elapsed / args.steps) / 1e9}
     out = {
@@ -641,7 +721,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": args.workload, "T": T, "H": H, "V": V, "temperature": tau,
+        "config": {"workload": workload_name, "T": T, "H": H, "V": V, "temperature": tau,
                    "pass": ("fwd+ppo_loss+bwd" if ppo else "fwd+bwd") + (" (d_hidden only: frozen head)" if args.frozen_head else ""),
                    "tokens_with_gradient": t_active},
         "memory": memory,

@@ -51,8 +51,9 @@ def test_abi_version_and_error_string():
 
 
 def test_default_chunk_rule_and_workspace_budget():
-    """Default: chunks of 8192 vocabulary columns (wider while one d_logits buffer stays within 256 MiB), so the backward's
-    workspace at config 2 is under 1 GiB; a byte budget (kernels.set_workspace_budget / LCE_OPT_WORKSPACE_BUDGET) makes
+    """Default: chunks of 16384 vocabulary columns (wider while one d_logits buffer stays within 256 MiB; from 8192 columns
+    on while one stays within 1 GiB; narrower once two of them would pass 4 GiB), so the backward's workspace at config 2
+    is under 1.5 GiB; a byte budget (kernels.set_workspace_budget / LCE_OPT_WORKSPACE_BUDGET) makes
     the library pick the widest chunk that fits, never exceeding its upper bound and never going below 2048 columns; an
     explicit chunk width wins over both."""
     from verl_amd.utils.kernel import kernels
@@ -62,8 +63,8 @@ def test_default_chunk_rule_and_workspace_budget():
     gate = 0.25 * T * V * 2 + 4 * V * H
     try:
         default = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
-        assert default < (1 << 30)
-        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 8192) == default  # 19 chunks of 8192 columns
+        assert default < (3 << 29)
+        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 15360) == default  # the 10 chunks that 16384 columns need, evened out
         # few tokens: the whole vocabulary in one chunk (one single-buffered d_logits tile)
         few = lib.lce_backward_workspace_bytes(64, H, V, 0, 0)
         assert few == lib.lce_backward_workspace_bytes(64, H, V, 0, 152064)
@@ -72,7 +73,7 @@ def test_default_chunk_rule_and_workspace_budget():
         assert lib.lce_backward_workspace_bytes(262144, 4096, 128256, 0, 0) == lib.lce_backward_workspace_bytes(262144, 4096, 128256, 0, 4096)
         assert lib.lce_backward_workspace_bytes(1 << 21, 4096, 128256, 0, 0) == lib.lce_backward_workspace_bytes(1 << 21, 4096, 128256, 0, 2048)
         sizes = []
-        for budget in (600 << 20, 1 << 30, 2 << 30, 1 << 40):
+        for budget in (600 << 20, 1 << 30, 5 << 29, 1 << 40):
             kernels.set_workspace_budget(budget)
             n = lib.lce_backward_workspace_bytes(T, H, V, 0, 0)
             sizes.append(n)
@@ -84,7 +85,7 @@ def test_default_chunk_rule_and_workspace_budget():
         kernels.set_workspace_budget(1 << 20)
         assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) == lib.lce_backward_workspace_bytes(T, H, V, 0, 2048)
         # an explicit width is not touched by the budget
-        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 8192) == default
+        assert lib.lce_backward_workspace_bytes(T, H, V, 0, 15360) == default
     finally:
         kernels.set_workspace_budget(0)
     assert lib.lce_backward_workspace_bytes(T, H, V, 0, 0) == default

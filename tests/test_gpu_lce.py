@@ -148,6 +148,36 @@ def test_reductions(reduction):
     torch.testing.assert_close(dw.float(), rdw, atol=2e-2, rtol=4e-2)
 
 
+def test_profiler_ranges_of_the_reference_bracket_forward_and_backward(monkeypatch):
+    """verl/utils/kernel/linear_cross_entropy.py:66,93: the autograd node's forward and backward run inside the ranges
+    "LinearCrossEntropy-forward" / "LinearCrossEntropy-backward" (roctx on this platform).  The ranges are pushed and
+    popped in pairs, also when the launcher raises, and the results inside them are the oracle's."""
+    from verl_amd import linear_cross_entropy
+
+    seen = []
+    push, pop = torch.cuda.nvtx.range_push, torch.cuda.nvtx.range_pop
+    monkeypatch.setattr(torch.cuda.nvtx, "range_push", lambda name: (seen.append(("push", name)), push(name))[1])
+    monkeypatch.setattr(torch.cuda.nvtx, "range_pop", lambda: (seen.append(("pop", None)), pop())[1])
+    T, H, V = 300, 128, 1003
+    h, w, y, g_lp, g_ent = _uniform_case(T, H, V, torch.bfloat16, seed=4)
+    h1, w1 = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    lp, ent = linear_cross_entropy(h1, w1, y, 0.9, "none")
+    assert seen == [("push", "LinearCrossEntropy-forward"), ("pop", None)]
+    torch.autograd.backward([lp, ent], [g_lp, g_ent])
+    assert seen[2:] == [("push", "LinearCrossEntropy-backward"), ("pop", None)]
+    rlp, rent = O.lce_forward(h, w, y, 0.9)
+    rdh, rdw = O.lce_backward(g_lp, g_ent, h, w, y, 0.9)
+    torch.testing.assert_close(lp, rlp, atol=2e-2, rtol=0)
+    torch.testing.assert_close(ent, rent, atol=2e-2, rtol=0)
+    torch.testing.assert_close(h1.grad.float(), rdh, atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(w1.grad.float(), rdw, atol=2e-2, rtol=4e-2)
+    # a failing launcher (bad reduction string) still closes its range
+    del seen[:]
+    with pytest.raises(ValueError):
+        linear_cross_entropy(h, w, y, 0.9, "median")
+    assert seen == [("push", "LinearCrossEntropy-forward"), ("pop", None)]
+
+
 def test_api_contract_on_device():
     from verl_amd import linear_cross_entropy
     from verl_amd.utils.kernel import kernels

@@ -204,7 +204,12 @@ int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
   for (int S = bc; S <= max_splits && (S <= nvt || S == bc); ++S) {
     const int64_t per_xcd = ((int64_t)ntt * S + 7) / 8;
     const int64_t rounds = (per_xcd + kNumCUs / 8 - 1) / (kNumCUs / 8);
-    const int64_t cost = rounds * (4 * ((nvt + S - 1) / S) + 1);
+    const int64_t tiles = (nvt + S - 1) / S;
+    // the longer a workgroup's walk, the further the 32 workgroups of an XCD drift apart and the fewer of them share a
+    // fetched slab: + 2 % per 100 tiles (measured, forward launch: T=16384, 149 tiles per workgroup 13.47 ms, 75 tiles
+    // in two rounds 13.30, 50 in three 13.26, 38 in four 13.51; T=32768, V=128256: 126 tiles 25.23 ms, 63 24.88,
+    // 42 24.69, 32 24.97; T=65536, H=5120: 149 tiles 74.8 ms, 75 72.6, 50 73.4)
+    const int64_t cost = rounds * (4 * tiles + 1) * (10000 + 2 * tiles);
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = S; }
   }
   return best;
@@ -425,18 +430,25 @@ BwdLayout bwd_layout_for(const Tuning& tu, int64_t T, int64_t H, int64_t V, size
 BwdLayout bwd_layout(const Tuning& tu, int64_t T, int64_t H, int64_t V, size_t esz, int64_t vchunk, int64_t gt = 256, int64_t gv = 256) {
   if (vchunk <= 0) {
     // Upper bound of the whole workspace: a quarter of one [T, V] tile plus one fp32 [V, H].  Below it the default is
-    // a chunk of 8192 columns, wider while one d_logits buffer stays within 256 MiB (few tokens: the whole vocabulary
-    // in one chunk, which saves a pass over W per chunk), narrower once two such buffers would pass 4 GiB.  Measured at config 2 on the 16x16x32 loop: 8192 columns cost
-    // 0.4% against the widest chunk the bound allows (56.2 against 56.0 ms per step) with 0.9 instead of 2.9 GiB of
-    // workspace; 4096 columns cost 6%.  A byte budget (LCE_OPT_WORKSPACE_BUDGET) replaces the default rule: the widest
-    // chunk whose workspace fits it, but never fewer than 2048 columns.
+    // a chunk of 16384 columns, wider while one d_logits buffer stays within 256 MiB (few tokens: the whole vocabulary
+    // in one chunk, which saves a pass over W per chunk), narrower once two such buffers would pass 4 GiB.  Measured on
+    // one box, three interleaved runs each: T=16384, H=3584, V=152064: 8192 columns 54.80 ms per step, 16384 columns
+    // 54.27, 24576 columns 54.26 (each halving of the chunk count halves the fp32 read-modify-write passes over d_hidden
+    // and the launch boundaries; 0.15 ms on another box); T=32768, H=4096, V=128256: 66.67 against 65.97; 4096 columns
+    // cost 6 %; up to 8192 tokens the width makes no difference from 16384 columns on.  T=65536, H=5120, V=152064, where a
+    // buffer of 16384 columns takes 2 GiB: 229.1 ms for the backward's launches with 8192 columns, 234.7 with 15360.  A byte budget (LCE_OPT_WORKSPACE_BUDGET) replaces the default
+    // rule: the widest chunk whose workspace fits it, but never fewer than 2048 columns.
     double gate = 0.25 * (double)T * V * esz + 4.0 * (double)V * H;
     vchunk = round_up(V, 256);
     if (tu.ws_budget > 0) {
       if ((double)tu.ws_budget < gate) gate = (double)tu.ws_budget;
     } else {
       int64_t cols = (((int64_t)256 << 20) / (T * (int64_t)esz)) / 256 * 256;
-      if (cols < 8192) cols = 8192;
+      if (cols < 16384) {
+        // many tokens: 16384 columns while one d_logits buffer stays within 1 GiB, never fewer than 8192
+        cols = (((int64_t)1 << 30) / (T * (int64_t)esz)) / 256 * 256;
+        cols = cols > 16384 ? 16384 : cols < 8192 ? 8192 : cols;
+      }
       // very many tokens: the two d_logits buffers stay within 4 GiB (at 262144 tokens chunks of 4096 columns take as
       // long as chunks of 8192, 567.1 against 567.2 ms per actor step, with 10.1 instead of 14.1 GiB of workspace: a
       // launch is long enough there for its fixed costs not to show)
