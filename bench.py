@@ -366,6 +366,18 @@ def run_mfma_ceiling(args):
                 cases.append({"shape": name, "M": M, "N": N, "K": K, "data": data, "engine": "lce_gemm_tn (16x16x32 loop, K-major operands, fp32 C)", **r})
                 del At, Bk, Cf
             del A, B
+    # what the memory system of this box sustains with vendor kernels, for the HBM-bound rows (few tokens, logits twins):
+    # write-only (fill), read-only (sum) and read + write (copy) over 2 GiB buffers
+    buf = torch.empty(1 << 29, device=dev, dtype=torch.float32)
+    dst = torch.empty_like(buf)
+    nbytes = buf.numel() * 4.0
+    hbm = []
+    for name, fn, moved in (("fill (write only)", lambda: buf.fill_(1.0), nbytes), ("sum (read only)", lambda: buf.sum(), nbytes),
+                            ("copy (read + write)", lambda: dst.copy_(buf), 2.0 * nbytes)):
+        r = timed(fn, 0.0)
+        hbm.append({"op": f"torch {name}, 2 GiB", "ms": r["ms"], "TBps": moved / (r["ms"] * 1e-3) / 1e12, "socket_watts": r["socket_watts"],
+                    "shader_mhz": r["shader_mhz"]})
+    del buf, dst
     sampler.stop()
     rand = [c for c in cases if c["data"] != "zeros"]
     best_lib = max(c["tflops"] for c in rand if c["engine"].startswith("lce_"))
@@ -381,6 +393,7 @@ def run_mfma_ceiling(args):
         "headline_step_ms_at_best_rate": step_flops / (max(best_lib, best_blas) * 1e12) * 1e3,
         "power_cap_watts": getattr(sampler, "cap_watts", None), "power_sampler_error": sampler.error,
         "cases": cases,
+        "hbm": hbm,
         "roofline": None, "cpu_baseline": None,
     }
     print(json.dumps(out), flush=True)
@@ -696,7 +709,7 @@ def main():
     # Algorithmic FLOPs of the step: forward 2*T*V*H, backward 4*Ta*V*H over the Ta tokens that carry an upstream gradient
     # (the mandated recompute of the logits is executed but not counted).  With Ta = T this is the reference's 6*T*V*H.
     algorithmic = (2.0 * T + 2.0 * n_grads * t_active) * V * H / (elapsed / args.steps)
-    if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM:
+    if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM and "lce_bwd_chunk_kernel" in kernels:
         # few tokens: the step is four streaming passes over [V, H] in the input dtype (W read by the forward, by the
         # d_logits tiles and by the d_hidden GEMM; d_weight written), and HBM bounds it.  The backward's two launches
         # (d_logits tiles; both gradient GEMMs) account for three of the four.
