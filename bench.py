@@ -172,6 +172,10 @@ def run_logits_workload(args, name):
     from verl_amd.utils import torch_functional as F
 
     lib = _abi.load()
+    state = {"abi": int(lib.lce_abi_version())}  # (these kernels have no workspace and no tuning flags)
+    if args.print_state:
+        print(json.dumps({"workload": name, "state": state}), flush=True)
+        return
     dev = torch.device("cuda:0")
     R, V = LOGITS_WORKLOADS[name][:2]
     combined = len(LOGITS_WORKLOADS[name]) > 2 and LOGITS_WORKLOADS[name][2]
@@ -236,7 +240,7 @@ def run_logits_workload(args, name):
         "data": "synthetic",
         "config": {"workload": name, "R": R, "V": V, "pass": "1 x fwd + 1 x bwd (one autograd node)" if combined else "2 x fwd + 2 x bwd (+ torch's accumulation of the two d_logits)"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-                     "frac": achieved / PEAK_HBM, "traffic": None, "avg_launch_ms": kernels[dom]["avg_ms"],
+                     "frac": achieved / PEAK_HBM, "traffic": measured_traffic(name, dom, state), "avg_launch_ms": kernels[dom]["avg_ms"],
                      "bytes_per_launch": bytes_per_launch[dom]},
         "kernels": kernels,
         "cpu_baseline": None,

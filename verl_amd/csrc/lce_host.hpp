@@ -199,19 +199,33 @@ constexpr int kMaxSplits = 256;
 int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
   const int bc = 32 / block_rows(ntt);
   if (max_splits < bc) return max_splits > 1 ? max_splits : 1;  // (a caller with very little room for partial results)
-  int best = bc;
-  int64_t best_cost = -1;
-  for (int S = bc; S <= max_splits && (S <= nvt || S == bc); ++S) {
+  auto cost_of = [&](int S, int64_t* tiles_out) {
     const int64_t per_xcd = ((int64_t)ntt * S + 7) / 8;
     const int64_t rounds = (per_xcd + kNumCUs / 8 - 1) / (kNumCUs / 8);
     const int64_t tiles = (nvt + S - 1) / S;
-    // the longer a workgroup's walk, the further the 32 workgroups of an XCD drift apart and the fewer of them share a
-    // fetched slab: + 2 % per 100 tiles (measured, forward launch: T=16384, 149 tiles per workgroup 13.47 ms, 75 tiles
-    // in two rounds 13.30, 50 in three 13.26, 38 in four 13.51; T=32768, V=128256: 126 tiles 25.23 ms, 63 24.88,
-    // 42 24.69, 32 24.97; T=65536, H=5120: 149 tiles 74.8 ms, 75 72.6, 50 73.4)
-    const int64_t cost = rounds * (4 * tiles + 1) * (10000 + 2 * tiles);
+    if (tiles_out) *tiles_out = tiles;
+    return rounds * (4 * tiles + 1);
+  };
+  int best = bc;
+  int64_t best_cost = -1;
+  for (int S = bc; S <= max_splits && (S <= nvt || S == bc); ++S) {
+    const int64_t cost = cost_of(S, nullptr);
     if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = S; }
   }
+  // Among the split counts within 2 % of the fewest tile-times, one that makes a workgroup walk 48 to 96 tiles is
+  // preferred: the longer the walk, the further the 32 workgroups of an XCD drift apart and the fewer of them share a
+  // fetched slab; the shorter, the more the rounds' ramp-up shows.  Measured, forward launch (tiles per workgroup: ms):
+  // T=16384, H=3584, V=152064: 149: 13.47, 75: 13.30, 50: 13.26, 38: 13.51, fetched through the fabric 59.6 -> 30.8 GB;
+  // T=32768, H=4096, V=128256: 126: 25.23, 63: 24.88, 42: 24.69, 32: 24.97; T=65536, H=5120: 149: 74.8, 75: 72.6, 50: 73.4.
+  int pick = -1;
+  int64_t pick_cost = -1;
+  for (int S = bc; S <= max_splits && (S <= nvt || S == bc); ++S) {
+    int64_t tiles;
+    const int64_t cost = cost_of(S, &tiles);
+    if (cost * 100 > best_cost * 102 || tiles < 48 || tiles > 96) continue;
+    if (pick_cost < 0 || cost < pick_cost) { pick_cost = cost; pick = S; }
+  }
+  if (pick > 0) best = pick;
   return best;
 }
 
