@@ -35,39 +35,62 @@ LCE_DEV uint32_t label_row(const LabelTerm& lt, int64_t tok, float& G) {
 // number G * (1 - p) is formed in fp32 instead of as the difference of G (fp32) and G * p (rounded to 16 bits).
 // Zero for tokens without upstream gradient and for labels outside this call's rows of W.  H a multiple of 8.
 template <typename T>
-__global__ __launch_bounds__(256) void label_coef_kernel(const T* h, int64_t ldh, const T* W, int64_t ldw, const int64_t* labels,
-                                                         int64_t v0, int64_t V, int64_t ntok, int64_t H, const float* maximum,
-                                                         const float* accumulate, const float* entropy_b, const float* g_lp,
-                                                         int64_t g_stride, float g_scale, const float* g_ent, float rcp_tau,
-                                                         float c, float* coef) {
+struct CoefArgs {
+  const T* h;
+  int64_t ldh;
+  const T* W;
+  int64_t ldw;
+  const int64_t* labels;
+  int64_t v0, V;      // this call's rows of W are vocabulary ids [v0, v0 + V)
+  int64_t ntok, H;
+  const float* maximum;
+  const float* accumulate;
+  const float* entropy_b;
+  const float* g_lp;  // upstream gradient of the log-probabilities, stride 0 when all tokens share one value
+  int64_t g_stride;
+  float g_scale;      // 1, or 1 / tokens for the mean
+  const float* g_ent; // upstream gradient of the entropy, or null
+  float rcp_tau, c;   // 1 / temperature, log2(e) / temperature
+  float* coef;        // [ntok]
+};
+
+// the coefficient of token t, computed by one whole wave (the same value in every lane)
+template <typename T>
+LCE_DEV float label_coef_wave(const CoefArgs<T>& a, int64_t t) {
   static_assert(sizeof(T) == 2, "16-bit inputs");
   typedef typename VecOf<T, 8>::type vec_t;
   const int lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= ntok) return;
-  const float glp = g_lp[t * g_stride] * g_scale;
-  const float gent = g_ent ? g_ent[t] : 0.f;
-  const int64_t y = labels[t] - v0;
+  const float glp = a.g_lp[t * a.g_stride] * a.g_scale;
+  const float gent = a.g_ent ? a.g_ent[t] : 0.f;
+  const int64_t y = a.labels[t] - a.v0;
   float out = 0.f;
-  if ((glp != 0.f || gent != 0.f) && y >= 0 && y < V) {  // (uniform over the wave)
-    const T* hr = h + t * ldh;
-    const T* wr = W + y * ldw;
+  if ((glp != 0.f || gent != 0.f) && y >= 0 && y < a.V) {  // (uniform over the wave)
+    const T* hr = a.h + t * a.ldh;
+    const T* wr = a.W + y * a.ldw;
     float x = 0.f;
-    for (int64_t k = (int64_t)lane * 8; k < H; k += 64 * 8) {
-      const vec_t a = *reinterpret_cast<const vec_t*>(hr + k);
-      const vec_t b = *reinterpret_cast<const vec_t*>(wr + k);
+    for (int64_t k = (int64_t)lane * 8; k < a.H; k += 64 * 8) {
+      const vec_t u = *reinterpret_cast<const vec_t*>(hr + k);
+      const vec_t w = *reinterpret_cast<const vec_t*>(wr + k);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x = __builtin_fmaf((float)a[e], (float)b[e], x);
+      for (int e = 0; e < 8; ++e) x = __builtin_fmaf((float)u[e], (float)w[e], x);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
-    const float lse2 = (maximum[t] + logf(accumulate[t])) * kLog2e;
-    const float G = glp * rcp_tau;
-    const float C1 = -gent * rcp_tau * rcp_tau;
-    const float C0 = -G + gent * entropy_b[t] * rcp_tau;
-    out = fast_exp2(__builtin_fmaf(x, c, -lse2)) * __builtin_fmaf(x, C1, C0) + G;
+    const float lse2 = (a.maximum[t] + logf(a.accumulate[t])) * kLog2e;
+    const float G = glp * a.rcp_tau;
+    const float C1 = -gent * a.rcp_tau * a.rcp_tau;
+    const float C0 = -G + gent * a.entropy_b[t] * a.rcp_tau;
+    out = fast_exp2(__builtin_fmaf(x, a.c, -lse2)) * __builtin_fmaf(x, C1, C0) + G;
   }
-  if (lane == 0) coef[t] = out;
+  return out;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void label_coef_kernel(CoefArgs<T> a) {
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= a.ntok) return;
+  const float out = label_coef_wave(a, t);
+  if ((threadIdx.x & 63) == 0) a.coef[t] = out;
 }
 
 // keys[k] = label row of the k-th listed token (rows[k], or k itself without a list), vals[k] = that token;
@@ -179,6 +202,33 @@ inline __global__ __launch_bounds__(256) void label_sort_single_kernel(LabelTerm
   __shared__ int gh[256];
   const int tid = threadIdx.x;
   const int64_t n = n_rows ? (int64_t)*n_rows : T;
+  if (n <= 256) {
+    // few tokens: every thread ranks its own item among all of them (stable: ties by position), one pass, no radix
+    // passes (16 -> 4 us with 64 tokens, where the whole backward takes 0.7 ms)
+    uint32_t key = kNoRow;
+    int tok = -1;
+    if (tid < n) {
+      tok = rows ? rows[tid] : tid;
+      float G;
+      key = label_row(lt, tok, G);
+    }
+    tab[tid] = (int)key;  // (bit pattern; compared as unsigned below)
+    __syncthreads();
+    int rank = 0;
+    for (int j = 0; j < 256; ++j) {
+      const uint32_t kj = (uint32_t)tab[j];
+      rank += (kj < key || (kj == key && j < tid)) ? 1 : 0;
+    }
+    uint32_t* kout = (passes & 1) ? keys1 : keys0;  // where the caller reads the result of `passes` radix passes
+    int* vout = (passes & 1) ? vals1 : vals0;
+    kout[rank] = key;
+    vout[rank] = tok;
+    for (int k = 256 + tid; k < kSortBlock; k += 256) {
+      kout[k] = kNoRow;
+      vout[k] = -1;
+    }
+    return;
+  }
   for (int k = tid; k < kSortBlock; k += 256) {
     uint32_t key = kNoRow;
     int tok = -1;
@@ -239,6 +289,119 @@ __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys
       const int64_t tok = toks[j];
       const float G = lt.g_lp[tok * lt.g_stride] * lt.scale;
       const vec_t hv = *reinterpret_cast<const vec_t*>(h + tok * ldh + c);
+#pragma unroll
+      for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(G, (float)hv[e], acc[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] += (float)cur[e];
+    ovec_t out;
+#pragma unroll
+    for (int e = 0; e < N; ++e) out[e] = (TOUT)acc[e];
+    *reinterpret_cast<ovec_t*>(row + c) = out;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Few tokens (at most 128, 16-bit inputs): a backward of well under a millisecond, where every small launch costs
+// 5 us or more.  One launch before the d_logits pass and one after the gradient GEMMs replace eight:
+//   few_prep_kernel    the list of tokens with a gradient (active_count / active_rows), the label coefficients
+//                      (label_coef) and the compact copy of hidden (gather_rows);
+//   few_finish_kernel  d_hidden from its partials (dh_finish) and the one-hot rows of d_weight (dw_label_rows), which
+//                      finds the tokens that share a label by comparing all pairs instead of sorting them.
+// Results are the same bits as from the separate kernels: same expressions, same order of every sum.
+// ------------------------------------------------------------------------------------------------------------------
+
+// Workgroup b: every workgroup lists the tokens itself (ballots over at most 128 gradients); workgroup 0 stores the
+// list; workgroup b then owns compact position b: the row of hidden it copies to Ht[b] (zeros from the list's end up to
+// the next multiple of 64, the K granule of the d_weight product) and that token's label coefficient (wave 0).
+// Grid: tokens rounded up to 64, at most rpad.  a.coef may be null (no coefficients wanted).
+template <typename T>
+__global__ __launch_bounds__(256) void few_prep_kernel(CoefArgs<T> a, T* Ht, int64_t ldHt, int64_t rpad, int* rows, int* inv, int* n_rows) {
+  static_assert(sizeof(T) == 2, "16-bit inputs");
+  typedef typename VecOf<T, 8>::type vec_t;
+  __shared__ int list[128];
+  __shared__ int cnt[2];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  bool on = false;
+  int before = 0;
+  if (wave < 2) {
+    on = tid < a.ntok && token_is_active(a.g_lp, a.g_stride, a.g_ent, tid);
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(on);
+    before = (int)__popcll(m & ((1ull << lane) - 1ull));
+    if (lane == 0) cnt[wave] = (int)__popcll(m);
+  }
+  __syncthreads();
+  const int n = cnt[0] + cnt[1];
+  if (wave < 2) {
+    const int pos = (wave ? cnt[0] : 0) + before;
+    if (on) list[pos] = tid;
+    if (blockIdx.x == 0 && tid < a.ntok) {
+      inv[tid] = on ? pos : -1;
+      if (on) rows[pos] = tid;
+      else if (a.coef) a.coef[tid] = 0.f;
+    }
+  }
+  if (blockIdx.x == 0 && tid == 0) *n_rows = n;
+  __syncthreads();
+  const int k = blockIdx.x;
+  const int64_t rend = ((int64_t)n + 63) / 64 * 64 < rpad ? ((int64_t)n + 63) / 64 * 64 : rpad;
+  if (k >= rend) return;
+  const int64_t tok = k < n ? list[k] : -1;
+  for (int64_t c = (int64_t)tid * 8; c < a.H; c += 256 * 8) {
+    vec_t v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (T)0.f;
+    if (tok >= 0) v = *reinterpret_cast<const vec_t*>(a.h + tok * a.ldh + c);
+    *reinterpret_cast<vec_t*>(Ht + (int64_t)k * ldHt + c) = v;
+  }
+  if (tok >= 0 && a.coef && wave == 0) {
+    const float out = label_coef_wave(a, tok);
+    if (lane == 0) a.coef[tok] = out;
+  }
+}
+
+// Workgroups [0, n_dh): d_hidden, as dh_finish_kernel with that many workgroups.  Workgroup n_dh + i: compact position
+// i of the token list; the first position of each label adds sum of G_t * hidden[t][:] over the positions with that
+// label, in order, to the label's row of d_weight (as dw_label_rows_kernel does over a sorted run).
+template <typename T, typename TOUT>
+__global__ __launch_bounds__(256) void few_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H,
+                                                         TOUT* d_hidden, LabelTerm lt, const T* W, int64_t ldw, int n_dh, const int* rows,
+                                                         const int* n_rows, const T* h, int64_t ldh, TOUT* dW) {
+  if ((int)blockIdx.x < n_dh) {
+    dh_finish_body<T, TOUT>(part, S, stride, inv, ntok, H, d_hidden, lt, W, ldw, (int64_t)blockIdx.x, (int64_t)n_dh);
+    return;
+  }
+  constexpr int N = 16 / (int)sizeof(T);
+  typedef typename VecOf<T, N>::type vec_t;
+  __shared__ uint32_t keys[128];
+  __shared__ float coefs[128];
+  __shared__ int toks[128];
+  const int i = (int)blockIdx.x - n_dh, tid = threadIdx.x;
+  const int n = *n_rows;
+  if (i >= n) return;
+  if (tid < n && tid < 128) {
+    const int tok = rows[tid];
+    float G;
+    keys[tid] = label_row(lt, tok, G);
+    coefs[tid] = G;
+    toks[tid] = tok;
+  }
+  __syncthreads();
+  const uint32_t key = keys[i];
+  if (key == kNoRow) return;
+  for (int j = 0; j < i; ++j)
+    if (keys[j] == key) return;  // (the same for every thread) an earlier position owns this row
+  TOUT* row = dW + (int64_t)key * H;
+  for (int64_t c = (int64_t)tid * N; c < H; c += 256 * N) {
+    typedef typename VecOf<TOUT, N>::type ovec_t;
+    const ovec_t cur = *reinterpret_cast<const ovec_t*>(row + c);
+    float acc[N];
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] = 0.f;
+    for (int j = i; j < n; ++j) {
+      if (keys[j] != key) continue;
+      const float G = coefs[j];
+      const vec_t hv = *reinterpret_cast<const vec_t*>(h + (int64_t)toks[j] * ldh + c);
 #pragma unroll
       for (int e = 0; e < N; ++e) acc[e] = __builtin_fmaf(G, (float)hv[e], acc[e]);
     }

@@ -269,8 +269,6 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
   int rc;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((T + 1023) / 1024)), dim3(256), 0, st, reinterpret_cast<uint32_t*>(p.xlabel), T);
-  if ((rc = check_launch("fill_zero_kernel"))) return rc;
   {
     ProfScope prof(PC_FWD, st);
     if constexpr (Cfg::CORE16) {
@@ -287,26 +285,26 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
     ProfScope prof(PC_FWD_MERGE, st);
     f32x4_t* out = reinterpret_cast<f32x4_t*>(shard_out);
     if (S >= 64)
-      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S,
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S,
                          T, p.c, 1.0f / temperature, out);
     else if (S >= 8)
-      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S, T,
                          p.c, 1.0f / temperature, out);
     else
-      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+      hipLaunchKernelGGL(lce_fwd_shard_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S, T,
                          p.c, 1.0f / temperature, out);
     return check_launch("lce_fwd_shard_merge_kernel");
   }
   {
     ProfScope prof(PC_FWD_MERGE, st);
     if (S >= 64)
-      hipLaunchKernelGGL(lce_fwd_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<64>, dim3((unsigned)((T * 64 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S, T,
                          p.c, 1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
     else if (S >= 8)
-      hipLaunchKernelGGL(lce_fwd_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T,
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<8>, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S, T,
                          p.c, 1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
     else
-      hipLaunchKernelGGL(lce_fwd_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, S, T, p.c,
+      hipLaunchKernelGGL(lce_fwd_merge_kernel<1>, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, p.parts, p.xlabel, labels, label_offset, V, S, T, p.c,
                          1.0f / temperature, lp_tok, entropy, maximum, accumulate, entropy_b);
     rc = check_launch("lce_fwd_merge_kernel");
   }
@@ -539,16 +537,6 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   int* rows = compact ? reinterpret_cast<int*>(ws + L.off_rows) : nullptr;
   int* inv = compact ? reinterpret_cast<int*>(ws + L.off_inv) : nullptr;
   int* n_rows = compact ? reinterpret_cast<int*>(ws + L.off_nrows) : nullptr;
-  if (compact) {
-    ProfScope prof(PC_ACTIVE_ROWS, st);
-    int* acounts = reinterpret_cast<int*>(ws + L.off_acounts);
-    const unsigned nblk = (unsigned)((T + kActiveBlock - 1) / kActiveBlock);
-    const int64_t gstride = reduction == LCE_REDUCTION_NONE ? 1 : 0;
-    hipLaunchKernelGGL(active_count_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, gstride, dentropy, T, acounts);
-    if ((rc = check_launch("active_count_kernel"))) return rc;
-    hipLaunchKernelGGL(active_rows_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, gstride, dentropy, T, acounts, rows, inv, n_rows);
-    if ((rc = check_launch("active_rows_kernel"))) return rc;
-  }
   // tokens grouped by label for the one-hot part of d_weight (added after the GEMMs)
   LabelTerm lt;
   lt.labels = nullptr; lt.v0 = vocab_offset; lt.V = V; lt.g_lp = dlogprobs;
@@ -556,16 +544,40 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   lt.scale = (reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f) / temperature;
   uint32_t* skeys[2] = {reinterpret_cast<uint32_t*>(ws + L.off_keys[0]), reinterpret_cast<uint32_t*>(ws + L.off_keys[1])};
   int* svals[2] = {reinterpret_cast<int*>(ws + L.off_vals[0]), reinterpret_cast<int*>(ws + L.off_vals[1])};
-  if (L.sort_items) {
-    lt.labels = labels;
+  CoefArgs<TIN> ca;
+  ca.h = h; ca.ldh = ldh; ca.W = W; ca.ldw = ldw; ca.labels = labels; ca.v0 = vocab_offset; ca.V = V; ca.ntok = T; ca.H = H;
+  ca.maximum = maximum; ca.accumulate = accumulate; ca.entropy_b = entropy_b; ca.g_lp = dlogprobs; ca.g_stride = lt.g_stride;
+  ca.g_scale = reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f; ca.g_ent = dentropy; ca.rcp_tau = 1.0f / temperature;
+  ca.c = kLog2e / temperature;
+  const bool with_coef = sizeof(TIN) == 2 && L.sort_items && tu.label_outside == 2;
+  ca.coef = with_coef ? reinterpret_cast<float*>(ws + L.off_coef) : nullptr;
+  if (L.sort_items) lt.labels = labels;
+  if (with_coef) { lt.g_lp = ca.coef; lt.g_stride = 1; lt.scale = 1.0f; }
+  // few tokens: the token list, the label coefficients and the compact copy of hidden come from one launch, and the
+  // one-hot rows of d_weight need no sorted list (few_finish_kernel at the end)
+  const bool few_prep = L.few && compact;
+  if (few_prep) {
+    if constexpr (sizeof(TIN) == 2) {
+      ProfScope prof(PC_ACTIVE_ROWS, st);
+      const int64_t r64 = round_up(T, 64);
+      hipLaunchKernelGGL(few_prep_kernel<TIN>, dim3((unsigned)(r64 < L.tpad ? r64 : L.tpad)), dim3(256), 0, st, ca, Ht, L.ldHt, L.tpad, rows,
+                         inv, n_rows);
+      if ((rc = check_launch("few_prep_kernel"))) return rc;
+    }
+  } else if (compact) {
+    ProfScope prof(PC_ACTIVE_ROWS, st);
+    int* acounts = reinterpret_cast<int*>(ws + L.off_acounts);
+    const unsigned nblk = (unsigned)((T + kActiveBlock - 1) / kActiveBlock);
+    hipLaunchKernelGGL(active_count_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, ca.g_stride, dentropy, T, acounts);
+    if ((rc = check_launch("active_count_kernel"))) return rc;
+    hipLaunchKernelGGL(active_rows_kernel, dim3(nblk), dim3(256), 0, st, dlogprobs, ca.g_stride, dentropy, T, acounts, rows, inv, n_rows);
+    if ((rc = check_launch("active_rows_kernel"))) return rc;
+  }
+  if (L.sort_items && !few_prep) {
     ProfScope prof(PC_LABEL_ROWS, st);
-    if constexpr (sizeof(TIN) == 2) if (tu.label_outside == 2) {
-      float* coef = reinterpret_cast<float*>(ws + L.off_coef);
-      hipLaunchKernelGGL(label_coef_kernel<TIN>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, h, ldh, W, ldw, labels, vocab_offset, V, T,
-                         H, maximum, accumulate, entropy_b, dlogprobs, lt.g_stride, reduction == LCE_REDUCTION_MEAN ? 1.0f / (float)T : 1.0f,
-                         dentropy, 1.0f / temperature, kLog2e / temperature, coef);
+    if constexpr (sizeof(TIN) == 2) if (with_coef) {
+      hipLaunchKernelGGL(label_coef_kernel<TIN>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st, ca);
       if ((rc = check_launch("label_coef_kernel"))) return rc;
-      lt.g_lp = coef; lt.g_stride = 1; lt.scale = 1.0f;
     }
     const int nblocks = L.sort_items / kSortBlock;
     if (!need_dw) {
@@ -601,7 +613,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
   }
   // second operand of the d_weight GEMM (W^T for d_hidden follows chunk by chunk): the listed rows of hidden,
   // as they are (K-major, for the transposing reads), or transposed to h^T [H][T]
-  if (L.tn) {
+  if (few_prep) {
+    // (few_prep_kernel has written the compact copy)
+  } else if (L.tn) {
     ProfScope prof(PC_TRANSPOSE, st);
     hipLaunchKernelGGL(gather_rows_kernel<TIN>, dim3(2048), dim3(256), 0, st, h, ldh, T, H, Ht, L.ldHt, L.tpad, rows, n_rows);
     if ((rc = check_launch("gather_rows_kernel"))) return rc;
@@ -762,6 +776,25 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
     }
     launch_chunk(p);
     if ((rc = check_launch("lce_bwd_chunk_kernel"))) return rc;
+  }
+  if (few_prep) {
+    // d_hidden and the one-hot rows of d_weight (every row holds its softmax terms by now), one launch
+    if constexpr (sizeof(TIN) == 2) {
+      ProfScope prof(PC_DH_FINISH, st);
+      const int n_dh = need_dh ? (int)((T * (H / 4) + 255) / 256) : 0;
+      const int n_lr = (L.sort_items && need_dw) ? (int)T : 0;
+      const int64_t part_stride = (int64_t)(align256((size_t)T * H * 4) / 4);
+      if (n_dh + n_lr > 0) {
+        if (grads_f32)
+          hipLaunchKernelGGL((few_finish_kernel<TIN, float>), dim3((unsigned)(n_dh + n_lr)), dim3(256), 0, st, dHacc, L.ksplit, part_stride, inv,
+                             T, H, static_cast<float*>(d_hidden), lt, W, ldw, n_dh, rows, n_rows, h, ldh, static_cast<float*>(d_weight));
+        else
+          hipLaunchKernelGGL((few_finish_kernel<TIN, TIN>), dim3((unsigned)(n_dh + n_lr)), dim3(256), 0, st, dHacc, L.ksplit, part_stride, inv,
+                             T, H, static_cast<TIN*>(d_hidden), lt, W, ldw, n_dh, rows, n_rows, h, ldh, static_cast<TIN*>(d_weight));
+        if ((rc = check_launch("few_finish_kernel"))) return rc;
+      }
+    }
+    return LCE_OK;
   }
   if (need_dh) {
     // d_hidden = ordered sum of the fp32 partials, rounded once; zero rows for tokens without gradient

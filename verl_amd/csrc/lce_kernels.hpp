@@ -42,7 +42,8 @@ struct FwdArgs {
   int64_t T, V, H;
   float c;           // log2(e) / temperature
   f32x4_t* parts;    // [S][T] of (m, a, b, unused)
-  float* xlabel;     // [T] raw accumulator value at the label (pre-zeroed; written by the one lane that owns it)
+  float* xlabel;     // [T] raw accumulator value at the label: written by the one lane that owns it, left as it was for a
+                     // token whose label is not a row of W (the merge kernels do not read it then)
   int S;             // vocabulary splits
   // Split s owns the tiles that start at rows s * split_stride + i * tile_step (i = 0, 1, ...) below its end row
   // min(V, s * split_stride + split_span).  Two layouts: tiles dealt round robin (split_stride = BM, tile_step =
@@ -186,12 +187,20 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
   }
 }
 
+// raw logit at the label of token t: what the forward tiles left in xlabel[t], or 0 when the label is not one of the V
+// rows of W that start at vocabulary id label_offset (no lane owns such a token, and xlabel[t] holds whatever the
+// workspace held before the call)
+LCE_DEV float label_logit(const float* xlabel, const int64_t* labels, int64_t label_offset, int64_t V, int64_t t) {
+  const int64_t y = labels[t] - label_offset;
+  return (y >= 0 && y < V) ? xlabel[t] : 0.f;
+}
+
 // merge the S partials of every token and emit the five per-token outputs; LANES (a power of two up
 // to 64) threads share a token: each merges every LANES-th partial, then a fixed shuffle tree joins
 // them (with few tokens there are hundreds of splits per token and only a handful of tokens)
 template <int LANES>
-__global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, int S, int64_t T, float c, float rcp_tau,
-                                     float* logprobs, float* entropy, float* maximum, float* accumulate,
+__global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, const int64_t* labels, int64_t label_offset, int64_t V,
+                                     int S, int64_t T, float c, float rcp_tau, float* logprobs, float* entropy, float* maximum, float* accumulate,
                                      float* entropy_b) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t t = gid / LANES;
@@ -210,7 +219,7 @@ __global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, 
     merge_stats(vm, va, vb, m2, a2, b2, c);
   }
   if (!live || sub != 0) return;
-  const float vz = xlabel[t];
+  const float vz = label_logit(xlabel, labels, label_offset, V, t);
   const float mz = vm * rcp_tau;
   const float lse = mz + logf(va);
   const float eb = (vb / va) * rcp_tau;
@@ -225,8 +234,8 @@ __global__ void lce_fwd_merge_kernel(const f32x4_t* parts, const float* xlabel, 
 // between the owners of the vocabulary shards: out[t] = (max logit, sum exp(logit - max),
 // sum logit * exp(logit - max), label logit or 0), in logit units (after the division by temperature).
 template <int LANES>
-__global__ void lce_fwd_shard_merge_kernel(const f32x4_t* parts, const float* xlabel, int S, int64_t T, float c, float rcp_tau,
-                                           f32x4_t* out) {
+__global__ void lce_fwd_shard_merge_kernel(const f32x4_t* parts, const float* xlabel, const int64_t* labels, int64_t label_offset,
+                                           int64_t V, int S, int64_t T, float c, float rcp_tau, f32x4_t* out) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t t = gid / LANES;
   const int sub = (int)(gid % LANES);
@@ -244,7 +253,7 @@ __global__ void lce_fwd_shard_merge_kernel(const f32x4_t* parts, const float* xl
     merge_stats(vm, va, vb, m2, a2, b2, c);
   }
   if (!live || sub != 0) return;
-  const f32x4_t v = {vm * rcp_tau, va, vb * rcp_tau, xlabel[t] * rcp_tau};
+  const f32x4_t v = {vm * rcp_tau, va, vb * rcp_tau, label_logit(xlabel, labels, label_offset, V, t) * rcp_tau};
   out[t] = v;
 }
 
@@ -534,9 +543,12 @@ LCE_DEV void ds_tile(const DsArgs<typename Cfg::TIN>& p, int bid, char* lds) {
     const int64_t pad_end = (p.vrows + Cfg::WM - 1) / Cfg::WM * Cfg::WM;  // (rows up to the wave tile are written as zeros)
     const int64_t r0 = (int64_t)bid * p.range_rows;
     const int64_t r1 = r0 + p.range_rows < pad_end ? r0 + p.range_rows : pad_end;
-    for (int64_t m0 = r0; m0 < r1; m0 += Cfg::BM) {
-      if (m0 > r0) __syncthreads();  // the staging tiles of the previous tile's epilogue are read out
-      ds_tile_at<Cfg>(p, 0, m0, r1, Tc, lds);
+    // Walked from the range's end: the forward, which ran last, walked the same ranges from their start, so what the
+    // memory-side cache still holds of W is read first (64 tokens, H=3584, V=152064: 8 us of 207)
+    const int64_t ntile = (r1 - r0 + Cfg::BM - 1) / Cfg::BM;
+    for (int64_t i = ntile - 1; i >= 0; --i) {
+      if (i < ntile - 1) __syncthreads();  // the staging tiles of the previous tile's epilogue are read out
+      ds_tile_at<Cfg>(p, 0, r0 + i * Cfg::BM, r1, Tc, lds);
     }
     return;
   }
@@ -848,11 +860,12 @@ struct LabelTerm {
 // without `inv`), or zeros where inv[t] < 0 (token without upstream gradient).  The sum runs in the
 // fixed order s = 0, 1, ..., so the result does not depend on scheduling.  H a multiple of 4.
 // With a label term, G_t * W[label_t][:] is added in fp32 before the one rounding.
+// (bid of nblocks workgroups: the kernel's own grid, or the part of a larger grid that does this work)
 template <typename T, typename TOUT>
-__global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, TOUT* out,
-                                 LabelTerm lt, const T* W, int64_t ldw) {
+LCE_DEV void dh_finish_body(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, TOUT* out,
+                            const LabelTerm& lt, const T* W, int64_t ldw, int64_t bid, int64_t nblocks) {
   const int64_t per_row = H / 4, n = ntok * per_row;
-  for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n; q += (int64_t)gridDim.x * blockDim.x) {
+  for (int64_t q = bid * blockDim.x + threadIdx.x; q < n; q += nblocks * blockDim.x) {
     const int64_t t = q / per_row, c = (q - t * per_row) * 4;
     const int64_t pos = inv ? (int64_t)inv[t] : t;
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -876,6 +889,12 @@ __global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const
     TOUT* dst = out + t * H + c;
     dst[0] = (TOUT)a.x; dst[1] = (TOUT)a.y; dst[2] = (TOUT)a.z; dst[3] = (TOUT)a.w;
   }
+}
+
+template <typename T, typename TOUT>
+__global__ void dh_finish_kernel(const float* part, int S, int64_t stride, const int* inv, int64_t ntok, int64_t H, TOUT* out,
+                                 LabelTerm lt, const T* W, int64_t ldw) {
+  dh_finish_body<T, TOUT>(part, S, stride, inv, ntok, H, out, lt, W, ldw, (int64_t)blockIdx.x, (int64_t)gridDim.x);
 }
 
 // Tokens whose upstream gradients are both zero add nothing to either gradient.  The others are listed in order:
