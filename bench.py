@@ -455,7 +455,8 @@ def run_token_sweep(args):
             torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
         rec = {"T": T}
-        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 4.0, 6.0 * T * V * H)):
+        # (streaming passes over [V, H]: up to 128 tokens the backward takes the logits the forward kept instead of a pass over W)
+        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 128 else 4.0, 6.0 * T * V * H)):
             ms = timed(fn)
             hbm_ms = passes * V * H * 2.0 / PEAK_HBM * 1e3
             mfma_ms = flops / PEAK_BF16 * 1e3
@@ -714,16 +715,19 @@ def main():
     # (the mandated recompute of the logits is executed but not counted).  With Ta = T this is the reference's 6*T*V*H.
     algorithmic = (2.0 * T + 2.0 * n_grads * t_active) * V * H / (elapsed / args.steps)
     if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM and "lce_bwd_chunk_kernel" in kernels:
-        # few tokens: the step is four streaming passes over [V, H] in the input dtype (W read by the forward, by the
-        # d_logits tiles and by the d_hidden GEMM; d_weight written), and HBM bounds it.  The backward's two launches
-        # (d_logits tiles; both gradient GEMMs) account for three of the four.
+        # few tokens: HBM bounds the step.  Its streaming passes over [V, H] in the input dtype: W read by the forward and
+        # by the d_hidden product, d_weight written; with up to 128 tokens the forward keeps the fp32 logits (T*V*4 bytes
+        # written, then read by the backward) and no pass recomputes them; beyond that the d_logits tiles read W once more.
         k = kernels["lce_bwd_chunk_kernel"]
-        nbytes = (1.0 + n_grads) * V * H * 2.0 / k["launches_per_step"]  # (W read twice, d_weight written; --frozen-head: W read twice)
+        kept = T <= 128
+        passes_bwd = n_grads if kept else 1.0 + n_grads
+        nbytes = passes_bwd * V * H * 2.0 / k["launches_per_step"]  # (W read for d_hidden, d_weight written; --frozen-head: W read)
+        step_bytes = (1.0 + passes_bwd) * V * H * 2.0 + (2.0 * T * V * 4.0 if kept else 0.0)
         roofline = {"bound": "hbm", "kernel": "lce_bwd_chunk_kernel", "achieved": nbytes / (k["avg_ms"] * 1e-3) / 1e9,
                     "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": nbytes / (k["avg_ms"] * 1e-3) / PEAK_HBM,
                     "traffic": measured_traffic(workload_name, "lce_bwd_chunk_kernel", state),
-                    "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes,
-                    "step_bytes": (2.0 + n_grads) * V * H * 2.0, "step_GBps": (2.0 + n_grads) * V * H * 2.0 / (elapsed / args.steps) / 1e9}
+                    "avg_launch_ms": k["avg_ms"], "bytes_per_launch": nbytes, "logits_kept": kept,
+                    "step_bytes": step_bytes, "step_GBps": step_bytes / (elapsed / args.steps) / 1e9}
     out = {
         "metric": "fwd+bwd tokens/s, 7B lm-head logprob+entropy; % of bf16 MFMA peak",
         "value": tokens_per_s,

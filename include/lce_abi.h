@@ -19,7 +19,7 @@
 extern "C" {
 #endif
 
-#define LCE_ABI_VERSION 9
+#define LCE_ABI_VERSION 10
 
 enum { LCE_DTYPE_BF16 = 0, LCE_DTYPE_F32 = 1, LCE_DTYPE_F16 = 2 };
 enum { LCE_REDUCTION_NONE = 0, LCE_REDUCTION_SUM = 1, LCE_REDUCTION_MEAN = 2 }; /* verl/utils/kernel/kernels.py:102-126 */
@@ -92,6 +92,30 @@ int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_
                      int64_t V, int dtype, float temperature, int reduction, const float* maximum, const float* accumulate,
                      const float* entropy_b, const float* dlogprobs, const float* dentropy, float* d_hidden, float* d_weight,
                      void* workspace, size_t workspace_bytes, int64_t vchunk, void* stream);
+
+/* Few tokens: the pair above with the logits kept between the two calls, the way autograd keeps any activation.  The
+ * reference's backward recomputes the logits from hidden and weight (verl/utils/kernel/kernels.py:1380-1515), which is
+ * what keeps [T, V] out of memory when T is large, and what lce_backward does; with at most 128 tokens the backward is
+ * bound by its passes over [V, H] (one for the logits, one for d_hidden, one written for d_weight) and [T, V] in fp32 is
+ * a fraction of one of them, so keeping it saves the first pass (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not read).
+ *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when the library keeps nothing for it (more than 128
+ *     tokens, fp32 inputs, diagnostic settings that replace the few-token kernels): then pass NULL below.
+ *   lce_forward_keep_logits: lce_forward; with logits_cache != NULL it also writes hidden . weight^T there in fp32
+ *     (private layout).  Same outputs, bit for bit.
+ *   lce_backward_from_logits: lce_backward (grads_fp32 = 0) or lce_backward_f32 (grads_fp32 = 1; d_hidden, d_weight are
+ *     float* then); with logits_cache != NULL, as written by lce_forward_keep_logits for the same hidden, weight, T, H, V
+ *     and dtype, the gradient of the logits is computed from it with the same expressions, so both gradients are bit for
+ *     bit those of lce_backward.  The cache is only read. */
+size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype);
+int lce_forward_keep_logits(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                            int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                            float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                            void* logits_cache, size_t logits_cache_bytes, void* stream);
+int lce_backward_from_logits(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                             int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                             const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                             void* d_hidden, void* d_weight, int grads_fp32, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                             const void* logits_cache, size_t logits_cache_bytes, void* stream);
 
 /* Vocabulary-parallel building blocks: what one rank of a tensor-parallel lm-head runs on its shard
  * W[vocab_offset : vocab_offset + V_local, :] of the vocabulary.  The exchange between the ranks (an

@@ -107,9 +107,10 @@ def test_signature_matches_reference():
         "dlogprobs", "dentropy", "hidden", "weight", "labels", "maximum", "acc", "entropy_b", "reduction",
         "should_return_fp32_grad", "temperature", "dist_process_group",
     ]  # fmt: skip
-    # beyond the reference's: two keyword-only switches that default to the reference's behaviour (both gradients)
+    # beyond the reference's: keyword-only arguments that default to the reference's behaviour (both gradients, the
+    # logits recomputed)
     extras = {n: p.default for n, p in bsig.parameters.items() if p.kind is inspect.Parameter.KEYWORD_ONLY}
-    assert extras == {"need_d_hidden": True, "need_d_weight": True}
+    assert extras == {"need_d_hidden": True, "need_d_weight": True, "logits_cache": None}
     assert kernels.get_entropy_reduction_enum_number("none") == 0
     assert kernels.get_entropy_reduction_enum_number("sum") == 1
     assert kernels.get_entropy_reduction_enum_number("mean") == 2

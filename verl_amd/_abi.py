@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("LCE_LIBRARY_PATH") or os.path.join(_HERE, "lib", "liblce_gfx950.so")
 
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 # every symbol include/lce_abi.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -29,6 +29,15 @@ SYMBOLS = {
     "lce_backward_f32": (
         _i,
         [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _p],
+    ),
+    "lce_logits_cache_bytes": (_sz, [_i64, _i64, _i64, _i]),
+    "lce_forward_keep_logits": (
+        _i,
+        [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _sz, _p, _sz, _p],
+    ),
+    "lce_backward_from_logits": (
+        _i,
+        [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _p, _i, _p, _sz, _i64, _p, _sz, _p],
     ),
     "lce_forward_shard": (_i, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i, _f, _p, _p, _sz, _p]),
     "lce_merge_shards": (_i, [_p, _i, _i64, _i, _p, _p, _p, _p, _p, _p, _sz, _p]),

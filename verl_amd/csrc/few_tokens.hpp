@@ -17,6 +17,7 @@
 // ds_read_b64_tr_b16.  Everything is plain HIP with compiler-placed waits.
 #pragma once
 #include "gemm_core.hpp"
+#include "lce_kernels.hpp"
 
 namespace lce {
 
@@ -361,6 +362,49 @@ __global__ __launch_bounds__(256, 2) void lce_bwd_few_kernel(FewArgs<TIN> p) {
   const int bid = blockIdx.x;
   if (bid < p.n_dw) dw_few_tile<TIN, TOUT, Perm, KT, S::HW_DW>(p, bid, lds);
   else dh_few_tile<TIN, Perm, S::NT, S::HW>(p, bid - p.n_dw, lds);
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// d_logits of a vocabulary chunk from logits that the forward kept (few tokens): what the d_logits tiles compute from
+// their accumulators, here from x[t * ldx + v], element by element with the same expressions, so the same bits.  One
+// pass over 4 bytes per logit instead of a pass over W.  Workgroup b owns the 64 columns [64 b, 64 b + 64) of dS, i.e.
+// one group of the vocabulary order Perm, and the first `nrows` compact token positions (64 or 128): rows beyond the
+// tokens that take part and columns beyond the chunk's rows are written as zeros, as the tiles write them.  Eight
+// lanes share a position: they read the 256 bytes of its token's logits of the group and write 128 bytes of dS.
+// p: the chunk's DsArgs (W, h, the tile map and the range are not used); x: the kept logit of the chunk's first row
+// for token 0.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename TIN, typename Perm>
+__global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, const float* x, int64_t ldx, int nrows) {
+  static_assert(sizeof(TIN) == 2 && Perm::GV == 64, "16-bit d_logits in groups of 64 vocabulary rows");
+  const int tid = threadIdx.x, c = tid & 7;
+  const int64_t u0 = (int64_t)blockIdx.x * 64;
+  const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;
+  for (int pos = tid >> 3; pos < nrows; pos += 32) {
+    float lse2 = 0.f, C0 = 0.f, C1 = 0.f, G = 0.f;
+    int64_t tok = -1;
+    int rel = -1;
+    if (pos < Tc) {
+      tok = p.rows ? (int64_t)p.rows[pos] : pos;
+      const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
+      const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
+      lse2 = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
+      G = glp * p.rcp_tau;
+      C1 = -gent * p.rcp_tau * p.rcp_tau;
+      C0 = -G + gent * p.entropy_b[tok] * p.rcp_tau;
+      const int64_t y = p.labels[tok] - p.v0;
+      rel = (p.label_outside != 1 && y >= u0 && y < u0 + 64) ? (int)(y - u0) : -1;
+    }
+    float d[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int row = (int)(Perm::vocab_at(u0 + c * 8 + e) - u0);  // the vocabulary row behind column c * 8 + e of the group
+      const bool dead = tok < 0 || u0 + row >= p.vrows;
+      const float xv = dead ? 0.f : x[tok * ldx + u0 + row];
+      d[e] = dlogit<true>(xv, p.c, lse2, C0, C1, G, row == rel, dead, p.label_outside == 2);
+    }
+    store_run<TIN, 8>(p.dS + (int64_t)pos * p.ldS + u0 + c * 8, d);
+  }
 }
 
 }  // namespace lce

@@ -173,7 +173,7 @@ size_t lce_forward_workspace_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
 static int forward_entry(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
                          int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
                          float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
-                         void* stream, int64_t label_offset, float* shard_out, int max_splits = kMaxSplits) {
+                         void* stream, int64_t label_offset, float* shard_out, int max_splits = kMaxSplits, float* xcache = nullptr) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -199,8 +199,31 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
     else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 1;
   }
+  if (xcache && sel != kSelT64 && sel != kSelT128) return fail(LCE_E_ARG, "forward: tile selector %d cannot keep the logits", sel);
   return kForward[dtype](sel, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum,
-                         accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits);
+                         accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits, xcache);
+}
+
+size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
+  (void)H;
+  if (!known_dtype(dtype) || V <= 0 || !logits_cache_applies(T, esize(dtype))) return 0;
+  const Tuning tu = tuning_snapshot();
+  if (tu.variant_forced || !tu.few_token_gemms) return 0;  // (diagnostic settings that take the few-token kernels out)
+  return (size_t)T * (size_t)logits_cache_row(V) * 4;
+}
+
+int lce_forward_keep_logits(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                            int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
+                            float* maximum, float* accumulate, float* entropy_b, void* workspace, size_t workspace_bytes,
+                            void* logits_cache, size_t logits_cache_bytes, void* stream) {
+  if (logits_cache) {
+    const size_t need = known_dtype(dtype) ? lce_logits_cache_bytes(T, H, V, dtype) : 0;
+    if (need == 0) return fail(LCE_E_ARG, "lce_forward_keep_logits: no logits are kept for this shape (lce_logits_cache_bytes is 0): pass NULL");
+    if (logits_cache_bytes < need) return fail(LCE_E_WORKSPACE, "logits cache too small: %zu < %zu", logits_cache_bytes, need);
+    if (reinterpret_cast<size_t>(logits_cache) % 16 != 0) return fail(LCE_E_ARG, "logits cache must be 16-byte aligned");
+  }
+  return forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
+                       accumulate, entropy_b, workspace, workspace_bytes, stream, 0, nullptr, kMaxSplits, static_cast<float*>(logits_cache));
 }
 
 int lce_forward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
@@ -238,8 +261,7 @@ int lce_forward_static(const void* hidden, int64_t ldh, const void* weight, int6
   if (!capturing && use->recorded && use->last_stream != st && hipEventQuery(use->done) == hipErrorNotReady)
     return fail(LCE_E_BUSY, "lce_forward_static: the previous call on this GPU, on another stream, is still running and owns the "
                             "built-in scratch buffer; order the two streams, or use lce_forward with a workspace of your own");
-  // (what must start at zero, the label logits, is cleared by a fill kernel inside the forward: nothing of the previous
-  // call's contents is read)
+  // (nothing in the buffer has to start at zero, and nothing of the previous call's contents is read)
   rc = forward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, logprobs, entropy, maximum,
                      accumulate, entropy_b, use->ptr, (size_t)LCE_STATIC_SCRATCH_BYTES, stream, 0, nullptr, max_splits);
   if (rc == LCE_OK && !capturing && T > 0) {
@@ -299,7 +321,7 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
                           int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
                           const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                           void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes, int64_t vchunk,
-                          void* stream, int64_t vocab_offset, bool grads_f32 = false) {
+                          void* stream, int64_t vocab_offset, bool grads_f32 = false, const float* xcache = nullptr) {
   int rc = check_common(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction);
   if (rc) return rc;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -320,7 +342,23 @@ static int backward_entry(const void* hidden, int64_t ldh, const void* weight, i
   char* ws = reinterpret_cast<char*>(align256(reinterpret_cast<size_t>(workspace)));
   return kBackward[dtype](bwd_variant(tu, T, esz), hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, maximum,
                           accumulate, entropy_b, dlogprobs, dentropy, d_hidden, d_weight, grads_f32, ws, vchunk, st, vocab_offset,
-                          tu);
+                          tu, xcache);
+}
+
+int lce_backward_from_logits(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
+                             int64_t H, int64_t V, int dtype, float temperature, int reduction, const float* maximum,
+                             const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
+                             void* d_hidden, void* d_weight, int grads_fp32, void* workspace, size_t workspace_bytes, int64_t vchunk,
+                             const void* logits_cache, size_t logits_cache_bytes, void* stream) {
+  if (logits_cache) {
+    const size_t need = known_dtype(dtype) ? lce_logits_cache_bytes(T, H, V, dtype) : 0;
+    if (need == 0) return fail(LCE_E_ARG, "lce_backward_from_logits: no logits are kept for this shape (lce_logits_cache_bytes is 0): pass NULL");
+    if (logits_cache_bytes < need) return fail(LCE_E_WORKSPACE, "logits cache too small: %zu < %zu", logits_cache_bytes, need);
+    if (reinterpret_cast<size_t>(logits_cache) % 16 != 0) return fail(LCE_E_ARG, "logits cache must be 16-byte aligned");
+  }
+  return backward_entry(hidden, ldh, weight, ldw, labels, T, H, V, dtype, temperature, reduction, maximum, accumulate, entropy_b,
+                        dlogprobs, dentropy, d_hidden, d_weight, workspace, workspace_bytes, vchunk, stream, 0, grads_fp32 != 0,
+                        static_cast<const float*>(logits_cache));
 }
 
 int lce_backward(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,

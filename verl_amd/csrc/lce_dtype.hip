@@ -28,7 +28,7 @@ namespace lce_shared {
 int TU_FN(forward)(int sel, LCE_FWD_PARAMS) {
 #define LCE_RUN(Vt)                                                                                                          \
   return forward_impl<typename Vt<TuT>::Cfg>((const TuT*)h, ldh, (const TuT*)W, ldw, labels, T, H, V, temperature, reduction, \
-                                             lp, ent, mx, ac, eb, ws, st, label_offset, shard_out, max_splits)
+                                             lp, ent, mx, ac, eb, ws, st, label_offset, shard_out, max_splits, xcache)
   switch (sel) {
     case 0: LCE_RUN(Variant0);
     case 1: LCE_RUN(Variant1);
@@ -59,7 +59,7 @@ int TU_FN(gemm_nt)(int sel, LCE_GEMM_PARAMS) {
 int TU_FN(backward)(int sel, LCE_BWD_PARAMS) {
 #define LCE_RUN(Vt)                                                                                                           \
   return backward_impl<typename Vt<TuT>::Cfg>((const TuT*)h, ldh, (const TuT*)W, ldw, labels, T, H, V, temperature, reduction, \
-                                              mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st, vocab_offset, tu)
+                                              mx, ac, eb, glp, gent, dh, dw, grads_f32, ws, vchunk, st, vocab_offset, tu, xcache)
   // (bwd_variant() hands over one of the two mainloops the backward is built on)
   switch (sel) {
     case kDefaultVariantBwd: LCE_RUN(Variant1);

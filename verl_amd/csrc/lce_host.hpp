@@ -56,12 +56,12 @@ enum { kSelT64 = 4, kSelT128 = 5 };
 #define LCE_FWD_PARAMS                                                                                                      \
   const void *h, int64_t ldh, const void *W, int64_t ldw, const int64_t *labels, int64_t T, int64_t H, int64_t V,          \
       float temperature, int reduction, float *lp, float *ent, float *mx, float *ac, float *eb, char *ws, hipStream_t st,   \
-      int64_t label_offset, float *shard_out, int max_splits
+      int64_t label_offset, float *shard_out, int max_splits, float *xcache
 #define LCE_BWD_PARAMS                                                                                                      \
   const void *h, int64_t ldh, const void *W, int64_t ldw, const int64_t *labels, int64_t T, int64_t H, int64_t V,          \
       float temperature, int reduction, const float *mx, const float *ac, const float *eb, const float *glp,               \
       const float *gent, void *dh, void *dw, bool grads_f32, char *ws, int64_t vchunk, hipStream_t st,                     \
-      int64_t vocab_offset, const Tuning &tu
+      int64_t vocab_offset, const Tuning &tu, const float *xcache
 #define LCE_GEMM_PARAMS                                                                                                     \
   const void *A, int64_t lda, const void *B, int64_t ldb, float *C, int64_t ldc, int64_t M, int64_t N, int64_t K,          \
       hipStream_t st
@@ -229,11 +229,16 @@ int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
   return best;
 }
 
+// Kept logits (few tokens): fp32 [T][logits_cache_row(V)], element [t][v] = hidden[t] . W[v].  A backward that is
+// given them computes d_logits from 4 bytes per logit instead of from a pass over W.
+int64_t logits_cache_row(int64_t V) { return round_up(V, 64); }
+bool logits_cache_applies(int64_t T, size_t esz) { return esz == 2 && T >= 1 && T <= 128; }
+
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
                  int64_t T, int64_t H, int64_t V, float temperature, int reduction, float* logprobs, float* entropy,
                  float* maximum, float* accumulate, float* entropy_b, char* ws, hipStream_t st, int64_t label_offset = 0,
-                 float* shard_out = nullptr, int max_splits = kMaxSplits) {
+                 float* shard_out = nullptr, int max_splits = kMaxSplits, float* xcache = nullptr) {
   // shard_out: W is one shard of a larger vocabulary starting at row label_offset; instead of the five
   // outputs the per-token partial (max, sum exp, sum logit*exp, label logit) goes to shard_out [T][4]
   typedef typename Cfg::TIN TIN;
@@ -266,6 +271,9 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.tile_step = rows_per_split ? Cfg::BM : (int64_t)S * Cfg::BM;
   p.split_span = rows_per_split ? rows_per_split : V;
   p.label_offset = label_offset;
+  // xcache: the raw logits are kept for the backward (token tiles of at most 128 only; see logits_cache_row)
+  if (xcache && Cfg::BN > 128) return fail(LCE_E_ARG, "forward: this tile variant cannot keep the logits");
+  p.xcache = xcache; p.ldx = logits_cache_row(V);
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
   int rc;
@@ -516,7 +524,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
                   int64_t T, int64_t H, int64_t V, float temperature, int reduction, const float* maximum,
                   const float* accumulate, const float* entropy_b, const float* dlogprobs, const float* dentropy,
                   void* d_hidden, void* d_weight, bool grads_f32, char* ws, int64_t vchunk, hipStream_t st,
-                  int64_t vocab_offset, const Tuning& tu) {
+                  int64_t vocab_offset, const Tuning& tu, const float* xcache = nullptr) {
   // vocab_offset: W is the shard [vocab_offset, vocab_offset + V) of a larger vocabulary (labels are global ids)
   // d_hidden or d_weight may be null (not both): that gradient is not wanted (a frozen lm-head, an input without
   // gradient) and its GEMM, a third of the backward's work, is left out
@@ -763,6 +771,19 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         if ((rc = check_launch("lce_bwd_chunk_kernel(split)"))) return rc;
       }
       continue;
+    }
+    if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
+      if (p.n_gw + p.n_gh == 0 && xcache && L.few) {
+        // d_logits from the logits the forward kept: no pass over W
+        const int64_t ldx = logits_cache_row(V);
+        const int nrows = (int)(T <= 64 ? 64 : 128) < (int)L.tpad ? (int)(T <= 64 ? 64 : 128) : (int)L.tpad;
+        const int64_t c0 = p.ds.v0 - vocab_offset;  // the chunk's first row of W
+        ProfScope prof(PC_BWD_DS, st);
+        hipLaunchKernelGGL((ds_from_logits_kernel<TIN, KPerm<Cfg>>), dim3((unsigned)((p.ds.vrows + 63) / 64)), dim3(256),
+                           0, st, p.ds, xcache + c0, ldx, nrows);
+        if ((rc = check_launch("ds_from_logits_kernel"))) return rc;
+        continue;
+      }
     }
     ProfScope prof(PC_BWD_CHUNK, st);
     if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {

@@ -128,6 +128,15 @@ def efficient_entropy_forward(
     dist_process_group=None,
 ) -> list[torch.Tensor]:
     """Returns (logprobs, entropy, maximum, accumulate, entropy_b), all fp32."""
+    return forward_keeping_logits(hidden, weight, labels, reduction, temperature, dist_process_group, keep_logits=False)[:5]
+
+
+def forward_keeping_logits(hidden, weight, labels, reduction=2, temperature=1.0, dist_process_group=None, *, keep_logits=True):
+    """``efficient_entropy_forward`` plus a sixth value: the kept logits for ``efficient_entropy_backward(...,
+    logits_cache=)``, or ``None`` where the library keeps none (more than 128 tokens, fp32 inputs, ``keep_logits=False``).
+    With few tokens the backward is bound by its passes over ``[V, H]`` and fp32 ``[T, V]`` is a small fraction of one
+    of them, so the autograd node keeps it like any activation and the backward skips the pass that recomputes it (not
+    in the reference, which always recomputes)."""
     _require_single_rank(dist_process_group)
     code = _check_inputs(hidden, weight, labels)
     reduction = get_entropy_reduction_enum(reduction)
@@ -144,18 +153,23 @@ def efficient_entropy_forward(
     if T == 0:
         if reduction != 0:
             logprobs.zero_()
-        return logprobs, entropy, maximum, accumulate, entropy_b
+        return logprobs, entropy, maximum, accumulate, entropy_b, None
     lib = _abi.load()
+    cache = None
     with torch.cuda.device(dev):
         ws_bytes = lib.lce_forward_workspace_bytes(T, H, V, code)
         ws = torch.empty((ws_bytes,), device=dev, dtype=torch.uint8)
-        rc = lib.lce_forward(
+        cache_bytes = lib.lce_logits_cache_bytes(T, H, V, code) if keep_logits else 0
+        if cache_bytes:
+            cache = torch.empty((cache_bytes,), device=dev, dtype=torch.uint8)
+        rc = lib.lce_forward_keep_logits(
             hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V, code,
             float(temperature), reduction, logprobs.data_ptr(), entropy.data_ptr(), maximum.data_ptr(),
-            accumulate.data_ptr(), entropy_b.data_ptr(), ws.data_ptr(), ws_bytes, _abi.current_stream(dev),
+            accumulate.data_ptr(), entropy_b.data_ptr(), ws.data_ptr(), ws_bytes, _abi.ptr(cache), cache_bytes,
+            _abi.current_stream(dev),
         )  # fmt: skip
-        _abi.check(rc, "lce_forward")
-    return logprobs, entropy, maximum, accumulate, entropy_b
+        _abi.check(rc, "lce_forward_keep_logits")
+    return logprobs, entropy, maximum, accumulate, entropy_b, cache
 
 
 def efficient_entropy_backward(
@@ -174,12 +188,14 @@ def efficient_entropy_backward(
     *,
     need_d_hidden: bool = True,
     need_d_weight: bool = True,
+    logits_cache: typing.Optional[torch.Tensor] = None,
 ) -> list[torch.Tensor]:
     """Returns (d_hidden, d_weight) in ``hidden.dtype`` (fp32 when ``should_return_fp32_grad``).
 
     ``need_d_hidden`` / ``need_d_weight`` (not in the reference, which always computes both): ``False`` leaves that
     gradient's GEMM out, a third of the backward's work, and returns ``None`` in its place, e.g. for a frozen lm-head
-    under LoRA."""
+    under LoRA.  ``logits_cache``: the sixth value of ``forward_keeping_logits`` for the same inputs; the gradients are
+    bit for bit the same with and without it."""
     if not (need_d_hidden or need_d_weight):
         return None, None
     _require_single_rank(dist_process_group)
@@ -216,6 +232,17 @@ def efficient_entropy_backward(
             vchunk = _config._vocab_chunk
             ws_bytes = lib.lce_backward_workspace_bytes(T, H, V, code, vchunk)
             ws = torch.empty((ws_bytes,), device=dev, dtype=torch.uint8)
+            if logits_cache is not None:
+                assert logits_cache.is_cuda and logits_cache.device == dev and logits_cache.is_contiguous()
+                rc = lib.lce_backward_from_logits(
+                    hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,
+                    code, float(temperature), reduction, maximum.data_ptr(), acc.data_ptr(), entropy_b.data_ptr(),
+                    g_lp.data_ptr(), _abi.ptr(g_ent), _abi.ptr(d_hidden), _abi.ptr(d_weight), int(should_return_fp32_grad),
+                    ws.data_ptr(), ws_bytes, vchunk, logits_cache.data_ptr(), logits_cache.numel() * logits_cache.element_size(),
+                    _abi.current_stream(dev),
+                )  # fmt: skip
+                _abi.check(rc, "lce_backward_from_logits")
+                return d_hidden, d_weight
             entry = lib.lce_backward_f32 if should_return_fp32_grad else lib.lce_backward
             rc = entry(
                 hidden.data_ptr(), hidden.stride(0), weight.data_ptr(), weight.stride(0), labels.data_ptr(), T, H, V,

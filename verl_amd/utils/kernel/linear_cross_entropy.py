@@ -4,7 +4,9 @@ Call-compatible with the reference's ``verl/utils/kernel/linear_cross_entropy.py
 ``linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None)
 -> (logprobs, entropy)``; outputs are fp32 and flattened to ``[T]`` (``logprobs`` is 0-dim for
 ``"sum"`` / ``"mean"``), ``d_hidden`` comes back in ``hidden``'s shape, ``d_weight`` has ``hidden.dtype``, the four
-non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory.
+non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory, except with at most
+128 tokens, where the node keeps them in fp32 for its backward (a few per cent of the weight's size; it saves the
+backward one of its three passes over ``[V, H]``).
 
 The autograd node is a thin shell: everything it does besides argument checks and reshapes happens in the two host
 launchers of ``kernels.py`` (one C-ABI call each).
@@ -12,6 +14,7 @@ launchers of ``kernels.py`` (one C-ABI call each).
 
 from __future__ import annotations
 
+import threading
 import typing
 
 import torch
@@ -48,8 +51,13 @@ class LinearCrossEntropy(torch.autograd.Function):
         try:
             mode = kernels.get_entropy_reduction_enum_number(reduction.lower())
             rows, flat_labels = _as_token_rows(hidden, labels)
-            logprobs, entropy, *stats = kernels.efficient_entropy_forward(rows, weight, flat_labels, mode, temperature, dist_process_group)
-            ctx.save_for_backward(rows, weight, flat_labels, *stats)  # stats = (maximum, accumulate, entropy_b), fp32 [T]
+            # (no backward will follow, under no_grad or with inputs that take no gradient: nothing is kept beyond the outputs)
+            keep = getattr(_caller, "grad_enabled", True) and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+            logprobs, entropy, *stats, cache = kernels.forward_keeping_logits(
+                rows, weight, flat_labels, mode, temperature, dist_process_group, keep_logits=keep
+            )
+            # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with at most 128 tokens only (else None)
+            ctx.save_for_backward(rows, weight, flat_labels, *stats, cache)
             ctx.call = (hidden.shape, mode, temperature, dist_process_group)
             ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
         finally:
@@ -60,7 +68,7 @@ class LinearCrossEntropy(torch.autograd.Function):
     def backward(ctx, dlogprobs: typing.Optional[torch.Tensor], dentropy: typing.Optional[torch.Tensor]):
         torch.cuda.nvtx.range_push("LinearCrossEntropy-backward")  # the reference's range (:93)
         try:
-            rows, weight, flat_labels, maximum, accumulate, entropy_b = ctx.saved_tensors
+            rows, weight, flat_labels, maximum, accumulate, entropy_b, cache = ctx.saved_tensors
             shape, mode, temperature, group = ctx.call
             if dlogprobs is None:  # only the entropy was used downstream
                 dlogprobs = torch.zeros((rows.shape[0],) if mode == 0 else (), device=rows.device, dtype=torch.float32)
@@ -69,11 +77,29 @@ class LinearCrossEntropy(torch.autograd.Function):
             d_rows, d_weight = kernels.efficient_entropy_backward(
                 dlogprobs, dentropy, rows, weight, flat_labels, maximum, accumulate, entropy_b, mode,
                 False,  # should_return_fp32_grad: autograd wants the inputs' dtype
-                temperature, group, need_d_hidden=need_hidden, need_d_weight=need_weight,
+                temperature, group, need_d_hidden=need_hidden, need_d_weight=need_weight, logits_cache=cache,
             )  # fmt: skip
         finally:
             torch.cuda.nvtx.range_pop()
         return (d_rows.view(shape) if d_rows is not None else None), d_weight, None, None, None, None
 
 
-linear_cross_entropy = LinearCrossEntropy.apply
+# what torch.is_grad_enabled() said where linear_cross_entropy was called (inside Function.forward it is always off)
+_caller = threading.local()
+
+
+def linear_cross_entropy(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: typing.Optional[float] = 1.0,
+    reduction: typing.Optional[str] = "none",
+    dist_process_group=None,
+):
+    """``LinearCrossEntropy.apply`` with the reference's argument list (the reference binds the name to ``apply`` itself,
+    verl/utils/kernel/linear_cross_entropy.py:119)."""
+    _caller.grad_enabled = torch.is_grad_enabled()
+    try:
+        return LinearCrossEntropy.apply(hidden, weight, labels, temperature, reduction, dist_process_group)
+    finally:
+        _caller.grad_enabled = True
