@@ -395,13 +395,27 @@ __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, cons
       const int64_t y = p.labels[tok] - p.v0;
       rel = (p.label_outside != 1 && y >= u0 && y < u0 + 64) ? (int)(y - u0) : -1;
     }
+    // columns c * 8 + (0..3) and c * 8 + (4..7) of the group are two runs of four consecutive vocabulary rows (the order
+    // Perm keeps what one lane of a d_logits tile holds together: four consecutive rows per register quad), and the
+    // cache's rows are padded to whole groups, so each run is one aligned 16-byte load
+    float xv[8];
+    int row[8];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int r0 = (int)(Perm::vocab_at(u0 + c * 8 + 4 * hf) - u0);
+      f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+      if (tok >= 0) v = *reinterpret_cast<const f32x4_t*>(x + tok * ldx + u0 + r0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        row[4 * hf + e] = r0 + e;
+        xv[4 * hf + e] = v[e];
+      }
+    }
     float d[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int row = (int)(Perm::vocab_at(u0 + c * 8 + e) - u0);  // the vocabulary row behind column c * 8 + e of the group
-      const bool dead = tok < 0 || u0 + row >= p.vrows;
-      const float xv = dead ? 0.f : x[tok * ldx + u0 + row];
-      d[e] = dlogit<true>(xv, p.c, lse2, C0, C1, G, row == rel, dead, p.label_outside == 2);
+      const bool dead = tok < 0 || u0 + row[e] >= p.vrows;
+      d[e] = dlogit<true>(dead ? 0.f : xv[e], p.c, lse2, C0, C1, G, row[e] == rel, dead, p.label_outside == 2);
     }
     store_run<TIN, 8>(p.dS + (int64_t)pos * p.ldS + u0 + c * 8, d);
   }
