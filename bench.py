@@ -455,8 +455,8 @@ def run_token_sweep(args):
             torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
         rec = {"T": T}
-        # (streaming passes over [V, H]: up to 128 tokens the backward takes the logits the forward kept instead of a pass over W)
-        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 128 else 4.0, 6.0 * T * V * H)):
+        # (streaming passes over [V, H]: up to 512 tokens the backward takes the logits the forward kept instead of a pass over W)
+        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 512 else 4.0, 6.0 * T * V * H)):
             ms = timed(fn)
             hbm_ms = passes * V * H * 2.0 / PEAK_HBM * 1e3
             mfma_ms = flops / PEAK_BF16 * 1e3
@@ -716,10 +716,10 @@ def main():
     algorithmic = (2.0 * T + 2.0 * n_grads * t_active) * V * H / (elapsed / args.steps)
     if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM and "lce_bwd_chunk_kernel" in kernels:
         # few tokens: HBM bounds the step.  Its streaming passes over [V, H] in the input dtype: W read by the forward and
-        # by the d_hidden product, d_weight written; with up to 128 tokens the forward keeps the fp32 logits (T*V*4 bytes
+        # by the d_hidden product, d_weight written; with up to 512 tokens the forward keeps the fp32 logits (T*V*4 bytes
         # written, then read by the backward) and no pass recomputes them; beyond that the d_logits tiles read W once more.
         k = kernels["lce_bwd_chunk_kernel"]
-        kept = T <= 128
+        kept = T <= 512
         passes_bwd = n_grads if kept else 1.0 + n_grads
         nbytes = passes_bwd * V * H * 2.0 / k["launches_per_step"]  # (W read for d_hidden, d_weight written; --frozen-head: W read)
         step_bytes = (1.0 + passes_bwd) * V * H * 2.0 + (2.0 * T * V * 4.0 if kept else 0.0)

@@ -93,13 +93,14 @@ int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_
                      const float* entropy_b, const float* dlogprobs, const float* dentropy, float* d_hidden, float* d_weight,
                      void* workspace, size_t workspace_bytes, int64_t vchunk, void* stream);
 
-/* Few tokens: the pair above with the logits kept between the two calls, the way autograd keeps any activation.  The
- * reference's backward recomputes the logits from hidden and weight (verl/utils/kernel/kernels.py:1380-1515), which is
- * what keeps [T, V] out of memory when T is large, and what lce_backward does; with at most 128 tokens the backward is
- * bound by its passes over [V, H] (one for the logits, one for d_hidden, one written for d_weight) and [T, V] in fp32 is
- * a fraction of one of them, so keeping it saves the first pass (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not read).
- *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when the library keeps nothing for it (more than 128
- *     tokens, fp32 inputs, diagnostic settings that replace the few-token kernels): then pass NULL below.
+/* The pair above with the logits kept between the two calls, the way autograd keeps any activation, for up to 512
+ * tokens.  The reference's backward recomputes the logits from hidden and weight (verl/utils/kernel/kernels.py:1380-1515),
+ * which is what keeps [T, V] out of memory when T is large, and what lce_backward does.  With few tokens [T, V] in fp32 is
+ * a fraction of the weight itself (512 tokens, H=3584: 29 %; 64 tokens: 4 %), and keeping it saves the backward its
+ * pass over the weight and its T x V x H product for the logits (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not
+ * read).
+ *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when the library keeps nothing for it (more than 512
+ *     tokens, fp32 inputs, diagnostic settings that replace the kernels involved): then pass NULL below.
  *   lce_forward_keep_logits: lce_forward; with logits_cache != NULL it also writes hidden . weight^T there in fp32
  *     (private layout).  Same outputs, bit for bit.
  *   lce_backward_from_logits: lce_backward (grads_fp32 = 0) or lce_backward_f32 (grads_fp32 = 1; d_hidden, d_weight are

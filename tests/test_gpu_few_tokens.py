@@ -145,9 +145,12 @@ def test_full_vocabulary_config2_head():
     (65, 1024, 32000, 0, 2),
     (128, 512, 100003, 8192, 0),
     (128, 128, 300, 0, 0),
+    (129, 256, 20011, 0, 0),     # beyond 128 tokens: the 256-token tiles write the logits, the tile GEMMs read d_logits
+    (300, 512, 50257, 8192, 2),  # two token tiles, seven chunks
+    (512, 384, 30000, 0, 1),
 ])
 def test_backward_from_kept_logits_is_bit_identical(T, H, V, vchunk, reduction, label_mode):
-    """With at most 128 tokens the forward can keep its fp32 logits and the backward then computes d_logits from them
+    """With at most 512 tokens the forward can keep its fp32 logits and the backward then computes d_logits from them
     instead of from a pass over W: same outputs from the forward, same bits in both gradients (16-bit and fp32), with
     tokens without gradient, labels outside the vocabulary, every reduction and every format of the label's entry."""
     from verl_amd import _abi
@@ -182,23 +185,24 @@ def test_backward_from_kept_logits_is_bit_identical(T, H, V, vchunk, reduction, 
         lib.lce_set_option(4, 2)
 
 
-def test_no_logits_are_kept_beyond_128_tokens_or_for_fp32():
+def test_no_logits_are_kept_beyond_512_tokens_or_for_fp32():
     from verl_amd import _abi
     from verl_amd.utils.kernel import kernels
 
     lib = _abi.load()
     assert lib.lce_logits_cache_bytes(128, 512, 1000, _abi.DTYPE_BF16) == 128 * 1024 * 4
-    assert lib.lce_logits_cache_bytes(129, 512, 1000, _abi.DTYPE_BF16) == 0
+    assert lib.lce_logits_cache_bytes(512, 512, 1000, _abi.DTYPE_BF16) == 512 * 1024 * 4
+    assert lib.lce_logits_cache_bytes(513, 512, 1000, _abi.DTYPE_BF16) == 0
     assert lib.lce_logits_cache_bytes(64, 512, 1000, _abi.DTYPE_F32) == 0
-    h, w, y, g_lp, g_ent = _case(129, 256, 3000, torch.bfloat16, seed=1)
+    h, w, y, g_lp, g_ent = _case(513, 256, 3000, torch.bfloat16, seed=1)
     assert kernels.forward_keeping_logits(h, w, y, 0, 1.0)[5] is None
     # a buffer where none is used, and one that is too small, are refused before anything is launched
     buf = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
     f32 = dict(device=DEV, dtype=torch.float32)
-    outs = [torch.empty(129, **f32) for _ in range(5)]
-    ws = torch.empty(lib.lce_forward_workspace_bytes(129, 256, 3000, 0), dtype=torch.uint8, device=DEV)
+    outs = [torch.empty(513, **f32) for _ in range(5)]
+    ws = torch.empty(lib.lce_forward_workspace_bytes(513, 256, 3000, 0), dtype=torch.uint8, device=DEV)
     args = lambda T: (h.data_ptr(), 256, w.data_ptr(), 256, y.data_ptr(), T, 256, 3000, 0, 1.0, 0,
                       *[o.data_ptr() for o in outs], ws.data_ptr(), ws.numel())
-    assert lib.lce_forward_keep_logits(*args(129), buf.data_ptr(), buf.numel(), None) == -1
+    assert lib.lce_forward_keep_logits(*args(513), buf.data_ptr(), buf.numel(), None) == -1
     assert lib.lce_forward_keep_logits(*args(64), buf.data_ptr(), 1000, None) == -2
     torch.cuda.synchronize()

@@ -368,8 +368,9 @@ __global__ __launch_bounds__(256, 2) void lce_bwd_few_kernel(FewArgs<TIN> p) {
 // d_logits of a vocabulary chunk from logits that the forward kept (few tokens): what the d_logits tiles compute from
 // their accumulators, here from x[t * ldx + v], element by element with the same expressions, so the same bits.  One
 // pass over 4 bytes per logit instead of a pass over W.  Workgroup b owns the 64 columns [64 b, 64 b + 64) of dS, i.e.
-// one group of the vocabulary order Perm, and the first `nrows` compact token positions (64 or 128): rows beyond the
-// tokens that take part and columns beyond the chunk's rows are written as zeros, as the tiles write them.  Eight
+// one group of the vocabulary order Perm, and the first `nrows` compact token positions: rows beyond the tokens that
+// take part and columns beyond the chunk's rows (the grid covers whole 256-row tiles) are written as zeros, as the
+// tiles write them.  Eight
 // lanes share a position: they read the 256 bytes of its token's logits of the group and write 128 bytes of dS.
 // p: the chunk's DsArgs (W, h, the tile map and the range are not used); x: the kept logit of the chunk's first row
 // for token 0.
@@ -404,7 +405,7 @@ __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, cons
     for (int hf = 0; hf < 2; ++hf) {
       const int r0 = (int)(Perm::vocab_at(u0 + c * 8 + 4 * hf) - u0);
       f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-      if (tok >= 0) v = *reinterpret_cast<const f32x4_t*>(x + tok * ldx + u0 + r0);
+      if (tok >= 0 && u0 + r0 < p.vrows) v = *reinterpret_cast<const f32x4_t*>(x + tok * ldx + u0 + r0);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         row[4 * hf + e] = r0 + e;

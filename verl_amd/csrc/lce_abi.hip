@@ -199,7 +199,7 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
     else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 1;
   }
-  if (xcache && sel != kSelT64 && sel != kSelT128) return fail(LCE_E_ARG, "forward: tile selector %d cannot keep the logits", sel);
+  if (xcache && sel != kSelT64 && sel != kSelT128 && sel != 0) return fail(LCE_E_ARG, "forward: tile selector %d cannot keep the logits", sel);
   return kForward[dtype](sel, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum,
                          accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits, xcache);
 }

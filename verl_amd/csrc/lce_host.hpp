@@ -229,10 +229,13 @@ int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
   return best;
 }
 
-// Kept logits (few tokens): fp32 [T][logits_cache_row(V)], element [t][v] = hidden[t] . W[v].  A backward that is
-// given them computes d_logits from 4 bytes per logit instead of from a pass over W.
+// Kept logits: fp32 [T][logits_cache_row(V)], element [t][v] = hidden[t] . W[v].  A backward that is given them
+// computes d_logits from 4 bytes per logit instead of from a pass over W and a T x V x H product.  Offered up to 512
+// tokens (16-bit inputs), where the cache stays below a third of a 7B head's weight and every forward of that size runs
+// lce_fwd_kernel, which can write it; beyond that nothing of size T x V is ever kept.
+constexpr int64_t kLogitsCacheMaxTokens = 512;
 int64_t logits_cache_row(int64_t V) { return round_up(V, 64); }
-bool logits_cache_applies(int64_t T, size_t esz) { return esz == 2 && T >= 1 && T <= 128; }
+bool logits_cache_applies(int64_t T, size_t esz) { return esz == 2 && T >= 1 && T <= kLogitsCacheMaxTokens; }
 
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
@@ -272,7 +275,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.split_span = rows_per_split ? rows_per_split : V;
   p.label_offset = label_offset;
   // xcache: the raw logits are kept for the backward (token tiles of at most 128 only; see logits_cache_row)
-  if (xcache && Cfg::BN > 128) return fail(LCE_E_ARG, "forward: this tile variant cannot keep the logits");
+  if (xcache && Cfg::CORE16) return fail(LCE_E_ARG, "forward: this tile variant cannot keep the logits");
   p.xcache = xcache; p.ldx = logits_cache_row(V);
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
@@ -772,17 +775,20 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       }
       continue;
     }
-    if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
-      if (p.n_gw + p.n_gh == 0 && xcache && L.few) {
-        // d_logits from the logits the forward kept: no pass over W
+    if constexpr (sizeof(TIN) == 2 && !Cfg::CORE16 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
+      if (xcache && L.tn && p.n_ds > 0) {
+        // d_logits of this chunk from the logits the forward kept: no pass over W, no T x V x H product
         const int64_t ldx = logits_cache_row(V);
-        const int nrows = (int)(T <= 64 ? 64 : 128) < (int)L.tpad ? (int)(T <= 64 ? 64 : 128) : (int)L.tpad;
+        const int nrows = L.few ? ((int)(T <= 64 ? 64 : 128) < (int)L.tpad ? (int)(T <= 64 ? 64 : 128) : (int)L.tpad) : (int)L.tpad;
         const int64_t c0 = p.ds.v0 - vocab_offset;  // the chunk's first row of W
-        ProfScope prof(PC_BWD_DS, st);
-        hipLaunchKernelGGL((ds_from_logits_kernel<TIN, KPerm<Cfg>>), dim3((unsigned)((p.ds.vrows + 63) / 64)), dim3(256),
-                           0, st, p.ds, xcache + c0, ldx, nrows);
-        if ((rc = check_launch("ds_from_logits_kernel"))) return rc;
-        continue;
+        {
+          ProfScope prof(PC_BWD_DS, st);
+          hipLaunchKernelGGL((ds_from_logits_kernel<TIN, KPerm<Cfg>>), dim3((unsigned)(round_up(p.ds.vrows, 256) / 64)), dim3(256), 0, st, p.ds,
+                             xcache + c0, ldx, nrows);
+          if ((rc = check_launch("ds_from_logits_kernel"))) return rc;
+        }
+        p.n_ds = 0;  // (what is left for the launch below: the gradient GEMMs of the previous chunk)
+        if (p.n_gw + p.n_gh == 0) continue;
       }
     }
     ProfScope prof(PC_BWD_CHUNK, st);

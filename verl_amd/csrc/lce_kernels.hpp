@@ -53,7 +53,7 @@ struct FwdArgs {
   int64_t split_stride, tile_step, split_span;
   TileMap map;       // rows = token tiles, cols = splits
   int64_t label_offset;  // W holds vocabulary rows [label_offset, label_offset + V) of a larger vocabulary (0 = all of it)
-  // Few tokens (token tiles of at most 128): when not null, the raw logits h . W[v] (fp32, before the division by the
+  // Up to kLogitsCacheMaxTokens tokens: when not null, the raw logits h . W[v] (fp32, before the division by the
   // temperature) are kept for the backward, xcache[t * ldx + v] for t < T, v < V (ldx a multiple of 4).
   float* xcache;
   int64_t ldx;
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       g.prologue(lds, p.H);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (Cfg::BN <= 128) {
+    {
       // the logits of this tile, for a backward that then has no need to recompute them: a lane holds four consecutive
       // vocabulary rows of a token in four consecutive registers, 16 bytes of that token's row of the cache; the lanes'
       // pieces of a 128-byte line meet in L2.  Issued behind the next tile's first loads: the stores complete while the K

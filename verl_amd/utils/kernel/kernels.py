@@ -133,10 +133,10 @@ def efficient_entropy_forward(
 
 def forward_keeping_logits(hidden, weight, labels, reduction=2, temperature=1.0, dist_process_group=None, *, keep_logits=True):
     """``efficient_entropy_forward`` plus a sixth value: the kept logits for ``efficient_entropy_backward(...,
-    logits_cache=)``, or ``None`` where the library keeps none (more than 128 tokens, fp32 inputs, ``keep_logits=False``).
-    With few tokens the backward is bound by its passes over ``[V, H]`` and fp32 ``[T, V]`` is a small fraction of one
-    of them, so the autograd node keeps it like any activation and the backward skips the pass that recomputes it (not
-    in the reference, which always recomputes)."""
+    logits_cache=)``, or ``None`` where the library keeps none (more than 512 tokens, fp32 inputs, ``keep_logits=False``).
+    With few tokens fp32 ``[T, V]`` is a fraction of the weight itself, so the autograd node keeps it like any activation
+    and the backward skips the pass over ``[V, H]`` and the ``T x V x H`` product that recompute it (not in the
+    reference, which always recomputes)."""
     _require_single_rank(dist_process_group)
     code = _check_inputs(hidden, weight, labels)
     reduction = get_entropy_reduction_enum(reduction)

@@ -5,8 +5,8 @@ Call-compatible with the reference's ``verl/utils/kernel/linear_cross_entropy.py
 -> (logprobs, entropy)``; outputs are fp32 and flattened to ``[T]`` (``logprobs`` is 0-dim for
 ``"sum"`` / ``"mean"``), ``d_hidden`` comes back in ``hidden``'s shape, ``d_weight`` has ``hidden.dtype``, the four
 non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory, except with at most
-128 tokens, where the node keeps them in fp32 for its backward (a few per cent of the weight's size; it saves the
-backward one of its three passes over ``[V, H]``).
+512 tokens, where the node keeps them in fp32 for its backward (a fraction of the weight's size; it saves the
+backward the pass over ``[V, H]`` and the product that recompute them).
 
 The autograd node is a thin shell: everything it does besides argument checks and reshapes happens in the two host
 launchers of ``kernels.py`` (one C-ABI call each).
@@ -56,7 +56,7 @@ class LinearCrossEntropy(torch.autograd.Function):
             logprobs, entropy, *stats, cache = kernels.forward_keeping_logits(
                 rows, weight, flat_labels, mode, temperature, dist_process_group, keep_logits=keep
             )
-            # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with at most 128 tokens only (else None)
+            # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with at most 512 tokens only (else None)
             ctx.save_for_backward(rows, weight, flat_labels, *stats, cache)
             ctx.call = (hidden.shape, mode, temperature, dist_process_group)
             ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
