@@ -636,6 +636,24 @@ def main():
     prof = _abi.profile_read(reset=True)
     lib.lce_profile_enable(0)
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
+    # Up to 512 tokens the autograd node keeps its fp32 logits for the backward (a bounded exception to "nothing of size
+    # T x V is kept"): how large that is, and the same step with the exception switched off (every backward recomputing
+    # its logits, as at every larger size), timed the same way after everything else.
+    logits_kept = None
+    cache_bytes = 0 if fwd_only else int(lib.lce_logits_cache_bytes(T, H, V, 0))
+    if cache_bytes:
+        K.set_keep_logits_tokens(0)
+        try:
+            for _ in range(max(2, args.warmup)):
+                step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            logits_kept = {"cache_bytes": cache_bytes, "ms_per_step_when_recomputing": (time.perf_counter() - t1) / args.steps * 1e3}
+        finally:
+            K.set_keep_logits_tokens(512)
     # Context only, never the target: the unfused torch path of the reference's own test (materialised fp32 [T, V] logits,
     # softmax, logsumexp, cross_entropy, autograd; tests/utils/test_linear_cross_entropy.py:49-62,290-349 prints the same
     # pair of figures) on the same GPU and inputs, after everything that is timed: one warm-up, then one timed forward + backward.
@@ -654,6 +672,9 @@ def main():
         algo.update({"gemm_nt_kernel(d_hidden)": 2.0 * t_active, "gemm_nt_kernel(d_weight)": 2.0 * t_active})
     executed = {"lce_fwd_kernel": 2.0 * T, "lce_bwd_chunk_kernel": (2.0 + 2.0 * n_grads) * t_active, "gemm_nt_kernel(d_hidden)": 2.0 * t_active,
                 "gemm_nt_kernel(d_weight)": 2.0 * t_active, "lce_bwd_ds_kernel": 2.0 * t_active}
+    if cache_bytes:  # (the d_logits come from the kept logits: an elementwise kernel under the d_logits tiles' name, no recompute)
+        executed["lce_bwd_chunk_kernel"] = 2.0 * n_grads * t_active
+        del executed["lce_bwd_ds_kernel"]
     mfma = {k: v for k, v in kernels.items() if k in algo}
     dom = max(mfma, key=lambda k: mfma[k]["ms_per_step"])
     flops_per_launch = algo[dom] * V * H / mfma[dom]["launches_per_step"]
@@ -719,7 +740,7 @@ def main():
         # by the d_hidden product, d_weight written; with up to 512 tokens the forward keeps the fp32 logits (T*V*4 bytes
         # written, then read by the backward) and no pass recomputes them; beyond that the d_logits tiles read W once more.
         k = kernels["lce_bwd_chunk_kernel"]
-        kept = T <= 512
+        kept = cache_bytes > 0
         passes_bwd = n_grads if kept else 1.0 + n_grads
         nbytes = passes_bwd * V * H * 2.0 / k["launches_per_step"]  # (W read for d_hidden, d_weight written; --frozen-head: W read)
         step_bytes = (1.0 + passes_bwd) * V * H * 2.0 + (2.0 * T * V * 4.0 if kept else 0.0)
@@ -746,6 +767,7 @@ def main():
                    "pass": ("fwd+ppo_loss+bwd" if ppo else "fwd+bwd") + (" (d_hidden only: frozen head)" if args.frozen_head else ""),
                    "tokens_with_gradient": t_active},
         "memory": memory,
+        "logits_kept": logits_kept,
         "algorithmic_tflops": algorithmic / 1e12,
         "frac_of_bf16_peak": algorithmic / PEAK_BF16,
         # tokens without upstream gradient are skipped by the backward: `value` counts them (they are part of the batch),

@@ -221,7 +221,7 @@ int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packe
                         float batch_num_tokens, float global_batch_size, float loss_scale_factor, float* out,
                         float* g_log_prob_packed, float* g_entropy_packed, void* workspace, size_t workspace_bytes, void* stream);
 
-/* One product-level option (process-wide; every entry point works from one snapshot of the settings taken when it starts).
+/* Product-level options (process-wide; every entry point works from one snapshot of the settings taken when it starts).
  * LCE_OPT_WORKSPACE_BUDGET (default 0 = the built-in rule, chunks of 8192 vocabulary columns or wider while one
  * d_logits buffer stays within 256 MiB): a byte count; lce_backward_workspace_bytes with vocab_chunk <= 0 then
  * returns the workspace of the widest chunk that fits it (never below 2048 columns, never above the bound
@@ -232,10 +232,13 @@ int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packe
  * (verl/utils/kernel/kernels.py:1666-1724); 1 = its one-hot part g_logprob / temperature * 1[v == label] is added to
  * d_hidden and to the label rows of d_weight in fp32 instead; 2 = the label's whole entry (one-hot and softmax part,
  * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32.  Changes the workspace size:
- * set it before querying lce_backward_workspace_bytes. */
+ * set it before querying lce_backward_workspace_bytes.
+ * LCE_OPT_KEEP_LOGITS_TOKENS (default 512, the most there is; 0..512): the token count up to which lce_logits_cache_bytes
+ * offers a cache; 0 makes every backward recompute its logits, as the reference does at every size. */
 enum {
   LCE_OPT_LABEL_TERM_OUTSIDE = 4,
-  LCE_OPT_WORKSPACE_BUDGET = 8
+  LCE_OPT_WORKSPACE_BUDGET = 8,
+  LCE_OPT_KEEP_LOGITS_TOKENS = 11
 };
 int lce_set_option(int key, int64_t value);
 

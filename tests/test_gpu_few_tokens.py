@@ -206,3 +206,27 @@ def test_no_logits_are_kept_beyond_512_tokens_or_for_fp32():
     assert lib.lce_forward_keep_logits(*args(513), buf.data_ptr(), buf.numel(), None) == -1
     assert lib.lce_forward_keep_logits(*args(64), buf.data_ptr(), 1000, None) == -2
     torch.cuda.synchronize()
+
+
+def test_keep_logits_option_switches_the_autograd_node_to_recomputing():
+    """LCE_OPT_KEEP_LOGITS_TOKENS = 0: no cache is offered, linear_cross_entropy's backward recomputes its logits, and
+    the gradients are the same bits as with the logits kept."""
+    from verl_amd import _abi, linear_cross_entropy
+    from verl_amd.utils.kernel import kernels
+
+    lib = _abi.load()
+    h, w, y, g_lp, g_ent = _case(96, 512, 30011, torch.bfloat16, seed=5)
+    grads = []
+    try:
+        for tokens in (512, 0, 64):
+            kernels.set_keep_logits_tokens(tokens)
+            assert (lib.lce_logits_cache_bytes(96, 512, 30011, 0) > 0) == (tokens >= 96)
+            hh, ww = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+            lp, ent = linear_cross_entropy(hh, ww, y, 0.9, "none")
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+            grads.append((hh.grad, ww.grad))
+        assert lib.lce_set_option(11, 513) != 0 and lib.lce_set_option(11, -1) != 0
+    finally:
+        kernels.set_keep_logits_tokens(512)
+    for dh, dw in grads[1:]:
+        assert torch.equal(dh, grads[0][0]) and torch.equal(dw, grads[0][1])

@@ -124,6 +124,10 @@ int lce_set_option(int key, int64_t value) {
       if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_WORKSPACE_BUDGET takes a byte count (0 = the built-in default)");
       t.ws_budget = value;
       return LCE_OK;
+    case LCE_OPT_KEEP_LOGITS_TOKENS:
+      if (value < 0 || value > kLogitsCacheMaxTokens) return fail(LCE_E_ARG, "LCE_OPT_KEEP_LOGITS_TOKENS takes 0..%d", (int)kLogitsCacheMaxTokens);
+      t.keep_logits_tokens = value;
+      return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);
   }
 }
@@ -208,7 +212,7 @@ size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
   (void)H;
   if (!known_dtype(dtype) || V <= 0 || !logits_cache_applies(T, esize(dtype))) return 0;
   const Tuning tu = tuning_snapshot();
-  if (tu.variant_forced || !tu.few_token_gemms) return 0;  // (diagnostic settings that take the few-token kernels out)
+  if (tu.variant_forced || T > tu.keep_logits_tokens) return 0;  // (a forced tile variant may be one that cannot write the cache)
   return (size_t)T * (size_t)logits_cache_row(V) * 4;
 }
 

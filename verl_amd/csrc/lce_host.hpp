@@ -45,6 +45,7 @@ struct Tuning {
   int label_outside = 2;         // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
   int dh_ksplit = 0;             // K slices of the d_hidden GEMM; 0: chosen by shape
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
+  int64_t keep_logits_tokens = 512;  // token count up to which lce_logits_cache_bytes offers a cache (0: never)
   int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
 };
 

@@ -87,6 +87,12 @@ def set_workspace_budget(num_bytes: int):
     _abi.check(_abi.load().lce_set_option(8, int(num_bytes)), "lce_set_option")
 
 
+def set_keep_logits_tokens(tokens: int):
+    """Token count up to which ``linear_cross_entropy`` keeps its fp32 logits for the backward (process-wide; default and
+    maximum 512).  0: every backward recomputes them from ``hidden`` and ``weight``, as the reference does at every size."""
+    _abi.check(_abi.load().lce_set_option(11, int(tokens)), "lce_set_option")
+
+
 def _require_single_rank(dist_process_group) -> None:
     """The vocabulary is not sharded here: only ``None`` or a process group of exactly one rank is accepted."""
     if dist_process_group is None:
