@@ -907,15 +907,7 @@ LCE_DEV void dh_finish_body(const float* part, int S, int64_t stride, const int*
     if (pos >= 0) {
       const float* src = part + pos * H + c;
       a = *reinterpret_cast<const float4*>(src);
-      int s = 1;
-      for (; s + 8 <= S; s += 8) {  // eight loads in flight, added in the order of s
-        float4 b[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) b[u] = *reinterpret_cast<const float4*>(src + (s + u) * stride);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
-      }
-      for (; s < S; ++s) {
+      for (int s = 1; s < S; ++s) {
         const float4 b = *reinterpret_cast<const float4*>(src + s * stride);
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
       }
