@@ -230,3 +230,40 @@ def test_keep_logits_option_switches_the_autograd_node_to_recomputing():
         kernels.set_keep_logits_tokens(512)
     for dh, dw in grads[1:]:
         assert torch.equal(dh, grads[0][0]) and torch.equal(dw, grads[0][1])
+
+
+def test_kept_logits_are_bounded_in_aggregate():
+    """A graph that holds several forwards at once (a long batch cut into pieces) keeps logits for at most 512 rows in
+    all: the third piece of 256 tokens keeps none and its backward recomputes, with the same gradients."""
+    import gc
+
+    import importlib
+
+    from verl_amd import linear_cross_entropy
+
+    mod = importlib.import_module("verl_amd.utils.kernel.linear_cross_entropy")  # (the package exports the function under this name)
+    H, V = 256, 5003
+    row = (V + 63) // 64 * 64 * 4
+    gc.collect()
+    base = mod.kept_logits_bytes(DEV)
+    pieces, outs = [], []
+    w = (torch.randn(V, H) * 0.05).bfloat16().to(DEV).requires_grad_(True)
+    for k in range(3):
+        h, _, y, g_lp, g_ent = _case(256, H, V, torch.bfloat16, seed=20 + k)
+        hh = h.clone().requires_grad_(True)
+        lp, ent = linear_cross_entropy(hh, w, y, 1.0, "none")
+        pieces.append((h, hh, y, g_lp, g_ent))
+        outs.append((lp, ent))
+        assert mod.kept_logits_bytes(DEV) - base == min(k + 1, 2) * 256 * row
+    loss = sum((lp * p[3]).sum() + (ent * p[4]).sum() for (lp, ent), p in zip(outs, pieces))
+    loss.backward()
+    del outs, loss, lp, ent
+    gc.collect()
+    assert mod.kept_logits_bytes(DEV) == base
+    dw = torch.zeros_like(w, dtype=torch.float32)
+    for h, hh, y, g_lp, g_ent in pieces:
+        rdh, rdw = O.lce_backward(g_lp, g_ent, h, w.detach(), y, 1.0)
+        _bar(hh.grad, rdh)
+        dw += rdw.float()
+    err = (w.grad.float() - dw).abs()
+    assert (err <= 3 * 2e-2 + 2.0**-6 * dw.abs()).all()  # three 16-bit gradients added by autograd

@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import threading
 import typing
+import weakref
 
 import torch
 
@@ -51,11 +52,15 @@ class LinearCrossEntropy(torch.autograd.Function):
         try:
             mode = kernels.get_entropy_reduction_enum_number(reduction.lower())
             rows, flat_labels = _as_token_rows(hidden, labels)
-            # (no backward will follow, under no_grad or with inputs that take no gradient: nothing is kept beyond the outputs)
+            # (no backward will follow, under no_grad or with inputs that take no gradient: nothing is kept beyond the outputs;
+            # nor when the logits that earlier calls keep, together with this call's, would pass what ONE call may keep)
             keep = getattr(_caller, "grad_enabled", True) and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+            keep = keep and _room_for_logits(rows, weight)
             logprobs, entropy, *stats, cache = kernels.forward_keeping_logits(
                 rows, weight, flat_labels, mode, temperature, dist_process_group, keep_logits=keep
             )
+            if cache is not None:
+                _account(cache)
             # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with at most 512 tokens only (else None)
             ctx.save_for_backward(rows, weight, flat_labels, *stats, cache)
             ctx.call = (hidden.shape, mode, temperature, dist_process_group)
@@ -86,6 +91,40 @@ class LinearCrossEntropy(torch.autograd.Function):
 
 # what torch.is_grad_enabled() said where linear_cross_entropy was called (inside Function.forward it is always off)
 _caller = threading.local()
+
+# Kept logits are bounded per device IN AGGREGATE, not only per call: a caller that cuts a long batch into pieces of a
+# few hundred tokens inside one autograd graph (to bound memory, as the reference's chunked torch backend does) would
+# otherwise end up holding fp32 logits for the whole batch.  Bytes of logits alive per device index:
+_kept_bytes: dict[int, int] = {}
+_kept_lock = threading.Lock()
+KEPT_LOGITS_TOKENS = 512  # the most one call keeps; all live caches of a device together stay within that many rows
+
+
+def kept_logits_bytes(device=None) -> int:
+    """Bytes of kept logits that autograd graphs on ``device`` (default: the current one) hold right now."""
+    index = torch.device("cuda", torch.cuda.current_device()).index if device is None else torch.device(device).index
+    return _kept_bytes.get(index, 0)
+
+
+def _row_bytes(weight: torch.Tensor) -> int:
+    return (weight.shape[0] + 63) // 64 * 64 * 4
+
+
+def _room_for_logits(rows: torch.Tensor, weight: torch.Tensor) -> bool:
+    want = rows.shape[0] * _row_bytes(weight)
+    return _kept_bytes.get(rows.device.index, 0) + want <= KEPT_LOGITS_TOKENS * _row_bytes(weight)
+
+
+def _release(index: int, nbytes: int) -> None:
+    with _kept_lock:
+        _kept_bytes[index] = _kept_bytes.get(index, 0) - nbytes
+
+
+def _account(cache: torch.Tensor) -> None:
+    nbytes = cache.numel() * cache.element_size()
+    with _kept_lock:
+        _kept_bytes[cache.device.index] = _kept_bytes.get(cache.device.index, 0) + nbytes
+    weakref.finalize(cache, _release, cache.device.index, nbytes)  # when the graph that saved it lets go of it
 
 
 def linear_cross_entropy(
