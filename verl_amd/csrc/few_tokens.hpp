@@ -389,10 +389,8 @@ __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, cons
       tok = p.rows ? (int64_t)p.rows[pos] : pos;
       const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
       const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
-      lse2 = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
-      G = glp * p.rcp_tau;
-      C1 = -gent * p.rcp_tau * p.rcp_tau;
-      C0 = -G + gent * p.entropy_b[tok] * p.rcp_tau;
+      const TokenConsts k = token_consts(glp, gent, p.maximum[tok], p.accumulate[tok], p.entropy_b[tok], p.rcp_tau);
+      lse2 = k.lse2; G = k.G; C1 = k.C1; C0 = k.C0;
       const int64_t y = p.labels[tok] - p.v0;
       rel = (p.label_outside != 1 && y >= u0 && y < u0 + 64) ? (int)(y - u0) : -1;
     }

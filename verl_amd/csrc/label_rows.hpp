@@ -76,11 +76,8 @@ LCE_DEV float label_coef_wave(const CoefArgs<T>& a, int64_t t) {
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
-    const float lse2 = (a.maximum[t] + logf(a.accumulate[t])) * kLog2e;
-    const float G = glp * a.rcp_tau;
-    const float C1 = -gent * a.rcp_tau * a.rcp_tau;
-    const float C0 = -G + gent * a.entropy_b[t] * a.rcp_tau;
-    out = fast_exp2(__builtin_fmaf(x, a.c, -lse2)) * __builtin_fmaf(x, C1, C0) + G;
+    const TokenConsts k = token_consts(glp, gent, a.maximum[t], a.accumulate[t], a.entropy_b[t], a.rcp_tau);
+    out = dlogit<true>(x, a.c, k.lse2, k.C0, k.C1, k.G, true, false, false);  // the label's own entry: p (C0 + C1 x) + G
   }
   return out;
 }

@@ -416,6 +416,16 @@ struct VecOf<f16_t, N> { typedef f16_t type __attribute__((ext_vector_type(N)));
 
 // store N consecutive elements (N * sizeof(T) <= 16 bytes per store; wider runs are split);
 // STREAM: non-temporal stores, for data that this kernel does not read back
+// The fp32 value that is rounded to 16 bits is made opaque to the optimiser first: where it is a product, the compiler
+// otherwise fuses the multiplication and the conversion into one v_fma_mixlo_f16 in some kernels and not in others, and
+// the single rounding of the exact product differs from the two roundings (to fp32, then to fp16) at ties (found as one
+// fp16 d_logits entry in 260000 that differed between the tiles and d_logits computed from kept logits).
+template <typename T>
+LCE_DEV T round_to(float x) {
+  if constexpr (sizeof(T) == 2) asm("" : "+v"(x));
+  return (T)x;
+}
+
 template <typename T, int N, bool STREAM = false>
 LCE_DEV void store_run(T* dst, const float (&v)[N]) {
   constexpr int PER = (16 / (int)sizeof(T)) < N ? (16 / (int)sizeof(T)) : N;
@@ -424,16 +434,35 @@ LCE_DEV void store_run(T* dst, const float (&v)[N]) {
   for (int k = 0; k < N; k += PER) {
     vec_t out;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) out[e] = (T)v[k + e];
+    for (int e = 0; e < PER; ++e) out[e] = round_to<T>(v[k + e]);
     if (STREAM) __builtin_nontemporal_store(out, reinterpret_cast<vec_t*>(dst + k));
     else *reinterpret_cast<vec_t*>(dst + k) = out;
   }
+}
+
+// The per-token constants of d_logits: with p = exp2(x c - lse2), dz = p (C0 + C1 x) (+ G at the label).  ONE function
+// with floating-point contraction switched off for every kernel that needs them (the d_logits tiles of both mainloops, the
+// per-position table of the 16x16x32 tiles, the label coefficients, d_logits from kept logits), so that the compiler
+// cannot fuse `a * b + c` in one kernel and not in the next and leave a token with constants that differ in their last bit.
+// glp: upstream gradient of the log-prob, already scaled for the reduction; gent: of the entropy.
+struct TokenConsts {
+  float lse2, C0, C1, G;
+};
+LCE_DEV TokenConsts token_consts(float glp, float gent, float maximum, float accumulate, float entropy_b, float rcp_tau) {
+#pragma clang fp contract(off)
+  TokenConsts k;
+  k.lse2 = (maximum + logf(accumulate)) * kLog2e;
+  k.G = glp * rcp_tau;
+  k.C1 = -gent * rcp_tau * rcp_tau;
+  k.C0 = -k.G + gent * entropy_b * rcp_tau;
+  return k;
 }
 
 // d_logits of one accumulator element; SLOW adds the label one-hot and masks padded rows / tokens
 // (drop: the label's entry is not part of the tile at all, it is added elsewhere in fp32)
 template <bool SLOW>
 LCE_DEV float dlogit(float x, float c, float lse2, float C0, float C1, float G, bool hit, bool dead, bool drop) {
+#pragma clang fp contract(off)
   const float pr = fast_exp2(__builtin_fmaf(x, c, -lse2));
   float dv = pr * __builtin_fmaf(x, C1, C0);
   if (SLOW) {
@@ -477,10 +506,8 @@ LCE_DEV void ds_epilogue(const DsArgs<typename Cfg::TIN>& p, const f32x16_t (&ac
       const int64_t tok = p.rows ? (int64_t)p.rows[pos] : pos;
       const float glp = p.g_lp[tok * p.g_lp_stride] * p.g_lp_scale;
       const float gent = p.g_ent ? p.g_ent[tok] : 0.f;
-      lse2[j] = (p.maximum[tok] + logf(p.accumulate[tok])) * kLog2e;
-      G[j] = glp * p.rcp_tau;
-      C1[j] = -gent * p.rcp_tau * p.rcp_tau;
-      C0[j] = -G[j] + gent * p.entropy_b[tok] * p.rcp_tau;
+      const TokenConsts k = token_consts(glp, gent, p.maximum[tok], p.accumulate[tok], p.entropy_b[tok], p.rcp_tau);
+      lse2[j] = k.lse2; G[j] = k.G; C1[j] = k.C1; C0[j] = k.C0;
       const int64_t y = p.labels[tok] - p.v0;
       rel[j] = (p.label_outside != 1 && y >= vloc0 && y < vloc0 + Cfg::WM) ? (int)(y - vloc0) : -1;
     }

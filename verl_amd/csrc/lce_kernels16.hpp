@@ -172,11 +172,11 @@ inline __global__ void ds_token_consts_kernel(const int* rows, const int* n_rows
     const int64_t tok = rows ? (int64_t)rows[pos] : pos;
     const float glp = g_lp[tok * g_lp_stride] * g_lp_scale;
     const float gent = g_ent ? g_ent[tok] : 0.f;
-    const float G = glp * rcp_tau;
-    c[0] = (maximum[tok] + logf(accumulate[tok])) * kLog2e;
-    c[1] = -G + gent * entropy_b[tok] * rcp_tau;
-    c[2] = -gent * rcp_tau * rcp_tau;
-    c[3] = G;
+    const TokenConsts k = token_consts(glp, gent, maximum[tok], accumulate[tok], entropy_b[tok], rcp_tau);
+    c[0] = k.lse2;
+    c[1] = k.C0;
+    c[2] = k.C1;
+    c[3] = k.G;
     const int64_t y = labels[tok] - vocab_offset;
     lab = (y >= 0 && y < V) ? (int)y : -1;
   }
