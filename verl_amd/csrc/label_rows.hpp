@@ -293,7 +293,7 @@ __global__ __launch_bounds__(256) void dw_label_rows_kernel(const uint32_t* keys
     for (int e = 0; e < N; ++e) acc[e] += (float)cur[e];
     ovec_t out;
 #pragma unroll
-    for (int e = 0; e < N; ++e) out[e] = (TOUT)acc[e];
+    for (int e = 0; e < N; ++e) out[e] = round_to<TOUT>(acc[e]);
     *reinterpret_cast<ovec_t*>(row + c) = out;
   }
 }
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(256) void few_finish_kernel(const float* part, int 
     for (int e = 0; e < N; ++e) acc[e] += (float)cur[e];
     ovec_t out;
 #pragma unroll
-    for (int e = 0; e < N; ++e) out[e] = (TOUT)acc[e];
+    for (int e = 0; e < N; ++e) out[e] = round_to<TOUT>(acc[e]);
     *reinterpret_cast<ovec_t*>(row + c) = out;
   }
 }

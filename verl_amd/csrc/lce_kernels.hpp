@@ -949,7 +949,7 @@ LCE_DEV void dh_finish_body(const float* part, int S, int64_t stride, const int*
       }
     }
     TOUT* dst = out + t * H + c;
-    dst[0] = (TOUT)a.x; dst[1] = (TOUT)a.y; dst[2] = (TOUT)a.z; dst[3] = (TOUT)a.w;
+    dst[0] = round_to<TOUT>(a.x); dst[1] = round_to<TOUT>(a.y); dst[2] = round_to<TOUT>(a.z); dst[3] = round_to<TOUT>(a.w);
   }
 }
 
