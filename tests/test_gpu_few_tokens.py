@@ -267,3 +267,43 @@ def test_kept_logits_are_bounded_in_aggregate():
         dw += rdw.float()
     err = (w.grad.float() - dw).abs()
     assert (err <= 3 * 2e-2 + 2.0**-6 * dw.abs()).all()  # three 16-bit gradients added by autograd
+
+
+def test_few_token_step_replays_from_a_graph():
+    """Forward (keeping its logits) and backward of a 64-token step recorded into a HIP graph: kernels only, no memset
+    nodes.  Every replay, with new values in the same buffers (another set of tokens without gradient each time, so the
+    token list built on the device changes) and eager work in between, must equal the eager calls on those inputs."""
+    from verl_amd.utils.kernel import kernels
+
+    T, H, V, tau = 64, 512, 20011, 0.9
+    h, w, y, g_lp, g_ent = _case(T, H, V, torch.bfloat16, seed=31)
+
+    def step():
+        lp, ent, mx, acc, eb, cache = kernels.forward_keeping_logits(h, w, y, 0, tau)
+        assert cache is not None
+        dh, dw = kernels.efficient_entropy_backward(g_lp, g_ent, h, w, y, mx, acc, eb, 0, False, tau, logits_cache=cache)
+        return lp, ent, dh, dw
+
+    side = torch.cuda.Stream(device=DEV)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = step()
+    for rep in range(3):
+        h.copy_(((torch.rand(T, H) - 0.5) * (rep + 1)).bfloat16())
+        y.copy_(torch.randint(0, V, (T,)))
+        g_lp.copy_(torch.randn(T))
+        g_ent.copy_(torch.randn(T))
+        g_lp[rep::3] = 0.0
+        g_ent[rep::3] = 0.0
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), (rep, (a.float() - b.float()).abs().max().item())

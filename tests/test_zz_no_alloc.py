@@ -110,8 +110,8 @@ def test_static_scratch_forward_allocates_no_device_memory():
 
 
 def test_static_scratch_forward_under_graph_capture_replays_correctly():
-    """After one call outside a capture the entry point can be recorded into a HIP graph (it launches kernels only; what
-    must start at zero is cleared by a fill kernel, not a memset node).  Every replay, with eager work and
+    """After one call outside a capture the entry point can be recorded into a HIP graph (it launches kernels only, no
+    memset node, and nothing in the buffer has to start at zero).  Every replay, with eager work and
     synchronisations of the program in between, must equal the workspace forward on the inputs of that moment."""
     from verl_amd import _abi
 
