@@ -455,8 +455,8 @@ def run_token_sweep(args):
             torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
         rec = {"T": T}
-        # (streaming passes over [V, H]: up to 512 tokens the backward takes the logits the forward kept instead of a pass over W)
-        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 512 else 4.0, 6.0 * T * V * H)):
+        # (streaming passes over [V, H]: up to 1280 tokens the backward takes the logits the forward kept instead of a pass over W)
+        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 1280 else 4.0, 6.0 * T * V * H)):
             ms = timed(fn)
             hbm_ms = passes * V * H * 2.0 / PEAK_HBM * 1e3
             mfma_ms = flops / PEAK_BF16 * 1e3
@@ -636,7 +636,7 @@ def main():
     prof = _abi.profile_read(reset=True)
     lib.lce_profile_enable(0)
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
-    # Up to 512 tokens the autograd node keeps its fp32 logits for the backward (a bounded exception to "nothing of size
+    # With few tokens (up to half the hidden size, at most 1280) the autograd node keeps its fp32 logits for the backward (a bounded exception to "nothing of size
     # T x V is kept"): how large that is, and the same step with the exception switched off (every backward recomputing
     # its logits, as at every larger size), timed the same way after everything else.
     logits_kept = None
@@ -653,7 +653,7 @@ def main():
             torch.cuda.synchronize()
             logits_kept = {"cache_bytes": cache_bytes, "ms_per_step_when_recomputing": (time.perf_counter() - t1) / args.steps * 1e3}
         finally:
-            K.set_keep_logits_tokens(512)
+            K.set_keep_logits_tokens(1280)
     # Context only, never the target: the unfused torch path of the reference's own test (materialised fp32 [T, V] logits,
     # softmax, logsumexp, cross_entropy, autograd; tests/utils/test_linear_cross_entropy.py:49-62,290-349 prints the same
     # pair of figures) on the same GPU and inputs, after everything that is timed: one warm-up, then one timed forward + backward.
@@ -737,7 +737,7 @@ def main():
     algorithmic = (2.0 * T + 2.0 * n_grads * t_active) * V * H / (elapsed / args.steps)
     if 6.0 * T * V * H / (4.0 * V * H * 2.0) < PEAK_BF16 / PEAK_HBM and "lce_bwd_chunk_kernel" in kernels:
         # few tokens: HBM bounds the step.  Its streaming passes over [V, H] in the input dtype: W read by the forward and
-        # by the d_hidden product, d_weight written; with up to 512 tokens the forward keeps the fp32 logits (T*V*4 bytes
+        # by the d_hidden product, d_weight written; with few tokens the forward keeps the fp32 logits (T*V*4 bytes
         # written, then read by the backward) and no pass recomputes them; beyond that the d_logits tiles read W once more.
         k = kernels["lce_bwd_chunk_kernel"]
         kept = cache_bytes > 0

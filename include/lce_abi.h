@@ -93,20 +93,23 @@ int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_
                      const float* entropy_b, const float* dlogprobs, const float* dentropy, float* d_hidden, float* d_weight,
                      void* workspace, size_t workspace_bytes, int64_t vchunk, void* stream);
 
-/* The pair above with the logits kept between the two calls, the way autograd keeps any activation, for up to 512
- * tokens.  The reference's backward recomputes the logits from hidden and weight (verl/utils/kernel/kernels.py:1380-1515),
- * which is what keeps [T, V] out of memory when T is large, and what lce_backward does.  With few tokens [T, V] in fp32 is
- * a fraction of the weight itself (512 tokens, H=3584: 29 %; 64 tokens: 4 %), and keeping it saves the backward its
- * pass over the weight and its T x V x H product for the logits (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not
- * read).
- *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when the library keeps nothing for it (more than 512
- *     tokens, fp32 inputs, diagnostic settings that replace the kernels involved): then pass NULL below.
+/* The pair above with the logits kept between the two calls, the way autograd keeps any activation, while they are no
+ * larger than the weight they came from.  The reference's backward recomputes the logits from hidden and weight
+ * (verl/utils/kernel/kernels.py:1380-1515), which is what keeps [T, V] out of memory when T is large, and what lce_backward
+ * does.  With few tokens [T, V] in fp32 is a fraction of the weight itself (T * V * 4 against V * H * 2 bytes: 4 % at 64
+ * tokens and H=3584, 57 % at 1024), and keeping it saves the backward its pass over the weight and its T x V x H product
+ * for the logits (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not read; 1024 tokens: a quarter of the matrix work).
+ *   lce_logits_cache_max_tokens: the largest T for which a cache is offered: min(H / 2, 1280) for 16-bit inputs (the
+ *     cache never exceeds the weight; 1280 tokens is where the backward changes to kernels that cannot use it), capped by
+ *     LCE_OPT_KEEP_LOGITS_TOKENS; 0 for fp32 inputs and under diagnostic settings that force a tile variant.
+ *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when T is beyond that: then pass NULL below.
  *   lce_forward_keep_logits: lce_forward; with logits_cache != NULL it also writes hidden . weight^T there in fp32
  *     (private layout).  Same outputs, bit for bit.
  *   lce_backward_from_logits: lce_backward (grads_fp32 = 0) or lce_backward_f32 (grads_fp32 = 1; d_hidden, d_weight are
  *     float* then); with logits_cache != NULL, as written by lce_forward_keep_logits for the same hidden, weight, T, H, V
  *     and dtype, the gradient of the logits is computed from it with the same expressions, so both gradients are bit for
  *     bit those of lce_backward.  The cache is only read. */
+int64_t lce_logits_cache_max_tokens(int64_t H, int dtype);
 size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype);
 int lce_forward_keep_logits(const void* hidden, int64_t ldh, const void* weight, int64_t ldw, const int64_t* labels, int64_t T,
                             int64_t H, int64_t V, int dtype, float temperature, int reduction, float* logprobs, float* entropy,
@@ -233,8 +236,9 @@ int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packe
  * d_hidden and to the label rows of d_weight in fp32 instead; 2 = the label's whole entry (one-hot and softmax part,
  * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32.  Changes the workspace size:
  * set it before querying lce_backward_workspace_bytes.
- * LCE_OPT_KEEP_LOGITS_TOKENS (default 512, the most there is; 0..512): the token count up to which lce_logits_cache_bytes
- * offers a cache; 0 makes every backward recompute its logits, as the reference does at every size. */
+ * LCE_OPT_KEEP_LOGITS_TOKENS (default 1280, the most there is; 0..1280): the token count up to which
+ * lce_logits_cache_bytes offers a cache (next to its own bound of H / 2 tokens); 0 makes every backward recompute its
+ * logits, as the reference does at every size. */
 enum {
   LCE_OPT_LABEL_TERM_OUTSIDE = 4,
   LCE_OPT_WORKSPACE_BUDGET = 8,

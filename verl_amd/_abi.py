@@ -30,6 +30,7 @@ SYMBOLS = {
         _i,
         [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i, _f, _i, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _i64, _p],
     ),
+    "lce_logits_cache_max_tokens": (_i64, [_i64, _i]),
     "lce_logits_cache_bytes": (_sz, [_i64, _i64, _i64, _i]),
     "lce_forward_keep_logits": (
         _i,

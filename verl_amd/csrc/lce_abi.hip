@@ -203,16 +203,22 @@ static int forward_entry(const void* hidden, int64_t ldh, const void* weight, in
     // 4.5% faster again once `hidden` is far larger than the memory-side cache (T=65536, H=5120: 671 MB)
     else if (T <= 8192 || (uint64_t)T * (uint64_t)H * esize(dtype) > (512ull << 20)) sel = 1;
   }
-  if (xcache && sel != kSelT64 && sel != kSelT128 && sel != 0) return fail(LCE_E_ARG, "forward: tile selector %d cannot keep the logits", sel);
+  if (xcache && sel != kSelT64 && sel != kSelT128 && sel != 0 && !(sel == kVariantCore16 && esize(dtype) == 2))
+    return fail(LCE_E_ARG, "forward: tile selector %d cannot keep the logits", sel);
   return kForward[dtype](sel, hidden, ldh, weight, ldw, labels, T, H, V, temperature, reduction, logprobs, entropy, maximum,
                          accumulate, entropy_b, ws, st, label_offset, shard_out, max_splits, xcache);
 }
 
-size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
-  (void)H;
-  if (!known_dtype(dtype) || V <= 0 || !logits_cache_applies(T, esize(dtype))) return 0;
+int64_t lce_logits_cache_max_tokens(int64_t H, int dtype) {
+  if (!known_dtype(dtype) || H <= 0) return 0;
   const Tuning tu = tuning_snapshot();
-  if (tu.variant_forced || T > tu.keep_logits_tokens) return 0;  // (a forced tile variant may be one that cannot write the cache)
+  if (tu.variant_forced) return 0;  // (a forced tile variant may be one that cannot write the cache)
+  const int64_t most = logits_cache_max_tokens(H, esize(dtype));
+  return most < tu.keep_logits_tokens ? most : tu.keep_logits_tokens;
+}
+
+size_t lce_logits_cache_bytes(int64_t T, int64_t H, int64_t V, int dtype) {
+  if (V <= 0 || T < 1 || T > lce_logits_cache_max_tokens(H, dtype)) return 0;
   return (size_t)T * (size_t)logits_cache_row(V) * 4;
 }
 

@@ -45,7 +45,7 @@ struct Tuning {
   int label_outside = 2;         // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
   int dh_ksplit = 0;             // K slices of the d_hidden GEMM; 0: chosen by shape
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
-  int64_t keep_logits_tokens = 512;  // token count up to which lce_logits_cache_bytes offers a cache (0: never)
+  int64_t keep_logits_tokens = 1280;  // token count up to which lce_logits_cache_bytes offers a cache (0: never)
   int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
 };
 
@@ -231,12 +231,16 @@ int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
 }
 
 // Kept logits: fp32 [T][logits_cache_row(V)], element [t][v] = hidden[t] . W[v].  A backward that is given them
-// computes d_logits from 4 bytes per logit instead of from a pass over W and a T x V x H product.  Offered up to 512
-// tokens (16-bit inputs), where the cache stays below a third of a 7B head's weight and every forward of that size runs
-// lce_fwd_kernel, which can write it; beyond that nothing of size T x V is ever kept.
-constexpr int64_t kLogitsCacheMaxTokens = 512;
+// computes d_logits from 4 bytes per logit instead of from a pass over W and a T x V x H product.  Offered for 16-bit
+// inputs while the cache is no larger than the weight it came from (T * V * 4 <= V * H * 2, i.e. up to H / 2 tokens) and
+// at most up to 1280 tokens, the size up to which the backward runs the tile kernels that can read d_logits made from
+// it; beyond that nothing of size T x V is ever kept.
+constexpr int64_t kLogitsCacheMaxTokens = kCore16MinTokensBwd;  // 1280
 int64_t logits_cache_row(int64_t V) { return round_up(V, 64); }
-bool logits_cache_applies(int64_t T, size_t esz) { return esz == 2 && T >= 1 && T <= kLogitsCacheMaxTokens; }
+int64_t logits_cache_max_tokens(int64_t H, size_t esz) {
+  if (esz != 2) return 0;
+  return H / 2 < kLogitsCacheMaxTokens ? H / 2 : kLogitsCacheMaxTokens;
+}
 
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
@@ -275,8 +279,7 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   p.tile_step = rows_per_split ? Cfg::BM : (int64_t)S * Cfg::BM;
   p.split_span = rows_per_split ? rows_per_split : V;
   p.label_offset = label_offset;
-  // xcache: the raw logits are kept for the backward (token tiles of at most 128 only; see logits_cache_row)
-  if (xcache && Cfg::CORE16) return fail(LCE_E_ARG, "forward: this tile variant cannot keep the logits");
+  // xcache: the raw logits are kept for the backward
   p.xcache = xcache; p.ldx = logits_cache_row(V);
   p.map = TileMap::make(ntt, S, br, 1);
   float* lp_tok = reduction == LCE_REDUCTION_NONE ? logprobs : reinterpret_cast<float*>(ws + align256((size_t)S * T * 16) + align256((size_t)T * 4));
@@ -284,8 +287,13 @@ int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TI
   {
     ProfScope prof(PC_FWD, st);
     if constexpr (Cfg::CORE16) {
-      allow_lds(lce_fwd16_kernel<Cfg>, Cfg::LDS_BYTES);
-      hipLaunchKernelGGL(lce_fwd16_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+      if (xcache) {
+        allow_lds((lce_fwd16_kernel<Cfg, true>), Cfg::LDS_BYTES);
+        hipLaunchKernelGGL((lce_fwd16_kernel<Cfg, true>), dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+      } else {
+        allow_lds((lce_fwd16_kernel<Cfg, false>), Cfg::LDS_BYTES);
+        hipLaunchKernelGGL((lce_fwd16_kernel<Cfg, false>), dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);
+      }
     } else {
       allow_lds(lce_fwd_kernel<Cfg>, Cfg::LDS_BYTES);
       hipLaunchKernelGGL(lce_fwd_kernel<Cfg>, dim3(p.map.total), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, st, p);

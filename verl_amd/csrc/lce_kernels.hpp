@@ -94,20 +94,14 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
     g.main(lds, p.H, acc);
     const int vbase = (int)m0 + g.wave_m * Cfg::WM;  // vocabulary index of this wave's first row
     const bool full = m0 + Cfg::BM <= vend64;
-    // start fetching the next tile's first slabs now: the loads fly while this tile's statistics are
-    // folded in (the epilogue touches neither LDS nor vector memory on its common path)
-    __syncthreads();  // every wave is past its last LDS read and has drained its own loads
-    if (m0 + p.tile_step < vend64) {
-      g.init(p.W, p.ldw, m0 + p.tile_step, vend64, p.h, p.ldh, n0, p.T);
-      g.prologue(lds, p.H);
-    }
     __builtin_amdgcn_sched_barrier(0);
     {
       // the logits of this tile, for a backward that then has no need to recompute them: a lane holds four consecutive
       // vocabulary rows of a token in four consecutive registers, 16 bytes of that token's row of the cache; the lanes'
-      // pieces of a 128-byte line meet in L2.  Issued behind the next tile's first loads: the stores complete while the K
-      // loop runs, whose counted waits only become a little stricter for them (issued ahead of those loads they
-      // delayed each tile's start by the time a store takes to be acknowledged: 64 tokens, 209 instead of 187 us).
+      // pieces of a 128-byte line meet in L2.  Issued AHEAD of the next tile's first loads: the K loop waits on counts
+      // of outstanding vector-memory operations, which is only safe when every operation that is younger than a load it
+      // waits for is itself a load of the ring (64 tokens: 209 instead of 187 us, the same as with the stores behind
+      // those loads).
       if (p.xcache) {
 #pragma unroll
         for (int j = 0; j < Cfg::FN; ++j) {
@@ -132,6 +126,13 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    // start fetching the next tile's first slabs now: the loads fly while this tile's statistics are
+    // folded in (the epilogue touches neither LDS nor vector memory on its common path)
+    __syncthreads();  // every wave is past its last LDS read and has drained its own loads
+    if (m0 + p.tile_step < vend64) {
+      g.init(p.W, p.ldw, m0 + p.tile_step, vend64, p.h, p.ldh, n0, p.T);
+      g.prologue(lds, p.H);
+    }
     if (!full) {
 #pragma unroll
       for (int i = 0; i < Cfg::FM; ++i)

@@ -83,7 +83,8 @@ LCE_DEV void fwd16_fold(const FwdArgs<typename Cfg::TIN>& p, const f32x4_t (&acc
   }
 }
 
-template <typename Cfg>
+// KEEP: the tiles also write their logits to p.xcache (FwdArgs), for a backward that then does not recompute them
+template <typename Cfg, bool KEEP>
 LCE_DEV void fwd16_body(const FwdArgs<typename Cfg::TIN>& p, char* lds) {
   constexpr int NB = Cfg::NB;
   int tt, s;
@@ -115,6 +116,30 @@ LCE_DEV void fwd16_body(const FwdArgs<typename Cfg::TIN>& p, char* lds) {
     g.main(lds, p.H, acc);
     const int vbase = (int)m0 + g.wave_m * Cfg::WM;  // vocabulary index of this wave's first row
     const bool full = m0 + Cfg::BM <= vend64;
+    if constexpr (KEEP) {
+      // a lane holds four consecutive vocabulary rows of a token per block: one 16-byte store.  Issued AHEAD of the next
+      // tile's first loads: the K loop waits on counts of outstanding vector-memory operations, which is only safe when
+      // every operation that is younger than a load it waits for is itself a load of the ring
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int64_t t = n0 + g.wave_n * Cfg::WN + j * 16 + l16;
+        if (t >= p.T) continue;
+        float* dst = p.xcache + t * p.ldx;
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+          const int v = vbase + 16 * i + 4 * g4;
+          if (v + 3 < vend) {
+            *reinterpret_cast<f32x4_t*>(dst + v) = acc[i][j];
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (v + r < vend) dst[v + r] = acc[i][j][r];
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // the next tile's first slabs fly while this tile's statistics are folded in
     __syncthreads();  // every wave is past its last LDS read and has drained its own loads
     if (m0 + p.tile_step < vend64) {
@@ -448,10 +473,10 @@ LCE_DEV void gemm16_tn_tile(const GemmArgs<typename Cfg::TIN>& pin, int bid, cha
 // ------------------------------------------------------------------------------------------------
 // kernels
 // ------------------------------------------------------------------------------------------------
-template <typename Cfg>
+template <typename Cfg, bool KEEP = false>
 __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd16_kernel(FwdArgs<typename Cfg::TIN> p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  fwd16_body<Cfg>(p, lds);
+  fwd16_body<Cfg, KEEP>(p, lds);
 }
 
 template <typename Cfg>

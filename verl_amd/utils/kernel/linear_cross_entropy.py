@@ -4,9 +4,9 @@ Call-compatible with the reference's ``verl/utils/kernel/linear_cross_entropy.py
 ``linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None)
 -> (logprobs, entropy)``; outputs are fp32 and flattened to ``[T]`` (``logprobs`` is 0-dim for
 ``"sum"`` / ``"mean"``), ``d_hidden`` comes back in ``hidden``'s shape, ``d_weight`` has ``hidden.dtype``, the four
-non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory, except with at most
-512 tokens, where the node keeps them in fp32 for its backward (a fraction of the weight's size; it saves the
-backward the pass over ``[V, H]`` and the product that recompute them).
+non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory, except while they are no
+larger than the weight (at most half the hidden size in tokens, and at most 1280), where the node keeps them in fp32 for
+its backward (it saves the backward the pass over ``[V, H]`` and the product that recompute them).
 
 The autograd node is a thin shell: everything it does besides argument checks and reshapes happens in the two host
 launchers of ``kernels.py`` (one C-ABI call each).
@@ -20,6 +20,7 @@ import weakref
 
 import torch
 
+from ... import _abi
 from . import kernels
 
 
@@ -61,7 +62,7 @@ class LinearCrossEntropy(torch.autograd.Function):
             )
             if cache is not None:
                 _account(cache)
-            # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with at most 512 tokens only (else None)
+            # stats = (maximum, accumulate, entropy_b), fp32 [T]; cache: the logits, with few tokens only (else None)
             ctx.save_for_backward(rows, weight, flat_labels, *stats, cache)
             ctx.call = (hidden.shape, mode, temperature, dist_process_group)
             ctx.set_materialize_grads(False)  # an unused output arrives as None and costs nothing
@@ -97,7 +98,6 @@ _caller = threading.local()
 # otherwise end up holding fp32 logits for the whole batch.  Bytes of logits alive per device index:
 _kept_bytes: dict[int, int] = {}
 _kept_lock = threading.Lock()
-KEPT_LOGITS_TOKENS = 512  # the most one call keeps; all live caches of a device together stay within that many rows
 
 
 def kept_logits_bytes(device=None) -> int:
@@ -111,8 +111,12 @@ def _row_bytes(weight: torch.Tensor) -> int:
 
 
 def _room_for_logits(rows: torch.Tensor, weight: torch.Tensor) -> bool:
+    """All live caches of a device together stay within what ONE call may keep at most for this weight."""
+    if not (rows.is_cuda and weight.dim() == 2 and weight.dtype in (torch.bfloat16, torch.float16)):
+        return False  # (nothing is kept for fp32; anything else is the launcher's to refuse)
+    most = _abi.load().lce_logits_cache_max_tokens(weight.shape[1], _abi.dtype_code(weight.dtype))
     want = rows.shape[0] * _row_bytes(weight)
-    return _kept_bytes.get(rows.device.index, 0) + want <= KEPT_LOGITS_TOKENS * _row_bytes(weight)
+    return _kept_bytes.get(rows.device.index, 0) + want <= most * _row_bytes(weight)
 
 
 def _release(index: int, nbytes: int) -> None:
