@@ -31,11 +31,20 @@ struct Mma16<bf16_t> {
   static LCE_DEV void run(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   }
+  // the same instruction as a builtin: the compiler schedules it and knows its latency
+  static LCE_DEV f32x4_t known(const f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    typedef __bf16 v8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), acc, 0, 0, 0);
+  }
 };
 template <>
 struct Mma16<f16_t> {
   static LCE_DEV void run(f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  static LCE_DEV f32x4_t known(const f32x4_t& acc, const u32x4_t& a, const u32x4_t& b) {
+    typedef _Float16 v8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8, a), __builtin_bit_cast(v8, b), acc, 0, 0, 0);
   }
 };
 
@@ -304,8 +313,17 @@ struct GemmCore16 {
     }
     wait_vm<0>();    // drain the redundant tail fetches before LDS is reused
     wait_lgkm<0>();  // and the reads of the slab after the last
-    // the accumulators are read by ordinary instructions from here on: let the last MFMAs retire
+    // The accumulators are read by ordinary instructions from here on: let the last MFMAs retire.  The MFMAs are inline
+    // assembly, so the compiler knows nothing of their latency, and it is free to place a copy of an accumulator (for the
+    // epilogue, or to spill it) right behind the statement that last wrote it, ahead of this wait (seen in a variant of
+    // the forward: accumulators copied to scratch a few instructions behind the last MFMA, wrong statistics).  Only the
+    // last blocks of the k-step can still be in the matrix pipe when the loop ends, so the last row of blocks is passed
+    // through one more MFMA that the compiler does know (zero operands: acc + 0): behind a builtin it keeps the
+    // distance to a read itself, and the matrix pipe orders it behind the assembly MFMA that wrote the same registers.
     asm volatile("s_nop 15\n\ts_nop 7" ::);
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < NB; ++j) acc[NB - 1][j] = Mma16<TIN>::known(acc[NB - 1][j], zero, zero);
   }
 
   LCE_DEV void run(char* lds, int64_t K, f32x4_t (&acc)[NB][NB]) const {

@@ -99,9 +99,8 @@ __global__ __launch_bounds__(Cfg::NTHREADS) void lce_fwd_kernel(FwdArgs<typename
       // the logits of this tile, for a backward that then has no need to recompute them: a lane holds four consecutive
       // vocabulary rows of a token in four consecutive registers, 16 bytes of that token's row of the cache; the lanes'
       // pieces of a 128-byte line meet in L2.  Issued AHEAD of the next tile's first loads: the K loop waits on counts
-      // of outstanding vector-memory operations, which is only safe when every operation that is younger than a load it
-      // waits for is itself a load of the ring (64 tokens: 209 instead of 187 us, the same as with the stores behind
-      // those loads).
+      // of outstanding vector-memory operations, and with the stores older than every load it waits for, those counts
+      // mean what they say (64 tokens: 209 instead of 187 us, the same as with the stores behind those loads).
       if (p.xcache) {
 #pragma unroll
         for (int j = 0; j < Cfg::FN; ++j) {

@@ -118,24 +118,35 @@ LCE_DEV void fwd16_body(const FwdArgs<typename Cfg::TIN>& p, char* lds) {
     const bool full = m0 + Cfg::BM <= vend64;
     if constexpr (KEEP) {
       // a lane holds four consecutive vocabulary rows of a token per block: one 16-byte store.  Issued AHEAD of the next
-      // tile's first loads: the K loop waits on counts of outstanding vector-memory operations, which is only safe when
-      // every operation that is younger than a load it waits for is itself a load of the ring
+      // tile's first loads: the K loop waits on counts of outstanding vector-memory operations, and with the stores older
+      // than every load it waits for, those counts mean what they say.  The count is a 6-bit field: the stores are
+      // issued 16 at a time and so many are waited for that, with the prologue's 32 loads behind them, fewer than 64
+      // operations are ever in flight.
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int64_t t = n0 + g.wave_n * Cfg::WN + j * 16 + l16;
-        if (t >= p.T) continue;
-        float* dst = p.xcache + t * p.ldx;
+        if (t < p.T) {
+          float* dst = p.xcache + t * p.ldx;
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-          const int v = vbase + 16 * i + 4 * g4;
-          if (v + 3 < vend) {
-            *reinterpret_cast<f32x4_t*>(dst + v) = acc[i][j];
-          } else {
+          for (int i = 0; i < NB; ++i) {
+            const int v = vbase + 16 * i + 4 * g4;
+            if (v + 3 < vend) {
+              *reinterpret_cast<f32x4_t*>(dst + v) = acc[i][j];
+            } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (v + r < vend) dst[v + r] = acc[i][j][r];
+              for (int r = 0; r < 4; ++r)
+                if (v + r < vend) dst[v + r] = acc[i][j][r];
+            }
           }
+        }
+        if (!full) {  // (a tile at the end of its split: up to four single stores per block)
+          __builtin_amdgcn_sched_barrier(0);
+          GemmCore16<Cfg>::template wait_vm<0>();
+        } else if (j % 2 == 1 && j >= 3) {
+          __builtin_amdgcn_sched_barrier(0);
+          if (j == NB - 1) GemmCore16<Cfg>::template wait_vm<24>();
+          else GemmCore16<Cfg>::template wait_vm<32>();
         }
       }
       __builtin_amdgcn_sched_barrier(0);
