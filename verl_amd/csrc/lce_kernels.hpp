@@ -422,7 +422,7 @@ struct VecOf<f16_t, N> { typedef f16_t type __attribute__((ext_vector_type(N)));
 // fp16 d_logits entry in 260000 that differed between the tiles and d_logits computed from kept logits).
 template <typename T>
 LCE_DEV T round_to(float x) {
-  if constexpr (sizeof(T) == 2) asm("" : "+v"(x));
+  if constexpr (__is_same(T, f16_t)) asm("" : "+v"(x));  // (no instruction fuses arithmetic with a conversion to bf16)
   return (T)x;
 }
 
