@@ -408,7 +408,7 @@ SWEEP_WORKLOAD = "token-sweep"
 
 def run_token_sweep(args):
     """Forward and forward + backward of the Qwen2.5-7B head (H=3584, V=152064, bf16) at token counts from 128 to 2048 in
-    steps of 64 plus ragged counts: the band where the launchers switch code paths (at 64, 128, 512 and 1280 tokens) and
+    steps of 64 plus ragged counts: the band where the launchers switch code paths (at 64, 128, 512 and 1280 tokens; beyond half the hidden size the backward recomputes its logits) and
     where the bound changes from HBM (one stream of W per pass: 4 passes of [V, H] forward + backward) to the matrix
     pipes (ridge at 2.5e15 / 8e12 = 312 tokens forward, 417 forward + backward).  Each point: median of `--steps`
     runs; `frac` is the larger of the two floors (algorithmic bytes / 8 TB/s, algorithmic FLOP / 2.5 PFLOP/s) over the
@@ -455,8 +455,8 @@ def run_token_sweep(args):
             torch.autograd.backward([lp, ent], [g_lp, g_ent])
 
         rec = {"T": T}
-        # (streaming passes over [V, H]: up to 1280 tokens the backward takes the logits the forward kept instead of a pass over W)
-        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= 1280 else 4.0, 6.0 * T * V * H)):
+        # (streaming passes over [V, H]: up to half the hidden size in tokens the backward takes the logits the forward kept instead of a pass over W)
+        for name, fn, passes, flops in (("fwd", fwd, 1.0, 2.0 * T * V * H), ("fwd_bwd", fwd_bwd, 3.0 if T <= H // 2 else 4.0, 6.0 * T * V * H)):
             ms = timed(fn)
             hbm_ms = passes * V * H * 2.0 / PEAK_HBM * 1e3
             mfma_ms = flops / PEAK_BF16 * 1e3
@@ -636,7 +636,7 @@ def main():
     prof = _abi.profile_read(reset=True)
     lib.lce_profile_enable(0)
     kernels = {k: {"ms_per_step": ms / nprof, "launches_per_step": n / nprof, "avg_ms": ms / n} for k, (ms, n) in prof.items()}
-    # With few tokens (up to half the hidden size, at most 1280) the autograd node keeps its fp32 logits for the backward (a bounded exception to "nothing of size
+    # With few tokens (up to half the hidden size) the autograd node keeps its fp32 logits for the backward (a bounded exception to "nothing of size
     # T x V is kept"): how large that is, and the same step with the exception switched off (every backward recomputing
     # its logits, as at every larger size), timed the same way after everything else.
     logits_kept = None
@@ -653,7 +653,7 @@ def main():
             torch.cuda.synchronize()
             logits_kept = {"cache_bytes": cache_bytes, "ms_per_step_when_recomputing": (time.perf_counter() - t1) / args.steps * 1e3}
         finally:
-            K.set_keep_logits_tokens(1280)
+            K.set_keep_logits_tokens(None)
     # Context only, never the target: the unfused torch path of the reference's own test (materialised fp32 [T, V] logits,
     # softmax, logsumexp, cross_entropy, autograd; tests/utils/test_linear_cross_entropy.py:49-62,290-349 prints the same
     # pair of figures) on the same GPU and inputs, after everything that is timed: one warm-up, then one timed forward + backward.

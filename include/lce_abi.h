@@ -99,9 +99,8 @@ int lce_backward_f32(const void* hidden, int64_t ldh, const void* weight, int64_
  * does.  With few tokens [T, V] in fp32 is a fraction of the weight itself (T * V * 4 against V * H * 2 bytes: 4 % at 64
  * tokens and H=3584, 57 % at 1024), and keeping it saves the backward its pass over the weight and its T x V x H product
  * for the logits (64 tokens, H=3584, V=152064: 39 MB kept, 1.09 GB not read; 1024 tokens: a quarter of the matrix work).
- *   lce_logits_cache_max_tokens: the largest T for which a cache is offered: min(H / 2, 1280) for 16-bit inputs (the
- *     cache never exceeds the weight; 1280 tokens is where the backward changes to kernels that cannot use it), capped by
- *     LCE_OPT_KEEP_LOGITS_TOKENS; 0 for fp32 inputs and under diagnostic settings that force a tile variant.
+ *   lce_logits_cache_max_tokens: the largest T for which a cache is offered: H / 2 for 16-bit inputs (the
+ *     cache never exceeds the weight), or LCE_OPT_KEEP_LOGITS_TOKENS where that is lower; 0 for fp32 inputs and under diagnostic settings that force a tile variant.
  *   lce_logits_cache_bytes: size of the buffer for this shape, or 0 when T is beyond that: then pass NULL below.
  *   lce_forward_keep_logits: lce_forward; with logits_cache != NULL it also writes hidden . weight^T there in fp32
  *     (private layout).  Same outputs, bit for bit.
@@ -236,9 +235,10 @@ int lce_ppo_loss_packed(const float* log_prob_packed, const float* entropy_packe
  * d_hidden and to the label rows of d_weight in fp32 instead; 2 = the label's whole entry (one-hot and softmax part,
  * with hidden . W[label] recomputed per token) is kept out of the tiles and added in fp32.  Changes the workspace size:
  * set it before querying lce_backward_workspace_bytes.
- * LCE_OPT_KEEP_LOGITS_TOKENS (default 1280, the most there is; 0..1280): the token count up to which
- * lce_logits_cache_bytes offers a cache (next to its own bound of H / 2 tokens); 0 makes every backward recompute its
+ * LCE_OPT_KEEP_LOGITS_TOKENS (default LCE_KEEP_LOGITS_NO_LIMIT; any count >= 0): the token count up to which
+ * lce_logits_cache_bytes offers a cache, next to its own bound of H / 2 tokens; 0 makes every backward recompute its
  * logits, as the reference does at every size. */
+#define LCE_KEEP_LOGITS_NO_LIMIT ((int64_t)1 << 40)
 enum {
   LCE_OPT_LABEL_TERM_OUTSIDE = 4,
   LCE_OPT_WORKSPACE_BUDGET = 8,

@@ -151,9 +151,13 @@ def test_full_vocabulary_config2_head():
     (513, 1152, 9001, 0, 0),     # beyond 512 tokens the 16x16x32 forward tiles write the logits
     (1000, 2048, 20011, 4096, 2),
     (1280, 2560, 5003, 0, 1),
+    (1281, 2688, 5003, 0, 0),    # beyond 1280 tokens the backward's tiles are those of the 16x16x32 loop (groups of 128 vocabulary rows)
+    (1500, 3584, 12007, 4096, 2),
+    (1792, 3584, 9001, 0, 1),
+    (2048, 4096, 3001, 2048, 0),
 ])
 def test_backward_from_kept_logits_is_bit_identical(T, H, V, vchunk, reduction, label_mode):
-    """With few tokens (at most half the hidden size, and at most 1280) the forward can keep its fp32 logits and the backward then computes d_logits from them
+    """With few tokens (at most half the hidden size) the forward can keep its fp32 logits and the backward then computes d_logits from them
     instead of from a pass over W: same outputs from the forward, same bits in both gradients (16-bit and fp32), with
     tokens without gradient, labels outside the vocabulary, every reduction and every format of the label's entry."""
     from verl_amd import _abi
@@ -188,7 +192,24 @@ def test_backward_from_kept_logits_is_bit_identical(T, H, V, vchunk, reduction, 
         lib.lce_set_option(4, 2)
 
 
-def test_no_logits_are_kept_beyond_half_the_hidden_size_or_1280_tokens_or_for_fp32():
+@pytest.mark.parametrize("T,H,V", [(100, 512, 20011), (700, 2048, 9001), (1500, 3072, 12007)])
+def test_backward_from_kept_logits_is_bit_identical_in_fp16(T, H, V):
+    """fp16 has exact ties where bf16 has few (a product of two short mantissas that lands on the middle of two fp16
+    values): both ways to d_logits round once, from the same fp32 value, in every kernel that writes them."""
+    from verl_amd.utils.kernel import kernels
+
+    h, w, y, g_lp, g_ent = _case(T, H, V, torch.float16, seed=3 * T + V)
+    *out, cache = kernels.forward_keeping_logits(h, w, y, 0, 0.5)
+    assert cache is not None
+    mx, acc, eb = out[2:]
+    for fp32 in (True, False):
+        dh0, dw0 = kernels.efficient_entropy_backward(g_lp, g_ent, h, w, y, mx, acc, eb, 0, fp32, 0.5)
+        dh1, dw1 = kernels.efficient_entropy_backward(g_lp, g_ent, h, w, y, mx, acc, eb, 0, fp32, 0.5, logits_cache=cache)
+        assert torch.equal(dh0, dh1) and torch.equal(dw0, dw1)
+    torch.cuda.synchronize()
+
+
+def test_no_logits_are_kept_beyond_half_the_hidden_size_or_for_fp32():
     from verl_amd import _abi
     from verl_amd.utils.kernel import kernels
 
@@ -197,9 +218,9 @@ def test_no_logits_are_kept_beyond_half_the_hidden_size_or_1280_tokens_or_for_fp
     assert lib.lce_logits_cache_bytes(256, 512, 1000, _abi.DTYPE_BF16) == 256 * 1024 * 4   # as large as the weight: the most
     assert lib.lce_logits_cache_bytes(257, 512, 1000, _abi.DTYPE_BF16) == 0
     assert lib.lce_logits_cache_max_tokens(512, _abi.DTYPE_BF16) == 256
-    assert lib.lce_logits_cache_max_tokens(3584, _abi.DTYPE_F16) == 1280
-    assert lib.lce_logits_cache_bytes(1280, 4096, 1000, _abi.DTYPE_BF16) == 1280 * 1024 * 4
-    assert lib.lce_logits_cache_bytes(1281, 4096, 1000, _abi.DTYPE_BF16) == 0
+    assert lib.lce_logits_cache_max_tokens(3584, _abi.DTYPE_F16) == 1792
+    assert lib.lce_logits_cache_bytes(2048, 4096, 1000, _abi.DTYPE_BF16) == 2048 * 1024 * 4
+    assert lib.lce_logits_cache_bytes(2049, 4096, 1000, _abi.DTYPE_BF16) == 0
     assert lib.lce_logits_cache_bytes(64, 512, 1000, _abi.DTYPE_F32) == 0 and lib.lce_logits_cache_max_tokens(512, _abi.DTYPE_F32) == 0
     h, w, y, g_lp, g_ent = _case(513, 256, 3000, torch.bfloat16, seed=1)
     assert kernels.forward_keeping_logits(h, w, y, 0, 1.0)[5] is None
@@ -225,16 +246,16 @@ def test_keep_logits_option_switches_the_autograd_node_to_recomputing():
     h, w, y, g_lp, g_ent = _case(96, 512, 30011, torch.bfloat16, seed=5)
     grads = []
     try:
-        for tokens in (1280, 0, 64):
+        for tokens in (None, 0, 64):
             kernels.set_keep_logits_tokens(tokens)
-            assert (lib.lce_logits_cache_bytes(96, 512, 30011, 0) > 0) == (tokens >= 96)
+            assert (lib.lce_logits_cache_bytes(96, 512, 30011, 0) > 0) == (tokens is None or tokens >= 96)
             hh, ww = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
             lp, ent = linear_cross_entropy(hh, ww, y, 0.9, "none")
             torch.autograd.backward([lp, ent], [g_lp, g_ent])
             grads.append((hh.grad, ww.grad))
-        assert lib.lce_set_option(11, 1281) != 0 and lib.lce_set_option(11, -1) != 0
+        assert lib.lce_set_option(11, -1) != 0
     finally:
-        kernels.set_keep_logits_tokens(1280)
+        kernels.set_keep_logits_tokens(None)
     for dh, dw in grads[1:]:
         assert torch.equal(dh, grads[0][0]) and torch.equal(dw, grads[0][1])
 

@@ -377,9 +377,10 @@ __global__ __launch_bounds__(256, 2) void lce_bwd_few_kernel(FewArgs<TIN> p) {
 // ------------------------------------------------------------------------------------------------------------------
 template <typename TIN, typename Perm>
 __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, const float* x, int64_t ldx, int nrows) {
-  static_assert(sizeof(TIN) == 2 && Perm::GV == 64, "16-bit d_logits in groups of 64 vocabulary rows");
+  static_assert(sizeof(TIN) == 2 && Perm::GV % 64 == 0, "16-bit d_logits, groups of the vocabulary order in multiples of 64 rows");
   const int tid = threadIdx.x, c = tid & 7;
-  const int64_t u0 = (int64_t)blockIdx.x * 64;
+  const int64_t u0 = (int64_t)blockIdx.x * 64;   // first of this workgroup's 64 columns of dS
+  const int64_t g0 = u0 - u0 % Perm::GV;         // first row (= first column) of their group of the vocabulary order
   const int64_t Tc = p.n_rows ? (int64_t)*p.n_rows : p.T;
   for (int pos = tid >> 3; pos < nrows; pos += 32) {
     float lse2 = 0.f, C0 = 0.f, C1 = 0.f, G = 0.f;
@@ -392,18 +393,18 @@ __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, cons
       const TokenConsts k = token_consts(glp, gent, p.maximum[tok], p.accumulate[tok], p.entropy_b[tok], p.rcp_tau);
       lse2 = k.lse2; G = k.G; C1 = k.C1; C0 = k.C0;
       const int64_t y = p.labels[tok] - p.v0;
-      rel = (p.label_outside != 1 && y >= u0 && y < u0 + 64) ? (int)(y - u0) : -1;
+      rel = (p.label_outside != 1 && y >= g0 && y < g0 + Perm::GV) ? (int)(y - g0) : -1;
     }
-    // columns c * 8 + (0..3) and c * 8 + (4..7) of the group are two runs of four consecutive vocabulary rows (the order
-    // Perm keeps what one lane of a d_logits tile holds together: four consecutive rows per register quad), and the
-    // cache's rows are padded to whole groups, so each run is one aligned 16-byte load
+    // columns c * 8 + (0..3) and c * 8 + (4..7) of the workgroup's 64 are two runs of four consecutive vocabulary rows
+    // (both orders Perm keep what one lane of a d_logits tile holds together: four consecutive rows per register quad),
+    // and the cache's rows are padded to whole groups, so each run is one aligned 16-byte load
     float xv[8];
-    int row[8];
+    int row[8];  // vocabulary row relative to the group's first
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
-      const int r0 = (int)(Perm::vocab_at(u0 + c * 8 + 4 * hf) - u0);
+      const int r0 = (int)(Perm::vocab_at(u0 + c * 8 + 4 * hf) - g0);
       f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-      if (tok >= 0 && u0 + r0 < p.vrows) v = *reinterpret_cast<const f32x4_t*>(x + tok * ldx + u0 + r0);
+      if (tok >= 0 && g0 + r0 < p.vrows) v = *reinterpret_cast<const f32x4_t*>(x + tok * ldx + g0 + r0);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         row[4 * hf + e] = r0 + e;
@@ -413,7 +414,7 @@ __global__ __launch_bounds__(256) void ds_from_logits_kernel(DsArgs<TIN> p, cons
     float d[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const bool dead = tok < 0 || u0 + row[e] >= p.vrows;
+      const bool dead = tok < 0 || g0 + row[e] >= p.vrows;
       d[e] = dlogit<true>(dead ? 0.f : xv[e], p.c, lse2, C0, C1, G, row[e] == rel, dead, p.label_outside == 2);
     }
     store_run<TIN, 8>(p.dS + (int64_t)pos * p.ldS + u0 + c * 8, d);

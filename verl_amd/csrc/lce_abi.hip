@@ -125,7 +125,7 @@ int lce_set_option(int key, int64_t value) {
       t.ws_budget = value;
       return LCE_OK;
     case LCE_OPT_KEEP_LOGITS_TOKENS:
-      if (value < 0 || value > kLogitsCacheMaxTokens) return fail(LCE_E_ARG, "LCE_OPT_KEEP_LOGITS_TOKENS takes 0..%d", (int)kLogitsCacheMaxTokens);
+      if (value < 0) return fail(LCE_E_ARG, "LCE_OPT_KEEP_LOGITS_TOKENS takes a token count >= 0 (0: no logits are kept)");
       t.keep_logits_tokens = value;
       return LCE_OK;
     default: return fail(LCE_E_ARG, "unknown option %d", key);

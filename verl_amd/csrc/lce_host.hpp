@@ -45,7 +45,7 @@ struct Tuning {
   int label_outside = 2;         // 16-bit inputs: the label's entry of d_logits added in fp32 outside the d_logits tiles (1: only its one-hot part)
   int dh_ksplit = 0;             // K slices of the d_hidden GEMM; 0: chosen by shape
   int64_t ws_budget = 0;         // byte budget of the backward workspace; 0: the built-in bound
-  int64_t keep_logits_tokens = 1280;  // token count up to which lce_logits_cache_bytes offers a cache (0: never)
+  int64_t keep_logits_tokens = LCE_KEEP_LOGITS_NO_LIMIT;  // a lower limit than half the hidden size for lce_logits_cache_bytes (0: never)
   int few_token_gemms = 1;       // gradient GEMMs of a backward with at most 128 tokens: the streaming kernels of few_tokens.hpp
 };
 
@@ -232,15 +232,10 @@ int forward_splits_256(int ntt, int nvt, int max_splits = kMaxSplits) {
 
 // Kept logits: fp32 [T][logits_cache_row(V)], element [t][v] = hidden[t] . W[v].  A backward that is given them
 // computes d_logits from 4 bytes per logit instead of from a pass over W and a T x V x H product.  Offered for 16-bit
-// inputs while the cache is no larger than the weight it came from (T * V * 4 <= V * H * 2, i.e. up to H / 2 tokens) and
-// at most up to 1280 tokens, the size up to which the backward runs the tile kernels that can read d_logits made from
-// it; beyond that nothing of size T x V is ever kept.
-constexpr int64_t kLogitsCacheMaxTokens = kCore16MinTokensBwd;  // 1280
+// inputs while the cache is no larger than the weight it came from: T * V * 4 <= V * H * 2, i.e. up to H / 2 tokens;
+// beyond that nothing of size T x V is ever kept.
 int64_t logits_cache_row(int64_t V) { return round_up(V, 64); }
-int64_t logits_cache_max_tokens(int64_t H, size_t esz) {
-  if (esz != 2) return 0;
-  return H / 2 < kLogitsCacheMaxTokens ? H / 2 : kLogitsCacheMaxTokens;
-}
+int64_t logits_cache_max_tokens(int64_t H, size_t esz) { return esz == 2 ? H / 2 : 0; }
 
 template <typename Cfg>
 int forward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::TIN* W, int64_t ldw, const int64_t* labels,
@@ -784,7 +779,7 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
       }
       continue;
     }
-    if constexpr (sizeof(TIN) == 2 && !Cfg::CORE16 && Cfg::BM == 256 && Cfg::WAVES_M == 4) {
+    if constexpr (sizeof(TIN) == 2 && Cfg::BM == 256) {
       if (xcache && L.tn && p.n_ds > 0) {
         // d_logits of this chunk from the logits the forward kept: no pass over W, no T x V x H product
         const int64_t ldx = logits_cache_row(V);
@@ -792,7 +787,9 @@ int backward_impl(const typename Cfg::TIN* h, int64_t ldh, const typename Cfg::T
         const int64_t c0 = p.ds.v0 - vocab_offset;  // the chunk's first row of W
         {
           ProfScope prof(PC_BWD_DS, st);
-          hipLaunchKernelGGL((ds_from_logits_kernel<TIN, KPerm<Cfg>>), dim3((unsigned)(round_up(p.ds.vrows, 256) / 64)), dim3(256), 0, st, p.ds,
+          DsArgs<TIN> dq = p.ds;
+          dq.rows = rows;  // (the 16x16x32 tiles read the compact copy of hidden and no list; the cache is indexed by token)
+          hipLaunchKernelGGL((ds_from_logits_kernel<TIN, KPerm<Cfg>>), dim3((unsigned)(round_up(p.ds.vrows, 256) / 64)), dim3(256), 0, st, dq,
                              xcache + c0, ldx, nrows);
           if ((rc = check_launch("ds_from_logits_kernel"))) return rc;
         }

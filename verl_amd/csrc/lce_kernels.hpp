@@ -53,7 +53,7 @@ struct FwdArgs {
   int64_t split_stride, tile_step, split_span;
   TileMap map;       // rows = token tiles, cols = splits
   int64_t label_offset;  // W holds vocabulary rows [label_offset, label_offset + V) of a larger vocabulary (0 = all of it)
-  // Up to kLogitsCacheMaxTokens tokens: when not null, the raw logits h . W[v] (fp32, before the division by the
+  // When not null (offered while the tokens are at most half the hidden size), the raw logits h . W[v] (fp32, before the division by the
   // temperature) are kept for the backward, xcache[t * ldx + v] for t < T, v < V (ldx a multiple of 4).
   float* xcache;
   int64_t ldx;

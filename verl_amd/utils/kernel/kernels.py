@@ -87,11 +87,11 @@ def set_workspace_budget(num_bytes: int):
     _abi.check(_abi.load().lce_set_option(8, int(num_bytes)), "lce_set_option")
 
 
-def set_keep_logits_tokens(tokens: int):
-    """Token count up to which ``linear_cross_entropy`` keeps its fp32 logits for the backward (process-wide; default and
-    maximum 1280; the library's own bound, half the hidden size, applies next to it).  0: every backward recomputes them
-    from ``hidden`` and ``weight``, as the reference does at every size."""
-    _abi.check(_abi.load().lce_set_option(11, int(tokens)), "lce_set_option")
+def set_keep_logits_tokens(tokens: int | None):
+    """Token count up to which ``linear_cross_entropy`` keeps its fp32 logits for the backward (process-wide), next to
+    the library's own bound of half the hidden size.  ``None`` (the default setting): only that bound.  0: every
+    backward recomputes them from ``hidden`` and ``weight``, as the reference does at every size."""
+    _abi.check(_abi.load().lce_set_option(11, (1 << 40) if tokens is None else int(tokens)), "lce_set_option")
 
 
 def _require_single_rank(dist_process_group) -> None:
@@ -140,7 +140,7 @@ def efficient_entropy_forward(
 
 def forward_keeping_logits(hidden, weight, labels, reduction=2, temperature=1.0, dist_process_group=None, *, keep_logits=True):
     """``efficient_entropy_forward`` plus a sixth value: the kept logits for ``efficient_entropy_backward(...,
-    logits_cache=)``, or ``None`` where the library keeps none (more tokens than half the hidden size or than 1280, fp32
+    logits_cache=)``, or ``None`` where the library keeps none (more tokens than half the hidden size, fp32
     inputs, ``keep_logits=False``).
     With few tokens fp32 ``[T, V]`` is a fraction of the weight itself, so the autograd node keeps it like any activation
     and the backward skips the pass over ``[V, H]`` and the ``T x V x H`` product that recompute it (not in the

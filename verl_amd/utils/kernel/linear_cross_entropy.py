@@ -5,7 +5,7 @@ Call-compatible with the reference's ``verl/utils/kernel/linear_cross_entropy.py
 -> (logprobs, entropy)``; outputs are fp32 and flattened to ``[T]`` (``logprobs`` is 0-dim for
 ``"sum"`` / ``"mean"``), ``d_hidden`` comes back in ``hidden``'s shape, ``d_weight`` has ``hidden.dtype``, the four
 non-tensor arguments get ``None`` gradients.  ``[T, V]`` logits are never written to memory, except while they are no
-larger than the weight (at most half the hidden size in tokens, and at most 1280), where the node keeps them in fp32 for
+larger than the weight (at most half the hidden size in tokens), where the node keeps them in fp32 for
 its backward (it saves the backward the pass over ``[V, H]`` and the product that recompute them).
 
 The autograd node is a thin shell: everything it does besides argument checks and reshapes happens in the two host
