@@ -299,6 +299,29 @@ class _PowerSampler:
         self._stop = True
 
 
+def power_context(step, seconds=2.0):
+    """Context only, never the target: mean socket power and shader clock (amdsmi, 50 ms samples of firmware averages)
+    while the same step repeats for `seconds`, after everything that is timed.  Next to the board's power cap it says
+    whether the step runs into the cap, i.e. whether its time is set by the energy it takes rather than by idle pipes."""
+    import torch
+
+    sampler = _PowerSampler()
+    time.sleep(0.2)
+    t0 = time.time()
+    n = 0
+    while time.time() - t0 < seconds:
+        step()
+        torch.cuda.synchronize()
+        n += 1
+    t1 = time.time()
+    sampler.stop()
+    watts, mhz, ns = sampler.window(t0, t1)
+    if sampler.error or watts is None:
+        return {"error": sampler.error or "no power readings"}
+    return {"mean_socket_watts": watts, "cap_watts": getattr(sampler, "cap_watts", None), "mean_shader_mhz": mhz, "samples": ns,
+            "seconds": t1 - t0, "ms_per_step_meanwhile": (t1 - t0) / n * 1e3, "joules_per_step": watts * (t1 - t0) / n}
+
+
 def run_mfma_ceiling(args):
     """What plain bf16 GEMMs of this path's shapes sustain on THIS box: the library's 16x16x32 mainloop (`lce_gemm_nt`,
     fp32 C; `lce_gemm_tn` for the K-major d_weight layout) next to torch.matmul (hipBLASLt, bf16 C), on all-zero operands
@@ -489,6 +512,7 @@ def main():
     ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE", help="diagnostic: lce_set_option(KEY, VALUE)")
     ap.add_argument("--no-unfused-context", action="store_true",
                     help="skip the context figure: the reference test's unfused torch path (fp32 [T, V] logits, autograd) timed on the same GPU")
+    ap.add_argument("--no-power-context", action="store_true", help="skip the two seconds of the same step under the power sampler")
     ap.add_argument("--frozen-head", action="store_true",
                     help="the weight takes no gradient (LoRA that leaves lm_head alone): the backward leaves the d_weight GEMM out")
     ap.add_argument("--print-state", action="store_true", help="print the library state that keys profiles/traffic.json and exit")
@@ -661,6 +685,11 @@ def main():
     if not args.no_unfused_context and not fwd_only and not ppo and not args.frozen_head and T * V <= 16384 * 152064:
         unfused = unfused_context(h, w, y, tau, g_lp, g_ent)
 
+    # socket power against the board's cap while the step repeats (steps long enough for 50 ms samples to mean something)
+    power = None
+    if not args.no_power_context and ms_per_step >= 5.0:
+        power = power_context(step)
+
     # the dominant kernel (largest share of the step) and its algorithmic FLOPs per launch:
     # algorithmic FLOPs per step of each MFMA kernel class (the recompute of the logits in the
     # backward is executed but not counted): forward 2*T*V*H; backward d_hidden + d_weight 4*Ta*V*H,
@@ -701,6 +730,7 @@ def main():
                              "traffic": measured_traffic(workload_name, "lce_fwd_kernel", state),
                              "avg_launch_ms": k["avg_ms"], "flops_per_launch": flops},
                 "kernels": kernels,
+                "socket_power": power,
                 "cpu_baseline": None,
             }
             print(json.dumps(out), flush=True)
@@ -779,6 +809,7 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
         "unfused_torch_same_gpu": unfused,
+        "socket_power": power,
         "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
     }
     print(json.dumps(out), flush=True)
