@@ -1,4 +1,4 @@
-// Gradient GEMMs of a backward with few tokens (at most 128), 16-bit inputs, gfx950.
+// Gradient GEMMs of a backward with few tokens (at most 128), and d_logits from kept logits; 16-bit inputs, gfx950.
 //
 // With T <= 128 both products are one streaming pass over a [V, H] matrix and bound by HBM, not by the matrix cores:
 //   d_weight[v][h] = sum_t dS[t][v] * hidden[t][h]      writes [V, H] once; its operands (dS, hidden) are small
@@ -365,13 +365,14 @@ __global__ __launch_bounds__(256, 2) void lce_bwd_few_kernel(FewArgs<TIN> p) {
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// d_logits of a vocabulary chunk from logits that the forward kept (few tokens): what the d_logits tiles compute from
-// their accumulators, here from x[t * ldx + v], element by element with the same expressions, so the same bits.  One
-// pass over 4 bytes per logit instead of a pass over W.  Workgroup b owns the 64 columns [64 b, 64 b + 64) of dS, i.e.
-// one group of the vocabulary order Perm, and the first `nrows` compact token positions: rows beyond the tokens that
-// take part and columns beyond the chunk's rows (the grid covers whole 256-row tiles) are written as zeros, as the
-// tiles write them.  Eight
-// lanes share a position: they read the 256 bytes of its token's logits of the group and write 128 bytes of dS.
+// d_logits of a vocabulary chunk from logits that the forward kept (tokens up to half the hidden size): what the
+// d_logits tiles compute from their accumulators, here from x[t * ldx + v], element by element with the same
+// expressions, so the same bits.  One pass over 4 bytes per logit instead of a pass over W.  Workgroup b owns the 64
+// columns [64 b, 64 b + 64) of dS, which lie within one group of the vocabulary order Perm (a whole group of the
+// eight-wave tiles' order, half a group of the 16x16x32 tiles'), and the first `nrows` compact token positions: rows
+// beyond the tokens that take part and columns beyond the chunk's rows (the grid covers whole 256-row tiles) are
+// written as zeros, as the tiles write them.  Eight lanes share a position: they read the 256 bytes of its token's
+// logits behind the 64 columns and write 128 bytes of dS.
 // p: the chunk's DsArgs (W, h, the tile map and the range are not used); x: the kept logit of the chunk's first row
 // for token 0.
 // ------------------------------------------------------------------------------------------------------------------
