@@ -8,7 +8,7 @@ import types
 import pytest
 import torch
 
-from verl_amd.models.transformers import dense_common, monkey_patch
+from verl_amd.models.transformers import dense_common, monkey_patch, vlm_common
 
 
 class _Model(torch.nn.Module):
@@ -76,9 +76,68 @@ def test_patch_selection(captured, capsys):
                          ("torch", dense_common.forward_with_torch_backend), ("liger", dense_common.forward_with_torch_backend)):
         monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend=backend)
         assert M.forward is fwd and m._verl_fused_kernels_backend == backend
-    m.config.model_type = "qwen2_vl"
+    # the model types with forwards of their own in the reference (monkey_patch.py:255-274) get the multimodal pair
+    for model_type in ("qwen2_vl", "qwen2_5_vl", "glm4v", "qwen3_vl", "qwen3_vl_moe", "qwen3_5", "qwen3_5_moe"):
+        m.config.model_type = model_type
+        for backend, name in (("triton", "forward_with_hip_backend"), ("liger", "forward_with_torch_backend")):
+            monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend=backend)
+            assert M.forward.__name__ == name and M.forward.__module__ == vlm_common.__name__
+
+
+def test_multimodal_forwards_route_inputs_and_targets(captured):
+    """qwen2_vl / glm4v: the image and video inputs reach ``self.model`` by name and position_ids must be (4, batch, seq)
+    (verl/models/transformers/qwen2_vl.py:402-413,438-456); qwen3_vl / qwen3_5: ``self.model(input_ids, **kwargs)`` with
+    cu_seqlens handed on only when given (qwen3_5.py:620-629).  Targets as in the dense forwards."""
+    seen = {}
+
+    class VLM(_Model):
+        def model(self, input_ids=None, **kw):
+            seen.clear()
+            seen.update(kw)
+            return super().model(input_ids=input_ids)
+
+    m = VLM()
+    ids = torch.tensor([[5, 6, 7, 8]])
+    pos = torch.zeros(4, 1, 4, dtype=torch.long)
+    flat, shaped = vlm_common.make_forwards("qwen2_vl")
+    out = flat(m, input_ids=ids, position_ids=pos, attention_mask=torch.ones_like(ids), pixel_values="px", image_grid_thw="thw",
+               temperature=0.7, use_cache=False)
+    assert seen["pixel_values"] == "px" and seen["image_grid_thw"] == "thw" and seen["position_ids"] is pos and seen["use_cache"] is False
+    assert seen["pixel_values_videos"] is None and "temperature" not in seen and "labels" not in seen
+    assert captured["labels"].tolist() == [[6, 7, 8, 5]] and captured["temperature"] == 0.7 and captured["reduction"] == "none"
+    assert out.log_probs.shape == (4,) and out.entropy.sum() == 4 and out.hidden_states is None
+    with pytest.raises(ValueError, match="shape \\(4, batch_size, seq_length\\)"):
+        flat(m, input_ids=ids, position_ids=pos[1:])
+    with pytest.raises(ValueError):
+        flat(m, input_ids=ids)
+    flat(m, input_ids=ids, position_ids=pos, shift_labels=torch.tensor([[9, 9, 9, 9]]))
+    assert captured["labels"].tolist() == [[9, 9, 9, 9]]
+    m._verl_fused_kernels_backend = "torch"
+    out = shaped(m, input_ids=ids, position_ids=pos, labels=torch.tensor([[1, 2, 3, 4]]))
+    assert out.log_probs.shape == (1, 4) and captured["labels"].tolist() == [2, 3, 4, 1]
+
+    flat, _ = vlm_common.make_forwards("qwen3_5")
+    flat(m, input_ids=ids, attention_mask=None)
+    assert "cu_seqlens" not in seen and "cu_seqlens_cpu" not in seen and "position_ids" not in seen
+    flat(m, input_ids=ids, cu_seqlens="cu", cu_seqlens_cpu="cpu")
+    assert seen["cu_seqlens"] == "cu" and seen["cu_seqlens_cpu"] == "cpu"
+    with pytest.raises(RuntimeError, match="either labels or input_ids"):
+        flat(m)
     with pytest.raises(NotImplementedError):
-        monkey_patch.patch_forward_with_backends(m, use_fused_kernels=True, fused_kernels_backend="hip")
+        vlm_common.make_forwards("llama")
+
+
+def test_sharded_head_weight_is_gathered(captured):
+    """A DTensor lm-head is un-sharded before the kernel, as verl/models/transformers/qwen3_5.py:645-648 does."""
+
+    class Sharded(torch.nn.Parameter):
+        def full_tensor(self):
+            return torch.full((9, 4), 2.0)
+
+    m = _Model()
+    m.lm_head.weight = Sharded(torch.zeros(9, 4))
+    dense_common.forward_with_hip_backend(m, input_ids=torch.tensor([[1, 2]]), return_dict=True)
+    assert captured["weight"].shape == (9, 4) and float(captured["weight"][0, 0]) == 2.0
 
 
 def test_torch_backend_returns_batch_shaped_outputs(captured):
